@@ -1,0 +1,134 @@
+/*
+ * C ABI of libmor_hip.so: MI355X (gfx950) fake quantization of bf16 tensors.
+ *
+ * These entry points are what a binding of the reference's operator layer needs:
+ * each one stands in for one host launcher of the reference file
+ * mor/csrc/cuda/fake_quantize.cu ("FQ").  All pointers are device pointers unless
+ * stated otherwise, tensors are row-major and contiguous, bf16 is passed as raw
+ * 16-bit patterns.  Calls are asynchronous on `stream` (a hipStream_t passed as
+ * void*; NULL = the null stream), allocate nothing, keep no state between calls
+ * and may be issued from several host threads.
+ *
+ * Return value: 0 on success, a negative MOR_ERR_* code otherwise; the message of
+ * the calling thread's last error is available from mor_last_error().
+ */
+#ifndef MOR_HIP_H_
+#define MOR_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOR_OK 0
+#define MOR_ERR_INVALID_ARGUMENT (-1)   /* a TORCH_CHECK of the reference would have failed */
+#define MOR_ERR_WORKSPACE (-2)          /* workspace missing or too small */
+#define MOR_ERR_LAUNCH (-3)             /* hipGetLastError() after a launch */
+
+/* flags */
+#define MOR_FLAG_DEFAULT 0u
+/* Return what the reference's torch emulation returns instead of what its CUDA
+ * kernel returns: nearest-even bf16 store, arithmetic power-of-two scaling (true
+ * zeros), sign-preserving zeros.  The two differ only on exact rounding ties and
+ * on values that quantize to zero in blocks whose amax exceeds the format maximum. */
+#define MOR_FLAG_TORCH_EMULATION 1u
+/* Do not use the gfx950 FP8 convert instructions; cast in integer/float software. */
+#define MOR_FLAG_SOFTWARE_CAST 2u
+
+/* element formats for mor_block_format / mor_quant_dequant */
+#define MOR_FMT_E4M3 0
+#define MOR_FMT_E5M2 1
+#define MOR_FMT_E3M2 2
+#define MOR_FMT_E2M3 3
+
+/* op ids for mor_workspace_bytes */
+#define MOR_OP_FAKE_QUANTIZE 0
+#define MOR_OP_BLOCK_SCALING 1
+#define MOR_OP_CHANNEL_SCALING 2
+#define MOR_OP_E8MX 3
+
+const char* mor_last_error(void);
+
+/* Library version and the offload architecture it was built for. */
+const char* mor_version(void);
+
+/* Bytes of device workspace an op needs for this shape (0 for ops that need none). */
+size_t mor_workspace_bytes(int op, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols);
+
+/*
+ * fake_quantize / fake_quantize_no_alloc: FQ:1839-1907 (launch decoding FQ:1763-1835,
+ * device code FQ:684-852).  mode % 10: 1 MoR, 2 block E4M3, 3 block E5M2, 4/5 current
+ * scaling E4M3/E5M2 with clamp_threshold as the scale, anything else bf16 copy;
+ * mode / 100 > 0 selects the dynamic-range MoR decision; sf_type 1 = fp32 scale,
+ * 2 = power-of-two (E8) scale.  meta has ceil(rows/block_rows) x ceil(cols/block_cols)
+ * int32 entries.  output may alias input.  Any shape is accepted (the reference
+ * requires even cols and launchable block shapes).
+ */
+int mor_fake_quantize(const void* input, void* output, int32_t* meta,
+                      int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
+                      double clamp_threshold, int64_t mode, int64_t sf_type,
+                      uint32_t flags, void* stream);
+
+/*
+ * Block fake quantization to one forced element format, scale fmax/amax per block as in
+ * the block modes of FQ:801-823; MOR_FMT_E2M3 follows the E2M3 branch FQ:758-770
+ * (software saturating cast).  The reference has no public op for a forced E2M3; this
+ * entry exists for the MX E2M3 benchmark configuration and for tests.
+ */
+int mor_block_format(const void* input, void* output,
+                     int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
+                     int fmt, int64_t sf_type, uint32_t flags, void* stream);
+
+/*
+ * fake_quantize_block_scaling(_inplace): FQ:2013-2230; fake_quantize_channel_scaling(_inplace):
+ * FQ:2431-2660 (channel != 0; block_rows == 1 or block_cols == 1).  E4M3 with the scale
+ * rule ss_mode (1 tensor-amax mantissa shared by all blocks, 2 block amax with E8 scale,
+ * 3 block amax with fp32 scale, 4 tensor amax), falling back to a bf16 copy of the input
+ * when the mean relative error exceeds e4m3_threshold.  Scalars meta / global_amax /
+ * global_non_zero / global_error are device pointers to one element each.  output may
+ * alias input (the in-place ops).  rows % block_rows == 0 and cols % block_cols == 0.
+ */
+int mor_block_scaling(const void* input, void* output, int32_t* meta,
+                      float* global_amax, int32_t* global_non_zero, float* global_error,
+                      int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
+                      double e4m3_threshold, int64_t ss_mode, int channel,
+                      void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
+
+/* fake_quantize_e8mx(_inplace): FQ:2232-2397.  quantize_type 1/2/3 = E8M1/2/3;
+ * scaling_strategy 1 = scale by the tensor amax, else no scale.  output may alias input. */
+int mor_e8mx(const void* input, void* output, int64_t rows, int64_t cols,
+             int64_t block_rows, int64_t block_cols, int64_t quantize_type, int64_t scaling_strategy,
+             void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
+
+/* quant_dequant_e4m3/e5m2/e3m2/e2m3: FQ:1909-1964 (fp32 in, fp32 out, n elements). */
+int mor_quant_dequant(const float* input, float* output, int64_t n, int fmt, void* stream);
+
+/* e4m3_with_e8_scale_rne / _rz: FQ:1966-2011 (fp32 in, fp32 out, n elements). */
+int mor_e4m3_with_e8_scale(const float* input, float* output, int64_t n, int rne, void* stream);
+
+/*
+ * Debug view that the public ops never return: per block amax, the fp32 scale fmax/amax
+ * and its biased exponent field (the E8M0 shared exponent of the power-of-two scale,
+ * FQ:251-252).  Arrays have ceil(rows/block_rows) x ceil(cols/block_cols) entries.
+ */
+int mor_block_stats(const void* input, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
+                    float fmax, float* amax, float* scale, int32_t* e8m0, void* stream);
+
+/* Per block {amax, min non-zero |x|, E4M3 error sum, E5M2 error sum} of the MoR decision
+ * (FQ:407-584); error sums are 0 for blocks that did not need them.  4 floats per block. */
+int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
+                  double clamp_threshold, int64_t mode, int64_t sf_type, float* stats, void* stream);
+
+/*
+ * Exhaustive on-device comparison of the gfx950 FP8 convert instructions with the software
+ * cast over all 2^32 fp32 inputs whose magnitude does not exceed the format maximum.
+ * mismatches[0] = E4M3 count, mismatches[1] = E5M2 count (device pointer, 2 x uint64).
+ */
+int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,34 @@
+"""Builds libmor_hip.so in-tree with hipcc for gfx950."""
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SOURCES = [os.path.join(_HERE, "csrc", "mor_kernels.hip")]
+OUT = os.path.join(_HERE, "lib", "libmor_hip.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # keep packed fp32 instructions out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def build_hip(verbose=False):
+    os.makedirs(os.path.dirname(OUT), exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc] + HIPCC_FLAGS + ["-o", OUT] + SOURCES
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # the host pass warns that it does not know the packed-fp32 feature; that is harmless
+    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l and l.strip())
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed:\n{out}")
+    if verbose and out:
+        print(out, flush=True)
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build_hip(verbose=True))

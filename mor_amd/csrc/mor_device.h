@@ -1,0 +1,309 @@
+// Device-side numerics of the fake-quantization path for gfx950 (wave64).
+//
+// Two implementations of every per-element step live here:
+//   *_exact : integer/float software that follows the reference arithmetic step by step
+//             (mor/csrc/cuda/fake_quantize.cu, "FQ") for every fp32 bit pattern;
+//   *_fast  : a few VALU instructions (hardware FP8 converts, ldexp, integer exponent
+//             arithmetic) that give the same bits whenever the block's scale exponent is
+//             in a safe range; kernels pick per block.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mor {
+
+enum : int { FMT_E4M3 = 0, FMT_E5M2 = 1, FMT_E3M2 = 2, FMT_E2M3 = 3 };
+
+__device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
+
+template <int F> struct Fmt;
+template <> struct Fmt<FMT_E4M3> { static constexpr float fmax = 448.0f;   static constexpr int mbits = 3; static constexpr int emin = -6;  static constexpr bool hw = true;  static constexpr float ovf = 464.0f; };
+template <> struct Fmt<FMT_E5M2> { static constexpr float fmax = 57344.0f; static constexpr int mbits = 2; static constexpr int emin = -14; static constexpr bool hw = true;  static constexpr float ovf = 61440.0f; };
+template <> struct Fmt<FMT_E3M2> { static constexpr float fmax = 28.0f;    static constexpr int mbits = 2; static constexpr int emin = -2;  static constexpr bool hw = false; static constexpr float ovf = 0.0f; };
+template <> struct Fmt<FMT_E2M3> { static constexpr float fmax = 7.5f;     static constexpr int mbits = 3; static constexpr int emin = 0;   static constexpr bool hw = false; static constexpr float ovf = 0.0f; };
+
+__host__ __device__ __forceinline__ float fmax_of(int fmt) {
+    return fmt == FMT_E4M3 ? 448.0f : fmt == FMT_E5M2 ? 57344.0f : fmt == FMT_E3M2 ? 28.0f : 7.5f;
+}
+
+// ---------------------------------------------------------------- bf16 <-> fp32
+// FQ:38-44: a bf16 is the upper half of an fp32.
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return u2f(w & 0xFFFF0000u); }
+__device__ __forceinline__ float bf16_one(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+// FQ:46-60: round half up on the magnitude.  Adding 0x8000 to the word does that, the carry
+// running into the exponent exactly as the reference's mantissa/exponent increments do.
+__device__ __forceinline__ uint32_t rhu_bits(float v) { return f2u(v) + 0x8000u; }
+// torch's nearest-even store (NaN kept as a quiet NaN)
+__device__ __forceinline__ uint32_t rne_bits(float v) {
+    uint32_t b = f2u(v);
+    uint32_t r = b + 0x7FFFu + ((b >> 16) & 1u);
+    return (v != v) ? ((b & 0x80000000u) | 0x7FC00000u) : r;
+}
+template <bool EMU> __device__ __forceinline__ uint32_t store_bits(float v) { return EMU ? rne_bits(v) : rhu_bits(v); }
+template <bool EMU> __device__ __forceinline__ uint16_t store_bf16(float v) { return (uint16_t)(store_bits<EMU>(v) >> 16); }
+// two results -> one packed word: bytes 3:2 of each rounded word
+template <bool EMU> __device__ __forceinline__ uint32_t store_pair(float lo, float hi) {
+    return __builtin_amdgcn_perm(store_bits<EMU>(hi), store_bits<EMU>(lo), 0x07060302u);
+}
+
+// ---------------------------------------------------------------- casts
+// Exact nearest-even rounding of |v| onto the grid of format F, saturating at fmax.
+// (a + M) - M with M = 2^(23 - mbits) * 2^max(exponent, emin) rounds a to that quantum in hardware.
+template <int F> __device__ __forceinline__ float round_mag_sat(float a) {
+    a = fminf(a, Fmt<F>::fmax);
+    int e = (int)(f2u(a) >> 23);
+    e = max(e, Fmt<F>::emin + 127);
+    float M = u2f((uint32_t)(e + 23 - Fmt<F>::mbits) << 23);
+    return (a + M) - M;
+}
+
+// Software model of the reference's hardware cast (FQ:223-227, cuda_fp8.hpp with SATFINITE):
+// nearest even, saturate to +-fmax, sign of a zero kept, NaN -> the canonical NaN 0x7fffffff.
+template <int F> __device__ __forceinline__ float cast_hwmodel_exact(float v) {
+    if (v != v) return u2f(0x7FFFFFFFu);
+    return u2f(f2u(round_mag_sat<F>(fabsf(v))) | (f2u(v) & 0x80000000u));
+}
+
+// The reference's software cast (FQ:125-215): nearest even; E3M2/E2M3 saturate, E4M3/E5M2 give
+// NaN 0x7fffffff above their range; a zero result is +0.
+template <int F> __device__ __forceinline__ float cast_sw_exact(float v) {
+    float a = fabsf(v);
+    if constexpr (F == FMT_E4M3) { if (!(a <= 464.0f)) return u2f(0x7FFFFFFFu); }
+    if constexpr (F == FMT_E5M2) { if (!(a < 61440.0f)) return u2f(0x7FFFFFFFu); }
+    if constexpr (F == FMT_E3M2 || F == FMT_E2M3) { if (v != v) return u2f(f2u(Fmt<F>::fmax) | (f2u(v) & 0x80000000u)); }
+    float r = round_mag_sat<F>(a);
+    uint32_t rb = f2u(r);
+    // sign only on a non-zero result
+    return u2f(rb | ((rb + 0x7FFFFFFFu) & f2u(v) & 0x80000000u));
+}
+
+// torch's CPU cast to float8_e4m3fn / float8_e5m2 and back
+template <int F> __device__ __forceinline__ float cast_torch_exact(float v) {
+    uint32_t s = f2u(v) & 0x80000000u;
+    if (v != v) return u2f(0x7FC00000u | s);
+    float a = fabsf(v);
+    bool over = (F == FMT_E4M3) ? (a > 464.0f) : (a >= 61440.0f);
+    if (over) return u2f(((F == FMT_E4M3) ? 0x7FC00000u : 0x7F800000u) | s);
+    return u2f(f2u(round_mag_sat<F>(a)) | s);
+}
+
+// which cast a production path uses (FQ:338-379): hardware for E4M3/E5M2, software for E2M3/E3M2
+template <int F, bool EMU> __device__ __forceinline__ float cast_exact(float v) {
+    if constexpr (EMU) {
+        if constexpr (Fmt<F>::hw) return cast_torch_exact<F>(v);
+        else {
+            float r = cast_sw_exact<F>(v);
+            return (r == 0.0f) ? u2f(f2u(v) & 0x80000000u) : r;
+        }
+    } else {
+        if constexpr (Fmt<F>::hw) return cast_hwmodel_exact<F>(v);
+        else return cast_sw_exact<F>(v);
+    }
+}
+
+// gfx950 converts.  In range (|v| <= fmax) they are nearest-even with the sign of zero kept.
+template <int F> __device__ __forceinline__ uint32_t hw_pack2(float a, float b) {
+    if constexpr (F == FMT_E4M3) return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    else return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+}
+template <int F, int BYTE> __device__ __forceinline__ float hw_unpack(uint32_t p) {
+    if constexpr (F == FMT_E4M3) return __builtin_amdgcn_cvt_f32_fp8((int)p, BYTE);
+    else return __builtin_amdgcn_cvt_f32_bf8((int)p, BYTE);
+}
+
+// ---------------------------------------------------------------- scale-quantize-dequantize-descale
+// FQ:248-306 with E8_RZ: the power of two is taken from the exponent field of the fp32 scale and
+// added to / subtracted from exponent fields, clamping at 0 and keeping the mantissa.
+template <int F, bool EMU> __device__ __forceinline__ float sqdd_e8_exact(float x, int e8) {
+    if constexpr (EMU) {
+        float p = ldexpf(1.0f, e8);
+        return cast_exact<F, true>(x * p) / p;
+    } else {
+        uint32_t xb = f2u(x);
+        int ve = (int)((xb >> 23) & 0xFF) + e8;
+        if (ve < 0) ve = 0;
+        float scaled = u2f((xb & 0x80000000u) | ((uint32_t)ve << 23) | (xb & 0x7FFFFFu));
+        uint32_t db = f2u(cast_exact<F, false>(scaled));
+        int de = (int)((db >> 23) & 0xFF) - e8;
+        if (de < 0) de = 0;
+        return u2f((db & 0x80000000u) | ((uint32_t)de << 23) | (db & 0x7FFFFFu));
+    }
+}
+
+// FQ:310-316.  NVIDIA arithmetic returns 0x7fffffff for a NaN result.
+template <int F, bool EMU> __device__ __forceinline__ float sqdd_fp32_exact(float x, float s) {
+    float r = cast_exact<F, EMU>(x * s) / s;
+    if constexpr (!EMU) { if (r != r) r = u2f(0x7FFFFFFFu); }
+    return r;
+}
+
+// Per-block scale state shared by the fast and exact paths.
+struct Scale {
+    float s;      // fp32 scale (fmax / amax, or the caller's)
+    int e8;       // exponent field of s minus 127
+    bool fast;    // the fast path reproduces the exact one for every finite bf16 element
+};
+
+__device__ __forceinline__ Scale make_scale(float s) {
+    Scale sc;
+    sc.s = s;
+    sc.e8 = (int)((f2u(s) >> 23) & 0xFF) - 127;
+    // |e8| <= 100 keeps every scaled / descaled exponent inside the normal range, so exponent-field
+    // arithmetic, ldexp and IEEE multiply/divide agree (see the fast paths below).
+    sc.fast = (sc.e8 >= -100) && (sc.e8 <= 100);
+    return sc;
+}
+
+// Fast E8 path on a pair (lo, hi) of one packed word, result packed.  For E4M3/E5M2:
+//   |x| * 2^e8 (exact), hardware convert and back, then integer exponent subtraction clamped at 0,
+//   which also yields the reference's 2^(-e8-127) for a zero cast result when e8 < 0.  The sign
+//   comes from the input word (the hardware cast keeps the sign, including on zeros).
+template <int F, bool CLAMP> __device__ __forceinline__ uint32_t e8_pair_fast(uint32_t w, int e8) {
+    const int e8s = e8 << 23;
+    if constexpr (Fmt<F>::hw) {
+        float a = ldexpf(fabsf(bf16_lo(w)), e8);
+        float b = ldexpf(fabsf(bf16_hi(w)), e8);
+        if constexpr (CLAMP) { a = fminf(a, Fmt<F>::fmax); b = fminf(b, Fmt<F>::fmax); }
+        uint32_t p = hw_pack2<F>(a, b);
+        int ma = max((int)f2u(hw_unpack<F, 0>(p)) - e8s, 0);
+        int mb = max((int)f2u(hw_unpack<F, 1>(p)) - e8s, 0);
+        uint32_t mag = __builtin_amdgcn_perm((uint32_t)mb, (uint32_t)ma, 0x07060302u);
+        return mag | (w & 0x80008000u);
+    } else {
+        // software saturating cast: a zero result is +0, so the sign is applied to non-zero results only
+        float a = round_mag_sat<F>(ldexpf(fabsf(bf16_lo(w)), e8));
+        float b = round_mag_sat<F>(ldexpf(fabsf(bf16_hi(w)), e8));
+        uint32_t ra = f2u(a), rb = f2u(b);
+        uint32_t sa = (ra + 0x7FFFFFFFu) & (w << 16) & 0x80000000u;
+        uint32_t sb = (rb + 0x7FFFFFFFu) & w & 0x80000000u;
+        uint32_t ma = (uint32_t)max((int)ra - e8s, 0) | sa;
+        uint32_t mb = (uint32_t)max((int)rb - e8s, 0) | sb;
+        return __builtin_amdgcn_perm(mb, ma, 0x07060302u);
+    }
+}
+
+// Fast fp32-scale path on a pair: multiply, convert, IEEE divide, round-half-up store.
+template <int F, bool CLAMP> __device__ __forceinline__ uint32_t fp32_pair_fast(uint32_t w, float s) {
+    float x0 = bf16_lo(w), x1 = bf16_hi(w);
+    float d0, d1;
+    if constexpr (Fmt<F>::hw) {
+        float v0 = x0 * s, v1 = x1 * s;
+        if constexpr (CLAMP) {   // the reference's hardware cast saturates (user-supplied scales only)
+            v0 = __builtin_amdgcn_fmed3f(v0, -Fmt<F>::fmax, Fmt<F>::fmax);
+            v1 = __builtin_amdgcn_fmed3f(v1, -Fmt<F>::fmax, Fmt<F>::fmax);
+        }
+        uint32_t p = hw_pack2<F>(v0, v1);
+        d0 = hw_unpack<F, 0>(p);
+        d1 = hw_unpack<F, 1>(p);
+    } else {
+        d0 = cast_sw_exact<F>(x0 * s);
+        d1 = cast_sw_exact<F>(x1 * s);
+    }
+    return store_pair<false>(d0 / s, d1 / s);
+}
+
+// One element, exact path, any flavour -> fp32 result before the bf16 store.
+template <int F, bool E8, bool EMU> __device__ __forceinline__ float sqdd_exact(float x, const Scale& sc) {
+    if constexpr (E8) return sqdd_e8_exact<F, EMU>(x, sc.e8);
+    else return sqdd_fp32_exact<F, EMU>(x, sc.s);
+}
+
+// One packed word -> one packed word.
+template <int F, bool E8, bool EMU, bool HWCAST, bool CLAMP = false>
+__device__ __forceinline__ uint32_t fq_pair(uint32_t w, const Scale& sc) {
+    if constexpr (!EMU && HWCAST) {
+        if (sc.fast) {
+            if constexpr (E8) return e8_pair_fast<F, CLAMP>(w, sc.e8);
+            else return fp32_pair_fast<F, CLAMP>(w, sc.s);
+        }
+    }
+    float lo = sqdd_exact<F, E8, EMU>(bf16_lo(w), sc);
+    float hi = sqdd_exact<F, E8, EMU>(bf16_hi(w), sc);
+    return store_pair<EMU>(lo, hi);
+}
+
+// fp32 result (no bf16 store) of one element, used by the error sums
+template <int F, bool E8, bool EMU, bool HWCAST> __device__ __forceinline__ float sqdd_value(float x, const Scale& sc) {
+    if constexpr (!EMU && HWCAST && Fmt<F>::hw) {
+        if (sc.fast) {
+            if constexpr (E8) {
+                const int e8s = sc.e8 << 23;
+                uint32_t p = hw_pack2<F>(ldexpf(fabsf(x), sc.e8), 0.0f);
+                int m = max((int)f2u(hw_unpack<F, 0>(p)) - e8s, 0);
+                return u2f((uint32_t)m | (f2u(x) & 0x80000000u));
+            } else {
+                uint32_t p = hw_pack2<F>(x * sc.s, 0.0f);
+                return hw_unpack<F, 0>(p) / sc.s;
+            }
+        }
+    }
+    return sqdd_exact<F, E8, EMU>(x, sc);
+}
+
+// ---------------------------------------------------------------- wave64 reductions
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+    return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_u(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+constexpr int DPP_XOR1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int DPP_XOR2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int DPP_HALF_MIRROR = 0x141; // lane i <-> 7 - i inside each 8 lanes
+constexpr int DPP_MIRROR = 0x140;      // lane i <-> 15 - i inside each 16 lanes
+
+// all-reduce max over aligned groups of G lanes (G power of two, 1..64); inputs are non-negative
+__device__ __forceinline__ float group_max(float v, int G) {
+    if (G >= 2) v = fmaxf(v, dpp_f<DPP_XOR1>(v));
+    if (G >= 4) v = fmaxf(v, dpp_f<DPP_XOR2>(v));
+    if (G >= 8) v = fmaxf(v, dpp_f<DPP_HALF_MIRROR>(v));
+    if (G >= 16) v = fmaxf(v, dpp_f<DPP_MIRROR>(v));
+    if (G >= 32) v = fmaxf(v, __shfl_xor(v, 16));
+    if (G >= 64) v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+__device__ __forceinline__ uint32_t group_umin(uint32_t v, int G) {
+    if (G >= 2) v = min(v, dpp_u<DPP_XOR1>(v));
+    if (G >= 4) v = min(v, dpp_u<DPP_XOR2>(v));
+    if (G >= 8) v = min(v, dpp_u<DPP_HALF_MIRROR>(v));
+    if (G >= 16) v = min(v, dpp_u<DPP_MIRROR>(v));
+    if (G >= 32) v = min(v, (uint32_t)__shfl_xor((int)v, 16));
+    if (G >= 64) v = min(v, (uint32_t)__shfl_xor((int)v, 32));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f<DPP_XOR1>(v);
+    v += dpp_f<DPP_XOR2>(v);
+    v += dpp_f<DPP_HALF_MIRROR>(v);
+    v += dpp_f<DPP_MIRROR>(v);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+    v += (int)dpp_u<DPP_XOR1>((uint32_t)v);
+    v += (int)dpp_u<DPP_XOR2>((uint32_t)v);
+    v += (int)dpp_u<DPP_HALF_MIRROR>((uint32_t)v);
+    v += (int)dpp_u<DPP_MIRROR>((uint32_t)v);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+// amax / min-nonzero accumulation over one packed word (FQ:431-441).
+// The minimum over non-zero magnitudes is taken on (bits - 1) as unsigned, which sends 0 to the top.
+__device__ __forceinline__ void acc_amax(float& amax, uint32_t w) {
+    amax = fmaxf(fmaxf(amax, fabsf(bf16_lo(w))), fabsf(bf16_hi(w)));
+}
+__device__ __forceinline__ void acc_amin(uint32_t& amin_m1, uint32_t w) {
+    uint32_t a = ((w << 16) & 0x7FFFFFFFu) - 1u;
+    uint32_t b = (w & 0x7FFF0000u) - 1u;
+    amin_m1 = min(min(amin_m1, a), b);
+}
+constexpr uint32_t AMIN_INIT_M1 = 0x7F7F0000u - 1u;   // bf16 max, FQ:409-412
+
+}  // namespace mor

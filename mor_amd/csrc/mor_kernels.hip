@@ -1,0 +1,671 @@
+// HIP kernels and C ABI of the MoR fake-quantization path for MI355X (gfx950, wave64).
+//
+// One pass over HBM wherever a quantization block fits in registers:
+//   k_rowgroup   blocks 1 x 8G elements (G = 1..64 lanes, 16-byte loads; the MX 1x32 case is G = 4):
+//                amax by DPP inside the lane group, quantize from registers, 16-byte stores.
+//   k_wgblock    one 256-thread workgroup per block of up to 16384 elements (128x128 tiles, 1x4096 rows):
+//                the block lives in registers as 16-byte vectors; amax / min-nonzero / MoR error sums by
+//                DPP + LDS; the MoR decision and the quantization reuse the registers.
+//   k_elementwise  current-scaling modes (the scale is an argument): flat 16-byte vectors + scalar tail.
+//   k_generic    any block shape and alignment (odd columns, partial blocks, huge blocks): scalar loads,
+//                exact arithmetic only, the block is re-read from cache for each pass.
+// "FQ" below is the reference file mor/csrc/cuda/fake_quantize.cu.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "mor_device.h"
+#include "../../include/mor_hip.h"
+
+namespace mor {
+
+constexpr int WG = 256;
+constexpr int WAVES = WG / 64;
+
+// MorQuantType, FQ:600-608 (the values written to meta)
+enum : int { Q_UNKNOWN = 0, Q_E4M3 = 1, Q_E5M2 = 2, Q_BF16 = 3, Q_E2M3 = 4, Q_E4M3_SMALL = 11, Q_E5M2_SMALL = 12 };
+
+struct Shape {
+    int64_t rows, cols, brows, bcols, gy, gx;
+};
+
+struct QuantArgs {
+    int qmode;        // 1 MoR, 2 fixed format (fmt), 4 current scaling (fmt, scale = clamp)
+    int fmt;          // forced format for qmode 2 / 4
+    int meta_val;     // value written to meta for qmode 2 / 4; < 0: leave meta alone
+    int dyn_range;    // MoR decision by dynamic range instead of quantization error
+    float clamp;      // clamp_threshold
+};
+
+// ------------------------------------------------------------------------------------------------
+// per-format dispatch of one packed word (block-uniform switch)
+template <bool E8, bool EMU, bool HWCAST, bool CLAMP = false>
+__device__ __forceinline__ uint32_t fq_word(uint32_t w, int fmt, const Scale& sc) {
+    switch (fmt) {
+        case FMT_E4M3: return fq_pair<FMT_E4M3, E8, EMU, HWCAST, CLAMP>(w, sc);
+        case FMT_E5M2: return fq_pair<FMT_E5M2, E8, EMU, HWCAST, CLAMP>(w, sc);
+        case FMT_E3M2: return fq_pair<FMT_E3M2, E8, EMU, HWCAST, CLAMP>(w, sc);
+        default:       return fq_pair<FMT_E2M3, E8, EMU, HWCAST, CLAMP>(w, sc);
+    }
+}
+
+template <int F, bool E8, bool EMU, bool HWCAST, bool CLAMP = false>
+__device__ __forceinline__ uint4 fq_vec(uint4 v, const Scale& sc) {
+    uint4 r;
+    r.x = fq_pair<F, E8, EMU, HWCAST, CLAMP>(v.x, sc);
+    r.y = fq_pair<F, E8, EMU, HWCAST, CLAMP>(v.y, sc);
+    r.z = fq_pair<F, E8, EMU, HWCAST, CLAMP>(v.z, sc);
+    r.w = fq_pair<F, E8, EMU, HWCAST, CLAMP>(v.w, sc);
+    return r;
+}
+
+template <bool E8, bool EMU>
+__device__ __forceinline__ uint16_t fq_one_exact(uint16_t h, int fmt, const Scale& sc) {
+    float x = bf16_one(h);
+    float r;
+    switch (fmt) {
+        case FMT_E4M3: r = sqdd_exact<FMT_E4M3, E8, EMU>(x, sc); break;
+        case FMT_E5M2: r = sqdd_exact<FMT_E5M2, E8, EMU>(x, sc); break;
+        case FMT_E3M2: r = sqdd_exact<FMT_E3M2, E8, EMU>(x, sc); break;
+        default:       r = sqdd_exact<FMT_E2M3, E8, EMU>(x, sc); break;
+    }
+    return store_bf16<EMU>(r);
+}
+
+// FQ:610-682 without the error pass: returns Q_UNKNOWN when the error sums are needed.
+__device__ __forceinline__ int mor_decide_range(float amax, float amin, float clamp, int dyn_range) {
+    float range = 0.0f;
+    if (amax == 0.0f) { amax = clamp; range = 1.0f; }
+    if (range == 0.0f) range = amax / amin;
+    const float e4m3_range = dyn_range ? 28672.0f : 114688.0f;
+    if (range <= 7.5f) return Q_E2M3;
+    if (range <= e4m3_range) return (amax <= clamp) ? Q_E4M3_SMALL : Q_E4M3;
+    if (range <= 939524096.0f) {
+        if (dyn_range) return (amax <= clamp) ? Q_E5M2_SMALL : Q_E5M2;
+        return Q_UNKNOWN;
+    }
+    return Q_BF16;
+}
+__device__ __forceinline__ int mor_decide_error(float amax, float clamp, float e4, float e5) {
+    if (e4 <= e5) return (amax <= clamp) ? Q_E4M3_SMALL : Q_E4M3;
+    return Q_BF16;
+}
+__device__ __forceinline__ int mor_fmt_of(int qt) {
+    switch (qt) {
+        case Q_E2M3: return FMT_E2M3;
+        case Q_E4M3: case Q_E4M3_SMALL: return FMT_E4M3;
+        case Q_E5M2: case Q_E5M2_SMALL: return FMT_E5M2;
+        default: return -1;
+    }
+}
+
+// One element's two error terms, FQ:504-542: |q/x - 1| for E4M3 and E5M2 with scales fmax/amax.
+template <bool E8, bool EMU, bool HWCAST>
+__device__ __forceinline__ void err_terms(float x, const Scale& s4, const Scale& s5, float& e4, float& e5) {
+    if (x != 0.0f) {
+        float q4 = sqdd_value<FMT_E4M3, E8, EMU, HWCAST>(x, s4);
+        float q5 = sqdd_value<FMT_E5M2, E8, EMU, HWCAST>(x, s5);
+        e4 += fabsf(q4 / x - 1.0f);
+        e5 += fabsf(q5 / x - 1.0f);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_elementwise: modes 4 / 5 (FQ:825-842): every element uses the caller's scale; meta is a constant.
+template <bool E8, bool EMU, bool HWCAST>
+__global__ __launch_bounds__(WG) void k_elementwise(const uint16_t* in, uint16_t* out,
+                                                    int32_t* __restrict__ meta, int64_t n, int64_t nvec,
+                                                    int64_t nmeta, int fmt, float scale, int meta_val) {
+    const Scale sc = make_scale(scale);
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    if (meta) for (int64_t i = gtid; i < nmeta; i += stride) meta[i] = meta_val;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    uint4* out4 = reinterpret_cast<uint4*>(out);
+    for (int64_t c = gtid; c < nvec; c += stride) {
+        uint4 v = in4[c];
+        uint4 r;
+        r.x = fq_word<E8, EMU, HWCAST, true>(v.x, fmt, sc);
+        r.y = fq_word<E8, EMU, HWCAST, true>(v.y, fmt, sc);
+        r.z = fq_word<E8, EMU, HWCAST, true>(v.z, fmt, sc);
+        r.w = fq_word<E8, EMU, HWCAST, true>(v.w, fmt, sc);
+        out4[c] = r;
+    }
+    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = fq_one_exact<E8, EMU>(in[i], fmt, sc);
+}
+
+__global__ __launch_bounds__(WG) void k_fill_i32(int32_t* p, int64_t n, int32_t v) {
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) p[i] = v;
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_rowgroup: blocks of 1 x 8G elements; the tensor is a flat array of 16-byte chunks and a block is G
+// consecutive chunks held by G consecutive lanes.  U chunks per thread are in flight per iteration.
+template <int F, bool E8, bool EMU, bool HWCAST, int U>
+__global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out,
+                                                 int32_t* __restrict__ meta, int64_t nchunks, int G, int logG,
+                                                 int meta_val) {
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    for (int64_t c0 = (int64_t)blockIdx.x * WG + threadIdx.x; c0 < nchunks; c0 += stride * U) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int64_t c = c0 + (int64_t)u * stride;
+            if (c < nchunks) v[u] = in[c];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int64_t c = c0 + (int64_t)u * stride;
+            if (c < nchunks) {
+                float amax = 0.0f;
+                acc_amax(amax, v[u].x); acc_amax(amax, v[u].y); acc_amax(amax, v[u].z); acc_amax(amax, v[u].w);
+                amax = group_max(amax, G);
+                uint4 r = v[u];
+                if (amax > 0.0f) {                       // FQ:802, 814: a zero block passes through
+                    const Scale sc = make_scale(Fmt<F>::fmax / amax);
+                    r = fq_vec<F, E8, EMU, HWCAST>(v[u], sc);
+                }
+                out[c] = r;
+                if (meta_val >= 0 && (c & (G - 1)) == 0) meta[c >> logG] = meta_val;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_wgblock: one workgroup per quantization block, the block held in registers (NV 16-byte vectors per lane).
+// Chunk ch = v * 256 + tid of the block sits at block row ch / cpr, chunk column ch % cpr.
+template <bool E8, bool EMU, bool HWCAST, int NV>
+__global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out,
+                                                int32_t* __restrict__ meta, float* __restrict__ stats,
+                                                Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
+    __shared__ float s_f[2][WAVES];
+    __shared__ uint32_t s_u[WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t bid = blockIdx.x;
+    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
+    const int64_t row_stride = sh.cols >> 3;                       // chunks per tensor row
+    const int rows_valid = (int)min(sh.brows, sh.rows - r0);
+    const int cols_valid = (int)min((int64_t)cpr, (sh.cols - c0) >> 3);
+    const int nch = (int)sh.brows * cpr;
+
+    uint4 v[NV];
+    int64_t idx[NV];
+    bool ok[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        int ch = k * WG + tid;
+        int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
+        int cc = ch - r * cpr;
+        ok[k] = (ch < nch) && (r < rows_valid) && (cc < cols_valid);
+        idx[k] = (r0 + r) * row_stride + (c0 >> 3) + cc;
+        if (ok[k]) v[k] = in[idx[k]];
+    }
+
+    // pass 1 (registers): amax and min over non-zero magnitudes, FQ:407-485
+    float amax = 0.0f;
+    uint32_t amin_m1 = AMIN_INIT_M1;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+        if (ok[k]) {
+            acc_amax(amax, v[k].x); acc_amax(amax, v[k].y); acc_amax(amax, v[k].z); acc_amax(amax, v[k].w);
+            if (qa.qmode == 1) { acc_amin(amin_m1, v[k].x); acc_amin(amin_m1, v[k].y); acc_amin(amin_m1, v[k].z); acc_amin(amin_m1, v[k].w); }
+        }
+    amax = group_max(amax, 64);
+    amin_m1 = group_umin(amin_m1, 64);
+    if (lane == 0) { s_f[0][wave] = amax; s_u[wave] = amin_m1; }
+    __syncthreads();
+    amax = fmaxf(fmaxf(s_f[0][0], s_f[0][1]), fmaxf(s_f[0][2], s_f[0][3]));
+    amin_m1 = min(min(s_u[0], s_u[1]), min(s_u[2], s_u[3]));
+    const float amin = u2f(amin_m1 + 1u);
+
+    int fmt = qa.fmt;
+    int meta_val = qa.meta_val;
+    float e4 = 0.0f, e5 = 0.0f;
+    if (qa.qmode == 1) {
+        int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
+        if (qt == Q_UNKNOWN) {
+            // pass 2 (registers): the two error sums, FQ:487-584.  amax > 0 here.
+            const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
+#pragma unroll
+            for (int k = 0; k < NV; ++k)
+                if (ok[k]) {
+                    const uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        err_terms<E8, EMU, HWCAST>(bf16_lo(w[j]), s4, s5, e4, e5);
+                        err_terms<E8, EMU, HWCAST>(bf16_hi(w[j]), s4, s5, e4, e5);
+                    }
+                }
+            e4 = wave_sum(e4);
+            e5 = wave_sum(e5);
+            __syncthreads();                     // s_f[0] was read by every wave above
+            if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+            __syncthreads();
+            e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
+            e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+            qt = mor_decide_error(amax, qa.clamp, e4, e5);
+        }
+        meta_val = qt;
+        fmt = mor_fmt_of(qt);
+    }
+    if (tid == 0) {
+        if (meta && meta_val >= 0) meta[bid] = meta_val;
+        if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+    }
+    if (!out) return;
+
+    // pass 3 (registers): quantize and store, FQ:733-851
+    const bool copy = (fmt < 0) || !(amax > 0.0f);
+    const Scale sc = make_scale(copy ? 1.0f : fmax_of(fmt) / amax);
+    if (copy) {
+        if (out != in) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = v[k];
+        }
+        return;
+    }
+    switch (fmt) {
+        case FMT_E4M3:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = fq_vec<FMT_E4M3, E8, EMU, HWCAST>(v[k], sc);
+            break;
+        case FMT_E5M2:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = fq_vec<FMT_E5M2, E8, EMU, HWCAST>(v[k], sc);
+            break;
+        case FMT_E3M2:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = fq_vec<FMT_E3M2, E8, EMU, HWCAST>(v[k], sc);
+            break;
+        default:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = fq_vec<FMT_E2M3, E8, EMU, HWCAST>(v[k], sc);
+            break;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_generic: any shape.  One workgroup per block, element i of the block at (i / bw, i % bw).
+template <bool EMU>
+__global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* out,
+                                                int32_t* __restrict__ meta, float* __restrict__ stats,
+                                                Shape sh, QuantArgs qa, int e8) {
+    __shared__ float s_f[2][WAVES];
+    __shared__ uint32_t s_u[WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t bid = blockIdx.x;
+    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
+    const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
+    const int64_t nel = bh * bw;
+
+    float amax = 0.0f;
+    uint32_t amin_m1 = AMIN_INIT_M1;
+    for (int64_t i = tid; i < nel; i += WG) {
+        int64_t r = i / bw, c = i - r * bw;
+        uint32_t a = ((uint32_t)in[(r0 + r) * sh.cols + c0 + c] << 16) & 0x7FFFFFFFu;
+        amax = fmaxf(amax, u2f(a));
+        amin_m1 = min(amin_m1, a - 1u);
+    }
+    amax = group_max(amax, 64);
+    amin_m1 = group_umin(amin_m1, 64);
+    if (lane == 0) { s_f[0][wave] = amax; s_u[wave] = amin_m1; }
+    __syncthreads();
+    amax = fmaxf(fmaxf(s_f[0][0], s_f[0][1]), fmaxf(s_f[0][2], s_f[0][3]));
+    amin_m1 = min(min(s_u[0], s_u[1]), min(s_u[2], s_u[3]));
+    const float amin = u2f(amin_m1 + 1u);
+
+    int fmt = qa.fmt;
+    int meta_val = qa.meta_val;
+    float e4 = 0.0f, e5 = 0.0f;
+    if (qa.qmode == 1) {
+        int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
+        if (qt == Q_UNKNOWN) {
+            const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
+            for (int64_t i = tid; i < nel; i += WG) {
+                int64_t r = i / bw, c = i - r * bw;
+                float x = bf16_one(in[(r0 + r) * sh.cols + c0 + c]);
+                if (e8) err_terms<true, EMU, false>(x, s4, s5, e4, e5);
+                else err_terms<false, EMU, false>(x, s4, s5, e4, e5);
+            }
+            e4 = wave_sum(e4);
+            e5 = wave_sum(e5);
+            __syncthreads();
+            if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+            __syncthreads();
+            e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
+            e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+            qt = mor_decide_error(amax, qa.clamp, e4, e5);
+        }
+        meta_val = qt;
+        fmt = mor_fmt_of(qt);
+    }
+    if (tid == 0) {
+        if (meta && meta_val >= 0) meta[bid] = meta_val;
+        if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+    }
+    if (!out) return;
+    const bool copy = (fmt < 0) || !(amax > 0.0f);
+    if (copy && out == in) return;
+    const Scale sc = make_scale(copy ? 1.0f : fmax_of(fmt) / amax);
+    for (int64_t i = tid; i < nel; i += WG) {
+        int64_t r = i / bw, c = i - r * bw;
+        int64_t at = (r0 + r) * sh.cols + c0 + c;
+        uint16_t h = in[at];
+        if (!copy) h = e8 ? fq_one_exact<true, EMU>(h, fmt, sc) : fq_one_exact<false, EMU>(h, fmt, sc);
+        out[at] = h;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Debug view: per block amax, fp32 scale, biased exponent of the scale.
+__global__ __launch_bounds__(WG) void k_block_stats(const uint16_t* __restrict__ in, Shape sh, float fmax,
+                                                    float* __restrict__ amax_o, float* __restrict__ scale_o,
+                                                    int32_t* __restrict__ e8m0_o) {
+    __shared__ float s_f[WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t bid = blockIdx.x;
+    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
+    const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
+    float amax = 0.0f;
+    for (int64_t i = tid; i < bh * bw; i += WG) {
+        int64_t r = i / bw, c = i - r * bw;
+        amax = fmaxf(amax, fabsf(bf16_one(in[(r0 + r) * sh.cols + c0 + c])));
+    }
+    amax = group_max(amax, 64);
+    if (lane == 0) s_f[wave] = amax;
+    __syncthreads();
+    if (tid == 0) {
+        amax = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        float s = amax > 0.0f ? fmax / amax : 1.0f;
+        amax_o[bid] = amax;
+        scale_o[bid] = s;
+        e8m0_o[bid] = (int32_t)((f2u(s) >> 23) & 0xFF);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Exhaustive check of the hardware converts against the software model, in range.
+__global__ __launch_bounds__(WG) void k_selftest_hw_cast(unsigned long long* mism) {
+    unsigned long long bad4 = 0, bad5 = 0;
+    const uint64_t stride = (uint64_t)gridDim.x * WG;
+    for (uint64_t i = (uint64_t)blockIdx.x * WG + threadIdx.x; i < (1ull << 32); i += stride) {
+        float v = u2f((uint32_t)i);
+        float a = fabsf(v);
+        if (a <= 448.0f) {
+            uint32_t hw = f2u(hw_unpack<FMT_E4M3, 0>(hw_pack2<FMT_E4M3>(v, 0.0f)));
+            bad4 += (hw != f2u(cast_hwmodel_exact<FMT_E4M3>(v)));
+        }
+        if (a <= 57344.0f) {
+            uint32_t hw = f2u(hw_unpack<FMT_E5M2, 1>(hw_pack2<FMT_E5M2>(0.0f, v)));
+            bad5 += (hw != f2u(cast_hwmodel_exact<FMT_E5M2>(v)));
+        }
+    }
+    if (bad4) atomicAdd(&mism[0], bad4);
+    if (bad5) atomicAdd(&mism[1], bad5);
+}
+
+// ------------------------------------------------------------------------------------------------
+// fp32 elementwise test ops, FQ:854-875
+__global__ __launch_bounds__(WG) void k_quant_dequant(const float* __restrict__ in, float* __restrict__ out, int64_t n, int fmt) {
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) {
+        float v = in[i], r;
+        switch (fmt) {
+            case FMT_E4M3: r = cast_sw_exact<FMT_E4M3>(v); break;
+            case FMT_E5M2: r = cast_sw_exact<FMT_E5M2>(v); break;
+            case FMT_E3M2: r = cast_sw_exact<FMT_E3M2>(v); break;
+            default:       r = cast_sw_exact<FMT_E2M3>(v); break;
+        }
+        out[i] = r;
+    }
+}
+
+// FQ:865-875 + FQ:259-281: per-element power-of-two scale of 448 / value, software E4M3 cast.
+__global__ __launch_bounds__(WG) void k_e4m3_e8_scale(const float* __restrict__ in, float* __restrict__ out, int64_t n, int rne) {
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) {
+        float v = in[i];
+        float sf = 448.0f / v;
+        uint32_t sb = f2u(sf), vb = f2u(v);
+        int e8 = (int)((sb >> 23) & 0xFF) - 127;
+        int ve = (int)((vb >> 23) & 0xFF);
+        uint32_t vman = vb & 0x7FFFFFu;
+        if (rne) {
+            uint32_t sman = sb & 0x7FFFFFu;
+            uint32_t guard = (sman >> 22) & 1u;
+            uint32_t sticky = (sman & ((1u << 22) - 1u)) != 0;
+            if (guard == 1 && vman <= 6815744u && ve + e8 < 135) {
+                if (sticky == 1 || (e8 & 1)) e8++;
+            }
+        }
+        ve += e8;
+        if (ve < 0) ve = 0;
+        float scaled = u2f((vb & 0x80000000u) | ((uint32_t)ve << 23) | vman);
+        uint32_t db = f2u(cast_sw_exact<FMT_E4M3>(scaled));
+        int de = (int)((db >> 23) & 0xFF) - e8;
+        if (de < 0) de = 0;
+        out[i] = u2f((db & 0x80000000u) | ((uint32_t)de << 23) | (db & 0x7FFFFFu));
+    }
+}
+
+}  // namespace mor
+
+// ================================================================================================
+// host side
+using namespace mor;
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(MOR_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return MOR_OK;
+}
+
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
+static inline int ilog2(int64_t x) { int l = 0; while ((1ll << l) < x) ++l; return l; }
+
+static int grid_for(int64_t work_items, int per_cu = 8) {
+    // enough workgroups to fill 256 CUs several times over, capped so grid-stride loops stay short
+    int64_t want = cdiv(work_items, WG);
+    int64_t cap = 256ll * per_cu;
+    if (want < 1) want = 1;
+    return (int)(want < cap ? want : cap);
+}
+
+extern "C" const char* mor_last_error(void) { return g_err; }
+extern "C" const char* mor_version(void) { return "mor_hip 0.1 (gfx950)"; }
+
+static int validate_shape(const void* input, int64_t rows, int64_t cols, int64_t brows, int64_t bcols) {
+    if (!input) return fail(MOR_ERR_INVALID_ARGUMENT, "input is NULL");
+    if (rows <= 0 || cols <= 0) return fail(MOR_ERR_INVALID_ARGUMENT, "rows and cols must be positive (got %lld x %lld)", (long long)rows, (long long)cols);
+    if (brows <= 0 || bcols <= 0) return fail(MOR_ERR_INVALID_ARGUMENT, "block dims must be positive (got %lld x %lld)", (long long)brows, (long long)bcols);
+    if (cdiv(rows, brows) * cdiv(cols, bcols) > 0x7FFFFFFFll) return fail(MOR_ERR_INVALID_ARGUMENT, "too many blocks");
+    return MOR_OK;
+}
+
+template <bool E8, bool EMU, bool HWCAST>
+static void launch_rowgroup(int fmt, const void* in, void* out, int32_t* meta, int64_t nchunks, int G, int meta_val, hipStream_t st) {
+    constexpr int U = 4;
+    int grid = grid_for(cdiv(nchunks, U), 16);
+    const uint4* i4 = static_cast<const uint4*>(in);
+    uint4* o4 = static_cast<uint4*>(out);
+    int lg = ilog2(G);
+    switch (fmt) {
+        case FMT_E4M3: k_rowgroup<FMT_E4M3, E8, EMU, HWCAST, U><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); break;
+        case FMT_E5M2: k_rowgroup<FMT_E5M2, E8, EMU, HWCAST, U><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); break;
+        case FMT_E3M2: k_rowgroup<FMT_E3M2, E8, EMU, HWCAST, U><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); break;
+        default:       k_rowgroup<FMT_E2M3, E8, EMU, HWCAST, U><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); break;
+    }
+}
+
+template <bool E8, bool EMU, bool HWCAST>
+static void launch_wgblock(const void* in, void* out, int32_t* meta, float* stats, const Shape& sh, const QuantArgs& qa, hipStream_t st) {
+    int cpr = (int)(sh.bcols / 8);
+    int nch = (int)sh.brows * cpr;
+    int nv = (int)cdiv(nch, WG);
+    int shift = is_pow2(cpr) ? ilog2(cpr) : -1;
+    int grid = (int)(sh.gy * sh.gx);
+    const uint4* i4 = static_cast<const uint4*>(in);
+    uint4* o4 = static_cast<uint4*>(out);
+    if (nv <= 1)      k_wgblock<E8, EMU, HWCAST, 1><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    else if (nv <= 2) k_wgblock<E8, EMU, HWCAST, 2><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    else if (nv <= 4) k_wgblock<E8, EMU, HWCAST, 4><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    else              k_wgblock<E8, EMU, HWCAST, 8><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+}
+
+template <bool E8, bool EMU, bool HWCAST>
+static void launch_elementwise(const void* in, void* out, int32_t* meta, int64_t n, int64_t nmeta, int fmt, float scale, int meta_val, hipStream_t st) {
+    int64_t nvec = (aligned16(in) && aligned16(out)) ? n / 8 : 0;
+    int grid = grid_for(nvec > 0 ? nvec : n, 16);
+    k_elementwise<E8, EMU, HWCAST><<<grid, WG, 0, st>>>(static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), meta, n, nvec, nmeta, fmt, scale, meta_val);
+}
+
+#define DISPATCH3(FN, e8, emu, hw, ...)                                            \
+    do {                                                                           \
+        if (e8) {                                                                  \
+            if (emu) FN<true, true, false>(__VA_ARGS__);                           \
+            else if (hw) FN<true, false, true>(__VA_ARGS__);                       \
+            else FN<true, false, false>(__VA_ARGS__);                              \
+        } else {                                                                   \
+            if (emu) FN<false, true, false>(__VA_ARGS__);                          \
+            else if (hw) FN<false, false, true>(__VA_ARGS__);                      \
+            else FN<false, false, false>(__VA_ARGS__);                             \
+        }                                                                          \
+    } while (0)
+
+// Common driver of mor_fake_quantize / mor_block_format / mor_mor_stats.
+static int run_quantize(const void* input, void* output, int32_t* meta, float* stats,
+                        int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                        const QuantArgs& qa, bool e8, uint32_t flags, hipStream_t st) {
+    Shape sh{rows, cols, brows, bcols, cdiv(rows, brows), cdiv(cols, bcols)};
+    const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
+    const bool hw = !(flags & MOR_FLAG_SOFTWARE_CAST);
+    const int64_t nblocks = sh.gy * sh.gx;
+
+    if (qa.qmode == 4) {
+        DISPATCH3(launch_elementwise, e8, emu, hw, input, output, meta, rows * cols, nblocks, qa.fmt, qa.clamp, qa.meta_val, st);
+        return check_launch("k_elementwise");
+    }
+    const bool vec_ok = aligned16(input) && (!output || aligned16(output)) && cols % 8 == 0 && bcols % 8 == 0;
+    const int64_t G = bcols / 8;
+    if (qa.qmode == 2 && !stats && output && vec_ok && brows == 1 && cols % bcols == 0 && is_pow2(G) && G <= 64) {
+        DISPATCH3(launch_rowgroup, e8, emu, hw, qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
+        return check_launch("k_rowgroup");
+    }
+    if (vec_ok && brows * (bcols / 8) <= 8 * WG) {
+        DISPATCH3(launch_wgblock, e8, emu, hw, input, output, meta, stats, sh, qa, st);
+        return check_launch("k_wgblock");
+    }
+    const uint16_t* in16 = static_cast<const uint16_t*>(input);
+    uint16_t* out16 = static_cast<uint16_t*>(output);
+    if (emu) k_generic<true><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, e8 ? 1 : 0);
+    else k_generic<false><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, e8 ? 1 : 0);
+    return check_launch("k_generic");
+}
+
+extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
+                                 int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                                 double clamp_threshold, int64_t mode, int64_t sf_type,
+                                 uint32_t flags, void* stream) {
+    if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
+    if (!output || !meta) return fail(MOR_ERR_INVALID_ARGUMENT, "output / meta is NULL");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int qmode = (int)(mode % 10);                 // FQ:1774
+    QuantArgs qa{};
+    qa.clamp = (float)clamp_threshold;
+    qa.dyn_range = (mode / 100 > 0) ? 1 : 0;            // FQ:1776-1779
+    const bool e8 = (sf_type == 2);                     // FQ:1792, 1797
+    switch (qmode) {
+        case 1: qa.qmode = 1; qa.fmt = -1; qa.meta_val = -1; break;
+        case 2: qa.qmode = 2; qa.fmt = FMT_E4M3; qa.meta_val = 1; break;
+        case 3: qa.qmode = 2; qa.fmt = FMT_E5M2; qa.meta_val = 2; break;
+        case 4: qa.qmode = 4; qa.fmt = FMT_E4M3; qa.meta_val = 1; break;
+        case 5: qa.qmode = 4; qa.fmt = FMT_E5M2; qa.meta_val = 2; break;
+        default: {
+            // FQ:1831-1833, 727-729, 843: bf16 copy, meta 3
+            const int64_t nblocks = cdiv(rows, brows) * cdiv(cols, bcols);
+            if (output != input) {
+                hipError_t e = hipMemcpyAsync(output, input, (size_t)rows * cols * 2, hipMemcpyDeviceToDevice, st);
+                if (e != hipSuccess) return fail(MOR_ERR_LAUNCH, "hipMemcpyAsync: %s", hipGetErrorString(e));
+            }
+            k_fill_i32<<<grid_for(nblocks), WG, 0, st>>>(meta, nblocks, 3);
+            return check_launch("k_fill_i32");
+        }
+    }
+    return run_quantize(input, output, meta, nullptr, rows, cols, brows, bcols, qa, e8, flags, st);
+}
+
+extern "C" int mor_block_format(const void* input, void* output,
+                                int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                                int fmt, int64_t sf_type, uint32_t flags, void* stream) {
+    if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
+    if (!output) return fail(MOR_ERR_INVALID_ARGUMENT, "output is NULL");
+    if (fmt < 0 || fmt > 3) return fail(MOR_ERR_INVALID_ARGUMENT, "unknown format %d", fmt);
+    QuantArgs qa{};
+    qa.qmode = 2; qa.fmt = fmt; qa.meta_val = -1;
+    return run_quantize(input, output, nullptr, nullptr, rows, cols, brows, bcols, qa, sf_type == 2, flags, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                             double clamp_threshold, int64_t mode, int64_t sf_type, float* stats, void* stream) {
+    if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
+    if (!stats) return fail(MOR_ERR_INVALID_ARGUMENT, "stats is NULL");
+    QuantArgs qa{};
+    qa.qmode = 1; qa.fmt = -1; qa.meta_val = -1;
+    qa.clamp = (float)clamp_threshold;
+    qa.dyn_range = (mode / 100 > 0) ? 1 : 0;
+    return run_quantize(input, nullptr, nullptr, stats, rows, cols, brows, bcols, qa, sf_type == 2, MOR_FLAG_DEFAULT, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mor_block_stats(const void* input, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                               float fmax, float* amax, float* scale, int32_t* e8m0, void* stream) {
+    if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
+    if (!amax || !scale || !e8m0) return fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
+    Shape sh{rows, cols, brows, bcols, cdiv(rows, brows), cdiv(cols, bcols)};
+    k_block_stats<<<(int)(sh.gy * sh.gx), WG, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const uint16_t*>(input), sh, fmax, amax, scale, e8m0);
+    return check_launch("k_block_stats");
+}
+
+extern "C" int mor_quant_dequant(const float* input, float* output, int64_t n, int fmt, void* stream) {
+    if (!input || !output || n < 0) return fail(MOR_ERR_INVALID_ARGUMENT, "bad pointer or size");
+    if (fmt < 0 || fmt > 3) return fail(MOR_ERR_INVALID_ARGUMENT, "unknown format %d", fmt);
+    if (n == 0) return MOR_OK;
+    k_quant_dequant<<<grid_for(n, 16), WG, 0, static_cast<hipStream_t>(stream)>>>(input, output, n, fmt);
+    return check_launch("k_quant_dequant");
+}
+
+extern "C" int mor_e4m3_with_e8_scale(const float* input, float* output, int64_t n, int rne, void* stream) {
+    if (!input || !output || n < 0) return fail(MOR_ERR_INVALID_ARGUMENT, "bad pointer or size");
+    if (n == 0) return MOR_OK;
+    k_e4m3_e8_scale<<<grid_for(n, 16), WG, 0, static_cast<hipStream_t>(stream)>>>(input, output, n, rne);
+    return check_launch("k_e4m3_e8_scale");
+}
+
+extern "C" int mor_selftest_hw_cast(uint64_t* mismatches, void* stream) {
+    if (!mismatches) return fail(MOR_ERR_INVALID_ARGUMENT, "mismatches is NULL");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    k_fill_i32<<<1, WG, 0, st>>>(reinterpret_cast<int32_t*>(mismatches), 4, 0);
+    k_selftest_hw_cast<<<256 * 16, WG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
+    return check_launch("k_selftest_hw_cast");
+}
+
+// ---- temporary: filled in by the scaling ops ----
+extern "C" size_t mor_workspace_bytes(int, int64_t, int64_t, int64_t, int64_t) { return 0; }
+extern "C" int mor_block_scaling(const void*, void*, int32_t*, float*, int32_t*, float*, int64_t, int64_t, int64_t, int64_t,
+                                 double, int64_t, int, void*, size_t, uint32_t, void*) { return fail(MOR_ERR_INVALID_ARGUMENT, "not built"); }
+extern "C" int mor_e8mx(const void*, void*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, void*, size_t, uint32_t, void*) { return fail(MOR_ERR_INVALID_ARGUMENT, "not built"); }

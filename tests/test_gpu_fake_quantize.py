@@ -1,0 +1,197 @@
+"""GPU parity of mor_fake_quantize / mor_block_format (C ABI) against the CPU oracle: bit-exact outputs and meta."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mor_oracle as O
+import data_gen
+import torch_emulation as E
+
+pytestmark = pytest.mark.gpu
+
+POKES_RANGE = [(128, 1, 18200, 50968), (0, 70, 21000, 53768), (1, 1, 17262, 50030)]
+POKES_ERROR = [(128, 1, 18403, 51171), (0, 70, 21000, 53768), (1, 1, 17264, 50032)]
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    assert torch.cuda.is_available()
+    return gpu_util
+
+
+def uniform_bits(seed, rows, cols, lo, hi):
+    g = torch.Generator().manual_seed(seed)
+    return E.bf16_to_bits(torch.empty(rows, cols).uniform_(lo, hi, generator=g).to(torch.bfloat16))
+
+
+def assert_same(got, want, what):
+    if not np.array_equal(got, want):
+        bad = np.argwhere(got != want)
+        r, c = bad[0]
+        raise AssertionError(f"{what}: {len(bad)} of {got.size} differ; first at ({r},{c}): got {got[r, c]:#06x} want {want[r, c]:#06x}")
+
+
+def test_hw_cast_selftest(G):
+    """All 2^32 fp32 inputs in range: the gfx950 converts equal the software model of the reference's cast."""
+    from mor_amd import _cabi
+    m = torch.zeros(2, dtype=torch.int64, device="cuda")
+    print("selftest hw cast", flush=True)
+    _cabi.check(_cabi.lib().mor_selftest_hw_cast(m.data_ptr(), G.stream_ptr()))
+    torch.cuda.synchronize()
+    assert m.tolist() == [0, 0], m.tolist()
+
+
+@pytest.mark.parametrize("pokes,mode,sf,clamp,want_meta", [
+    (POKES_RANGE, 101, 1, 1e-15, [[1, 3], [2, 4]]),
+    (POKES_ERROR, 1, 1, 1e-15, [[1, 3], [3, 4]]),
+    (POKES_RANGE, 101, 2, 1e-25, [[1, 3], [2, 4]]),
+    (POKES_ERROR, 1, 2, 1e-25, None),
+])
+def test_reference_fixtures(G, pokes, mode, sf, clamp, want_meta):
+    a = E.fixture_words(256, 256, pokes)
+    print("fixture", mode, sf, flush=True)
+    out, meta = G.fake_quantize(a, 128, 128, clamp, mode, sf)
+    want, wmeta = O.fake_quantize(a, 128, 128, clamp, mode, sf)
+    if want_meta is not None:
+        assert meta.tolist() == want_meta
+    assert np.array_equal(meta, wmeta)
+    assert_same(out, want, "fixture")
+
+
+def test_golden_file(G):
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_fixtures.npz"))
+    for key, mode, sf, clamp in (("range", 101, 1, 1e-15), ("error", 1, 1, 1e-15), ("range_e8", 101, 2, 1e-25)):
+        out, meta = G.fake_quantize(g[f"{key}_in"], 128, 128, clamp, mode, sf)
+        assert np.array_equal(meta, g[f"{key}_meta"])
+        assert_same(out, g[f"{key}_out"], key)
+
+
+def test_zero_tiny_and_bf16_modes(G):
+    z = np.zeros((256, 256), np.uint16)
+    out, meta = G.fake_quantize(z, 128, 128, 1e-25, 101, 2)
+    assert (meta == 4).all() and np.array_equal(out, z)
+    t = E.bf16_to_bits(torch.ones(256, 256, dtype=torch.bfloat16) * 1e-27)
+    out, meta = G.fake_quantize(t, 128, 128, 1e-25, 101, 2)
+    want, wmeta = O.fake_quantize(t, 128, 128, 1e-25, 101, 2)
+    assert (meta == 4).all() and np.array_equal(out, want)
+    a = uniform_bits(1, 256, 256, -53768.0, 53768.0)
+    for mode in (7, 0, 6, 8, 9):
+        out, meta = G.fake_quantize(a, 128, 128, 1e-15, mode, 1)
+        assert (meta == 3).all() and np.array_equal(out, a)
+
+
+SHAPES = [
+    # rows, cols, brows, bcols        kernel that serves it
+    (64, 256, 1, 32),                 # row groups of 4 lanes (MX)
+    (16, 1024, 1, 8),                 # 1 lane per block
+    (8, 2048, 1, 512),                # 64 lanes per block
+    (32, 4096, 1, 4096),              # workgroup per row
+    (256, 384, 128, 128),             # workgroup per tile
+    (200, 256, 128, 128),             # partial tile rows
+    (64, 192, 64, 64),
+    (48, 112, 16, 56),                # odd chunk count per block row
+    (37, 45, 16, 32),                 # odd columns: generic kernel
+    (1, 32, 1, 32),
+    (130, 260, 128, 128),             # ragged, cols not a multiple of 8
+    (16, 40000, 1, 40000),            # block larger than the register-resident limit
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("mode", [1, 101, 2, 3])
+@pytest.mark.parametrize("sf", [1, 2])
+def test_shapes_modes_vs_oracle(G, shape, mode, sf):
+    rows, cols, br, bc = shape
+    a = data_gen.c2_student_t(rows, cols, seed=rows * 7 + cols)
+    a[0, : min(32, cols)] = 0                      # a zero block / zero elements
+    if rows > 2:
+        a[2, 0] = 0x8000                            # negative zero
+    print("shape", shape, mode, sf, flush=True)
+    out, meta = G.fake_quantize(a, br, bc, 1e-15, mode, sf)
+    want, wmeta, stats = O.fake_quantize(a, br, bc, 1e-15, mode, sf, want_stats=True)
+    if mode == 1:
+        # a decision between E4M3 and BF16 may legitimately flip only if the two error sums tie to 1e-6
+        flip = meta != wmeta
+        if flip.any():
+            e4, e5 = stats[..., 2][flip], stats[..., 3][flip]
+            assert np.all(np.abs(e4 - e5) <= 1e-6 * np.maximum(e4, e5)), (e4, e5)
+            pytest.skip("error sums tie within 1e-6")
+    assert np.array_equal(meta, wmeta)
+    assert_same(out, want, f"{shape} mode {mode} sf {sf}")
+
+
+@pytest.mark.parametrize("mode,fmax", [(4, 448.0), (5, 57344.0)])
+@pytest.mark.parametrize("sf", [1, 2])
+@pytest.mark.parametrize("shape", [(256, 256), (33, 77)])
+def test_current_scaling(G, mode, fmax, sf, shape):
+    a = uniform_bits(5 + mode, shape[0], shape[1], -53768.0, 53768.0)
+    amax = float(E.bits_to_bf16(a).float().abs().max())
+    for scale in (float(np.float32(fmax) / np.float32(amax)), float(np.float32(fmax) / np.float32(amax)) * 3.7):
+        print("current scaling", mode, sf, shape, scale, flush=True)
+        out, meta = G.fake_quantize(a, 128, 128, scale, mode, sf)
+        want, wmeta = O.fake_quantize(a, 128, 128, scale, mode, sf)
+        assert np.array_equal(meta, wmeta)
+        assert_same(out, want, "current scaling")
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2, O.E3M2, O.E2M3])
+@pytest.mark.parametrize("sf", [1, 2])
+@pytest.mark.parametrize("shape", [(64, 512, 1, 32), (256, 256, 128, 128), (37, 45, 16, 32)])
+def test_block_format(G, fmt, sf, shape):
+    rows, cols, br, bc = shape
+    a = data_gen.c2_student_t(rows, cols, seed=fmt * 13 + sf)
+    print("block_format", fmt, sf, shape, flush=True)
+    out = G.block_format(a, br, bc, fmt, sf)
+    assert_same(out, O.block_format(a, br, bc, fmt, sf), "block_format")
+
+
+@pytest.mark.parametrize("flags", [1, 2])
+@pytest.mark.parametrize("mode,sf,shape", [(1, 1, (256, 256, 128, 128)), (2, 2, (64, 512, 1, 32)), (3, 1, (32, 4096, 1, 4096)),
+                                           (1, 2, (256, 256, 128, 128)), (2, 1, (37, 45, 16, 32))])
+def test_flavours(G, flags, mode, sf, shape):
+    """flag 1: torch-emulation flavour == oracle EMU flavour; flag 2: software casts == hardware casts."""
+    rows, cols, br, bc = shape
+    a = data_gen.c4_mixture(rows, cols, seed=mode * 5 + sf, tile=64)
+    print("flavour", flags, mode, sf, shape, flush=True)
+    out, meta = G.fake_quantize(a, br, bc, 1e-15, mode, sf, flags=flags)
+    want, wmeta = O.fake_quantize(a, br, bc, 1e-15, mode, sf, flavour=O.EMU if flags == 1 else O.KERNEL)
+    assert np.array_equal(meta, wmeta)
+    assert_same(out, want, "flavour")
+
+
+def test_inplace_and_stats(G):
+    a = data_gen.c4_mixture(512, 512, seed=77)
+    x = G.to_dev_u16(a)
+    out, meta = G.fake_quantize(a, 128, 128, 1e-15, 1, 1)
+    out2, meta2 = G.fake_quantize(a, 128, 128, 1e-15, 1, 1, inplace=True, x_dev=x)
+    assert np.array_equal(meta, meta2) and np.array_equal(out, out2)
+    st = G.mor_stats(a, 128, 128, 1e-15, 1, 1)
+    _, _, want = O.fake_quantize(a, 128, 128, 1e-15, 1, 1, want_stats=True)
+    assert np.array_equal(st[..., 0], want[..., 0]) and np.array_equal(st[..., 1], want[..., 1])
+    np.testing.assert_allclose(st[..., 2:], want[..., 2:], rtol=1e-6, atol=0)
+    amax, scale, e8 = G.block_stats(a, 1, 32, 448.0)
+    wa, ws, we = O.block_stats(a, 1, 32, 448.0)
+    assert np.array_equal(amax, wa) and np.array_equal(scale.view(np.uint32), ws.view(np.uint32)) and np.array_equal(e8, we)
+
+
+def test_extreme_exponents(G):
+    """Blocks whose scale exponent is outside the fast-path range, bf16 denormals and the largest finite values."""
+    rng = np.random.default_rng(5)
+    a = np.zeros((8, 256), np.uint16)
+    a[0] = rng.integers(0x0001, 0x0080, 256)            # denormals only
+    a[1] = rng.integers(0x0001, 0x0400, 256)            # denormals and tiny normals
+    a[2] = rng.integers(0x7E00, 0x7F80, 256)            # near the top of the range
+    a[3] = rng.integers(0x0000, 0x7F80, 256)            # everything finite, positive
+    a[4] = rng.integers(0x8000, 0xFF80, 256)            # everything finite, negative
+    a[5] = rng.integers(0x0080, 0x1000, 256)
+    a[6] = rng.integers(0x7000, 0x7F80, 256)
+    a[7, ::2] = rng.integers(0x0001, 0x7F80, 128)
+    for (br, bc) in ((1, 32), (1, 256), (8, 256)):
+        for mode, sf in ((2, 1), (2, 2), (3, 1), (3, 2), (1, 1), (1, 2), (101, 2)):
+            print("extreme", br, bc, mode, sf, flush=True)
+            out, meta = G.fake_quantize(a, br, bc, 1e-15, mode, sf)
+            want, wmeta = O.fake_quantize(a, br, bc, 1e-15, mode, sf)
+            assert np.array_equal(meta, wmeta), (br, bc, mode, sf)
+            assert_same(out, want, f"extreme {br}x{bc} mode {mode} sf {sf}")
