@@ -1,0 +1,258 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X fake-quantization path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+One step = one pass of the MX block-scaling workload (BASELINE configs[1]) over an 8192 x 8192 bf16 tensor
+resident in HBM: 1 x 32 blocks, power-of-two (E8M0) shared scale, elements cast to E4M3, E5M2 and E2M3 (three
+launches).  The printed JSON line reports algorithmic HBM GB/s (2 B read + 2 B written per element + 4 B of meta per
+block where the op returns meta) for the whole step, the roofline fraction of the slowest of the three kernels
+from HIP events recorded around every launch in the timed region, the other configurations, and the CPU oracle
+timed on a bounded sample of the same workload on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
+    ap.add_argument("--rows", type=int, default=8192)
+    ap.add_argument("--cols", type=int, default=8192)
+    return ap.parse_args()
+
+
+def gen_c2_gpu(torch, rows, cols, seed=1002):
+    """Student-t(3) * 0.02 with 0.1 % of the elements x1000, generated on the GPU."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    z = torch.randn(rows, cols, device="cuda", generator=g)
+    d = torch.zeros(rows, cols, device="cuda")
+    for _ in range(3):
+        d += torch.randn(rows, cols, device="cuda", generator=g) ** 2
+    t = z / torch.sqrt(d / 3) * 0.02
+    mask = torch.rand(rows, cols, device="cuda", generator=g) < 1e-3
+    return torch.where(mask, t * 1000, t).to(torch.bfloat16).contiguous()
+
+
+def gen_c4_gpu(torch, rows, cols, seed=1004, tile=128):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    gy, gx = (rows + tile - 1) // tile, (cols + tile - 1) // tile
+    u = torch.rand(gy, gx, device="cuda", generator=g)
+    kind = torch.where(u < 0.7, 0, torch.where(u < 0.9, 1, 2)).repeat_interleave(tile, 0).repeat_interleave(tile, 1)[:rows, :cols]
+    t = torch.randn(rows, cols, device="cuda", generator=g)
+    sign = torch.where(torch.rand(rows, cols, device="cuda", generator=g) < 0.5, -1.0, 1.0)
+    t = torch.where(kind == 1, torch.exp(3 * t) * sign, torch.where(kind == 2, t * 1e-4, t))
+    return t.to(torch.bfloat16).contiguous()
+
+
+class Launcher:
+    """Thin caller of the C ABI on torch's current stream."""
+
+    def __init__(self, torch, cabi):
+        self.torch, self.cabi, self.L = torch, cabi, cabi.lib()
+
+    def stream(self):
+        return self.torch.cuda.current_stream().cuda_stream
+
+    def fake_quantize(self, x, out, meta, br, bc, clamp, mode, sf):
+        r, c = x.shape
+        self.cabi.check(self.L.mor_fake_quantize(x.data_ptr(), out.data_ptr(), meta.data_ptr(), r, c, br, bc,
+                                                 float(clamp), mode, sf, 0, self.stream()))
+
+    def block_format(self, x, out, br, bc, fmt, sf):
+        r, c = x.shape
+        self.cabi.check(self.L.mor_block_format(x.data_ptr(), out.data_ptr(), r, c, br, bc, fmt, sf, 0, self.stream()))
+
+
+def time_launches(torch, fn, steps, warmup):
+    """-> (mean ms per launch from per-launch HIP events, wall ms per launch)"""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return sum(a.elapsed_time(b) for a, b in ev) / steps, wall
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every quantization block is independent, so more GPUs only shard rows; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from mor_amd import _cabi
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP library has no CPU path)", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    run = Launcher(torch, _cabi)
+    rows, cols = args.rows, args.cols
+    K, W = args.steps, args.warmup
+
+    x = gen_c2_gpu(torch, rows, cols)
+    out = torch.empty_like(x)
+    meta = torch.empty((rows, cols // 32), dtype=torch.int32, device="cuda")
+    nelem = rows * cols
+    nblocks = nelem // 32
+    launches = [
+        ("mx_e4m3", lambda: run.fake_quantize(x, out, meta, 1, 32, 0.0, 2, 2), nelem * 4 + nblocks * 4),
+        ("mx_e5m2", lambda: run.fake_quantize(x, out, meta, 1, 32, 0.0, 3, 2), nelem * 4 + nblocks * 4),
+        ("mx_e2m3", lambda: run.block_format(x, out, 1, 32, _cabi.FMT_E2M3, 2), nelem * 4),
+    ]
+    bytes_per_step = sum(b for _, _, b in launches)
+
+    def step(events=None):
+        for i, (_, fn, _) in enumerate(launches):
+            if events is not None:
+                events[i][0].record()
+            fn()
+            if events is not None:
+                events[i][1].record()
+
+    for _ in range(W):
+        step()
+    torch.cuda.synchronize()
+    evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in launches] for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(K):
+        step(evs[k])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / K
+    value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
+
+    per_kernel = {}
+    for i, (name, _, nbytes) in enumerate(launches):
+        ms = sum(evs[k][i][0].elapsed_time(evs[k][i][1]) for k in range(K)) / K
+        per_kernel[name] = {"ms": round(ms, 5), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                            "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "bytes": nbytes}
+    dom = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": per_kernel[dom]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": per_kernel[dom]["frac"], "traffic": None, "per_kernel": per_kernel}
+
+    extra = {}
+    if not args.no_extra:
+        extra = other_configs(torch, run, _cabi, max(5, K // 2), max(2, W // 2))
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(torch, x)
+
+    line = {
+        "metric": "fake-quant HBM GB/s (rd+wr), MX 1x32 E8M0 block scaling on 8192x8192 bf16 (E4M3+E5M2+E2M3)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 in/out, fp32 + fp8/fp6 arithmetic", "data": "synthetic",
+        "config": {"workload": f"configs[1]: MX block scaling {rows}x{cols} bf16, 1x32 blocks, E8M0 scale, E4M3+E5M2+E2M3 per step",
+                   "elements_per_s": round(3 * nelem / (ms_per_step * 1e-3), 0), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "other_configs": extra,
+    }
+    print(json.dumps(line))
+
+
+def other_configs(torch, run, cabi, K, W):
+    """Per-launch figures for the remaining configurations (HIP events around each launch)."""
+    res = {}
+
+    def add(name, fn, nbytes, nelem):
+        ms, wall = time_launches(torch, fn, K, W)
+        res[name] = {"ms": round(ms, 5), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "elements_per_s": round(nelem / (ms * 1e-3), 0)}
+
+    # MoR 128x128 on 8192x8192 N(0,1) and on the C4 mixture at its full size
+    g = torch.Generator(device="cuda").manual_seed(1001)
+    x = torch.randn(8192, 8192, device="cuda", generator=g).to(torch.bfloat16)
+    out = torch.empty_like(x)
+    meta = torch.empty((64, 64), dtype=torch.int32, device="cuda")
+    n = x.numel()
+    add("mor_128x128_8192x8192_normal", lambda: run.fake_quantize(x, out, meta, 128, 128, 1e-15, 1, 1), n * 4 + meta.numel() * 4, n)
+    add("copy_mode7_8192x8192", lambda: run.fake_quantize(x, out, meta, 128, 128, 0.0, 7, 1), n * 4 + meta.numel() * 4, n)
+    add("block_e4m3_128x128_8192x8192_fp32scale", lambda: run.fake_quantize(x, out, meta, 128, 128, 0.0, 2, 1), n * 4 + meta.numel() * 4, n)
+    # C1: per-tensor E4M3, 4096x4096, scale from the tensor amax (the quantize pass only: 4 B/element)
+    x1 = x[:4096, :4096].contiguous()
+    o1 = torch.empty_like(x1)
+    m1 = torch.empty((32, 32), dtype=torch.int32, device="cuda")
+    scale = float(448.0 / x1.float().abs().max().item())
+    add("c1_per_tensor_e4m3_4096x4096", lambda: run.fake_quantize(x1, o1, m1, 128, 128, scale, 4, 1), x1.numel() * 4, x1.numel())
+    del x, out, x1, o1
+    # C3: per-row fp32 scale, 16384x4096
+    g = torch.Generator(device="cuda").manual_seed(1003)
+    w = torch.randn(16384, 4096, device="cuda", generator=g) * 0.02
+    hot = torch.randperm(16384, device="cuda", generator=g)[:164]
+    w[hot] *= 100
+    w[7] = 0
+    w = w.to(torch.bfloat16)
+    ow = torch.empty_like(w)
+    mw = torch.empty((16384, 1), dtype=torch.int32, device="cuda")
+    add("c3_per_row_e4m3_16384x4096", lambda: run.fake_quantize(w, ow, mw, 1, 4096, 0.0, 2, 1), w.numel() * 4 + 16384 * 4, w.numel())
+    add("c3_per_row_e5m2_16384x4096", lambda: run.fake_quantize(w, ow, mw, 1, 4096, 0.0, 3, 1), w.numel() * 4 + 16384 * 4, w.numel())
+    del w, ow
+    # C4: MoR 128x128 on the 16384x14336 mixture
+    x4 = gen_c4_gpu(torch, 16384, 14336)
+    o4 = torch.empty_like(x4)
+    m4 = torch.empty((128, 112), dtype=torch.int32, device="cuda")
+    add("c4_mor_128x128_16384x14336_mixture", lambda: run.fake_quantize(x4, o4, m4, 128, 128, 1e-15, 1, 1), x4.numel() * 4 + m4.numel() * 4, x4.numel())
+    torch.cuda.synchronize()
+    hist = torch.bincount(m4.flatten(), minlength=13).tolist()
+    res["c4_mor_128x128_16384x14336_mixture"]["meta_histogram"] = {str(i): h for i, h in enumerate(hist) if h}
+    # launch overhead: a 1x32 tensor
+    xs = torch.randn(1, 32, device="cuda").to(torch.bfloat16)
+    os_ = torch.empty_like(xs)
+    ms_ = torch.empty((1, 1), dtype=torch.int32, device="cuda")
+    ms, wall = time_launches(torch, lambda: run.fake_quantize(xs, os_, ms_, 1, 32, 0.0, 2, 2), 200, 20)
+    res["tiny_1x32"] = {"us_per_call_events": round(ms * 1e3, 2), "us_per_call_wall": round(wall * 1e3, 2)}
+    return res
+
+
+def cpu_baseline(torch, x_gpu):
+    """The CPU oracle (a port of the reference arithmetic) on the first rows of the same tensor, all host threads."""
+    from oracle import mor_oracle as O
+    import numpy as np
+    O.lib()
+    rows = 512
+    a = x_gpu[:rows].cpu().view(torch.int16).numpy().view(np.uint16).copy()
+    n = a.size
+    nbytes = 0
+    t_total = 0.0
+    reps = 0
+    t_start = time.perf_counter()
+    while True:
+        t0 = time.perf_counter()
+        O.fake_quantize(a, 1, 32, 0.0, 2, 2)
+        O.fake_quantize(a, 1, 32, 0.0, 3, 2)
+        O.block_format(a, 1, 32, O.E2M3, 2)
+        t_total += time.perf_counter() - t0
+        nbytes += 3 * n * 4 + 2 * (n // 32) * 4
+        reps += 1
+        if time.perf_counter() - t_start > 12.0 or reps >= 50:
+            break
+    return {"value": round(nbytes / t_total / 1e9, 3), "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+            "sample": f"first {rows} rows of the benchmark tensor ({n} elements), E4M3+E5M2+E2M3, {reps} repetitions, "
+                      f"C oracle with OpenMP over blocks"}
+
+
+if __name__ == "__main__":
+    main()

@@ -158,6 +158,22 @@ __device__ __forceinline__ Scale make_scale(float s) {
     return sc;
 }
 
+// Exponent of the power-of-two scale without the division: for amax = m * 2^ea (1 <= m < 2, a normal bf16)
+// and fmax = f * 2^eb, floor(log2(fl(fmax / amax))) = eb - ea - (m > f).  The fp32 quotient cannot round up to a
+// power of two because m has 8 significant bits.  Returns the Scale of FQ:251-252 with s left unset (E8 paths only
+// use e8); `fast` additionally requires a normal amax.
+template <int F> __device__ __forceinline__ Scale make_scale_e8(float amax) {
+    constexpr int eb = (F == FMT_E4M3) ? 8 : (F == FMT_E5M2) ? 15 : (F == FMT_E3M2) ? 4 : 2;
+    constexpr uint32_t mth = (F == FMT_E2M3) ? 0x70u : 0x60u;       // mantissa field of 1.875 / 1.75
+    const uint32_t b = f2u(amax);
+    const int ea = (int)(b >> 23);
+    Scale sc;
+    sc.s = 0.0f;
+    sc.e8 = (127 + eb) - ea - (((b >> 16) & 0x7Fu) > mth ? 1 : 0);
+    sc.fast = (ea != 0) && (sc.e8 >= -100) && (sc.e8 <= 100);
+    return sc;
+}
+
 // Fast E8 path on a pair (lo, hi) of one packed word, result packed.  For E4M3/E5M2:
 //   |x| * 2^e8 (exact), hardware convert and back, then integer exponent subtraction clamped at 0,
 //   which also yields the reference's 2^(-e8-127) for a zero cast result when e8 < 0.  The sign
@@ -212,36 +228,25 @@ template <int F, bool E8, bool EMU> __device__ __forceinline__ float sqdd_exact(
     else return sqdd_fp32_exact<F, EMU>(x, sc.s);
 }
 
-// One packed word -> one packed word.
-template <int F, bool E8, bool EMU, bool HWCAST, bool CLAMP = false>
-__device__ __forceinline__ uint32_t fq_pair(uint32_t w, const Scale& sc) {
-    if constexpr (!EMU && HWCAST) {
-        if (sc.fast) {
-            if constexpr (E8) return e8_pair_fast<F, CLAMP>(w, sc.e8);
-            else return fp32_pair_fast<F, CLAMP>(w, sc.s);
-        }
-    }
-    float lo = sqdd_exact<F, E8, EMU>(bf16_lo(w), sc);
-    float hi = sqdd_exact<F, E8, EMU>(bf16_hi(w), sc);
-    return store_pair<EMU>(lo, hi);
+// One packed word -> one packed word, fast path only (the caller has checked sc.fast).
+template <int F, bool E8, bool CLAMP = false>
+__device__ __forceinline__ uint32_t fq_pair_fast(uint32_t w, const Scale& sc) {
+    if constexpr (E8) return e8_pair_fast<F, CLAMP>(w, sc.e8);
+    else return fp32_pair_fast<F, CLAMP>(w, sc.s);
 }
-
-// fp32 result (no bf16 store) of one element, used by the error sums
-template <int F, bool E8, bool EMU, bool HWCAST> __device__ __forceinline__ float sqdd_value(float x, const Scale& sc) {
-    if constexpr (!EMU && HWCAST && Fmt<F>::hw) {
-        if (sc.fast) {
-            if constexpr (E8) {
-                const int e8s = sc.e8 << 23;
-                uint32_t p = hw_pack2<F>(ldexpf(fabsf(x), sc.e8), 0.0f);
-                int m = max((int)f2u(hw_unpack<F, 0>(p)) - e8s, 0);
-                return u2f((uint32_t)m | (f2u(x) & 0x80000000u));
-            } else {
-                uint32_t p = hw_pack2<F>(x * sc.s, 0.0f);
-                return hw_unpack<F, 0>(p) / sc.s;
-            }
-        }
-    }
-    return sqdd_exact<F, E8, EMU>(x, sc);
+template <int F, bool E8, bool CLAMP = false>
+__device__ __forceinline__ uint4 fq_vec_fast(uint4 v, const Scale& sc) {
+    uint4 r;
+    r.x = fq_pair_fast<F, E8, CLAMP>(v.x, sc);
+    r.y = fq_pair_fast<F, E8, CLAMP>(v.y, sc);
+    r.z = fq_pair_fast<F, E8, CLAMP>(v.z, sc);
+    r.w = fq_pair_fast<F, E8, CLAMP>(v.w, sc);
+    return r;
+}
+// One packed word -> one packed word, exact path.
+template <int F, bool E8, bool EMU>
+__device__ __forceinline__ uint32_t fq_pair_exact(uint32_t w, const Scale& sc) {
+    return store_pair<EMU>(sqdd_exact<F, E8, EMU>(bf16_lo(w), sc), sqdd_exact<F, E8, EMU>(bf16_hi(w), sc));
 }
 
 // ---------------------------------------------------------------- wave64 reductions
@@ -265,6 +270,19 @@ __device__ __forceinline__ float group_max(float v, int G) {
     if (G >= 32) v = fmaxf(v, __shfl_xor(v, 16));
     if (G >= 64) v = fmaxf(v, __shfl_xor(v, 32));
     return v;
+}
+// same with the group size known at compile time (GT > 0), else the run-time G
+template <int GT> __device__ __forceinline__ float group_max_t(float v, int G) {
+    if constexpr (GT == 0) return group_max(v, G);
+    else {
+        if constexpr (GT >= 2) v = fmaxf(v, dpp_f<DPP_XOR1>(v));
+        if constexpr (GT >= 4) v = fmaxf(v, dpp_f<DPP_XOR2>(v));
+        if constexpr (GT >= 8) v = fmaxf(v, dpp_f<DPP_HALF_MIRROR>(v));
+        if constexpr (GT >= 16) v = fmaxf(v, dpp_f<DPP_MIRROR>(v));
+        if constexpr (GT >= 32) v = fmaxf(v, __shfl_xor(v, 16));
+        if constexpr (GT >= 64) v = fmaxf(v, __shfl_xor(v, 32));
+        return v;
+    }
 }
 __device__ __forceinline__ uint32_t group_umin(uint32_t v, int G) {
     if (G >= 2) v = min(v, dpp_u<DPP_XOR1>(v));

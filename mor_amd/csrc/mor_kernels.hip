@@ -15,6 +15,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <string.h>
 
 #include "mor_device.h"
 #include "../../include/mor_hip.h"
@@ -40,36 +41,25 @@ struct QuantArgs {
 };
 
 // ------------------------------------------------------------------------------------------------
-// per-format dispatch of one packed word (block-uniform switch)
-template <bool E8, bool EMU, bool HWCAST, bool CLAMP = false>
-__device__ __forceinline__ uint32_t fq_word(uint32_t w, int fmt, const Scale& sc) {
-    switch (fmt) {
-        case FMT_E4M3: return fq_pair<FMT_E4M3, E8, EMU, HWCAST, CLAMP>(w, sc);
-        case FMT_E5M2: return fq_pair<FMT_E5M2, E8, EMU, HWCAST, CLAMP>(w, sc);
-        case FMT_E3M2: return fq_pair<FMT_E3M2, E8, EMU, HWCAST, CLAMP>(w, sc);
-        default:       return fq_pair<FMT_E2M3, E8, EMU, HWCAST, CLAMP>(w, sc);
-    }
-}
-
-template <int F, bool E8, bool EMU, bool HWCAST, bool CLAMP = false>
-__device__ __forceinline__ uint4 fq_vec(uint4 v, const Scale& sc) {
-    uint4 r;
-    r.x = fq_pair<F, E8, EMU, HWCAST, CLAMP>(v.x, sc);
-    r.y = fq_pair<F, E8, EMU, HWCAST, CLAMP>(v.y, sc);
-    r.z = fq_pair<F, E8, EMU, HWCAST, CLAMP>(v.z, sc);
-    r.w = fq_pair<F, E8, EMU, HWCAST, CLAMP>(v.w, sc);
-    return r;
-}
-
-template <bool E8, bool EMU>
-__device__ __forceinline__ uint16_t fq_one_exact(uint16_t h, int fmt, const Scale& sc) {
+// exact one-element quantization with run-time format / scale type (only used inside non-unrolled loops)
+template <bool EMU>
+__device__ __forceinline__ uint16_t fq_one_exact(uint16_t h, int fmt, bool e8, const Scale& sc) {
     float x = bf16_one(h);
     float r;
-    switch (fmt) {
-        case FMT_E4M3: r = sqdd_exact<FMT_E4M3, E8, EMU>(x, sc); break;
-        case FMT_E5M2: r = sqdd_exact<FMT_E5M2, E8, EMU>(x, sc); break;
-        case FMT_E3M2: r = sqdd_exact<FMT_E3M2, E8, EMU>(x, sc); break;
-        default:       r = sqdd_exact<FMT_E2M3, E8, EMU>(x, sc); break;
+    if (e8) {
+        switch (fmt) {
+            case FMT_E4M3: r = sqdd_exact<FMT_E4M3, true, EMU>(x, sc); break;
+            case FMT_E5M2: r = sqdd_exact<FMT_E5M2, true, EMU>(x, sc); break;
+            case FMT_E3M2: r = sqdd_exact<FMT_E3M2, true, EMU>(x, sc); break;
+            default:       r = sqdd_exact<FMT_E2M3, true, EMU>(x, sc); break;
+        }
+    } else {
+        switch (fmt) {
+            case FMT_E4M3: r = sqdd_exact<FMT_E4M3, false, EMU>(x, sc); break;
+            case FMT_E5M2: r = sqdd_exact<FMT_E5M2, false, EMU>(x, sc); break;
+            case FMT_E3M2: r = sqdd_exact<FMT_E3M2, false, EMU>(x, sc); break;
+            default:       r = sqdd_exact<FMT_E2M3, false, EMU>(x, sc); break;
+        }
     }
     return store_bf16<EMU>(r);
 }
@@ -101,203 +91,25 @@ __device__ __forceinline__ int mor_fmt_of(int qt) {
     }
 }
 
-// One element's two error terms, FQ:504-542: |q/x - 1| for E4M3 and E5M2 with scales fmax/amax.
-template <bool E8, bool EMU, bool HWCAST>
-__device__ __forceinline__ void err_terms(float x, const Scale& s4, const Scale& s5, float& e4, float& e5) {
+// One element's two error terms with IEEE divisions, FQ:504-542.
+template <bool EMU>
+__device__ __forceinline__ void err_terms_exact(float x, bool e8, const Scale& s4, const Scale& s5, float& e4, float& e5) {
     if (x != 0.0f) {
-        float q4 = sqdd_value<FMT_E4M3, E8, EMU, HWCAST>(x, s4);
-        float q5 = sqdd_value<FMT_E5M2, E8, EMU, HWCAST>(x, s5);
+        float q4 = e8 ? sqdd_exact<FMT_E4M3, true, EMU>(x, s4) : sqdd_exact<FMT_E4M3, false, EMU>(x, s4);
+        float q5 = e8 ? sqdd_exact<FMT_E5M2, true, EMU>(x, s5) : sqdd_exact<FMT_E5M2, false, EMU>(x, s5);
         e4 += fabsf(q4 / x - 1.0f);
         e5 += fabsf(q5 / x - 1.0f);
     }
 }
 
 // ------------------------------------------------------------------------------------------------
-// k_elementwise: modes 4 / 5 (FQ:825-842): every element uses the caller's scale; meta is a constant.
-template <bool E8, bool EMU, bool HWCAST>
-__global__ __launch_bounds__(WG) void k_elementwise(const uint16_t* in, uint16_t* out,
-                                                    int32_t* __restrict__ meta, int64_t n, int64_t nvec,
-                                                    int64_t nmeta, int fmt, float scale, int meta_val) {
-    const Scale sc = make_scale(scale);
-    const int64_t stride = (int64_t)gridDim.x * WG;
-    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
-    if (meta) for (int64_t i = gtid; i < nmeta; i += stride) meta[i] = meta_val;
-    const uint4* in4 = reinterpret_cast<const uint4*>(in);
-    uint4* out4 = reinterpret_cast<uint4*>(out);
-    for (int64_t c = gtid; c < nvec; c += stride) {
-        uint4 v = in4[c];
-        uint4 r;
-        r.x = fq_word<E8, EMU, HWCAST, true>(v.x, fmt, sc);
-        r.y = fq_word<E8, EMU, HWCAST, true>(v.y, fmt, sc);
-        r.z = fq_word<E8, EMU, HWCAST, true>(v.z, fmt, sc);
-        r.w = fq_word<E8, EMU, HWCAST, true>(v.w, fmt, sc);
-        out4[c] = r;
-    }
-    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = fq_one_exact<E8, EMU>(in[i], fmt, sc);
-}
-
-__global__ __launch_bounds__(WG) void k_fill_i32(int32_t* p, int64_t n, int32_t v) {
-    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) p[i] = v;
-}
-
-// ------------------------------------------------------------------------------------------------
-// k_rowgroup: blocks of 1 x 8G elements; the tensor is a flat array of 16-byte chunks and a block is G
-// consecutive chunks held by G consecutive lanes.  U chunks per thread are in flight per iteration.
-template <int F, bool E8, bool EMU, bool HWCAST, int U>
-__global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out,
-                                                 int32_t* __restrict__ meta, int64_t nchunks, int G, int logG,
-                                                 int meta_val) {
-    const int64_t stride = (int64_t)gridDim.x * WG;
-    for (int64_t c0 = (int64_t)blockIdx.x * WG + threadIdx.x; c0 < nchunks; c0 += stride * U) {
-        uint4 v[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int64_t c = c0 + (int64_t)u * stride;
-            if (c < nchunks) v[u] = in[c];
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int64_t c = c0 + (int64_t)u * stride;
-            if (c < nchunks) {
-                float amax = 0.0f;
-                acc_amax(amax, v[u].x); acc_amax(amax, v[u].y); acc_amax(amax, v[u].z); acc_amax(amax, v[u].w);
-                amax = group_max(amax, G);
-                uint4 r = v[u];
-                if (amax > 0.0f) {                       // FQ:802, 814: a zero block passes through
-                    const Scale sc = make_scale(Fmt<F>::fmax / amax);
-                    r = fq_vec<F, E8, EMU, HWCAST>(v[u], sc);
-                }
-                out[c] = r;
-                if (meta_val >= 0 && (c & (G - 1)) == 0) meta[c >> logG] = meta_val;
-            }
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
-// k_wgblock: one workgroup per quantization block, the block held in registers (NV 16-byte vectors per lane).
-// Chunk ch = v * 256 + tid of the block sits at block row ch / cpr, chunk column ch % cpr.
-template <bool E8, bool EMU, bool HWCAST, int NV>
-__global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out,
-                                                int32_t* __restrict__ meta, float* __restrict__ stats,
-                                                Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
-    __shared__ float s_f[2][WAVES];
-    __shared__ uint32_t s_u[WAVES];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t bid = blockIdx.x;
-    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
-    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
-    const int64_t row_stride = sh.cols >> 3;                       // chunks per tensor row
-    const int rows_valid = (int)min(sh.brows, sh.rows - r0);
-    const int cols_valid = (int)min((int64_t)cpr, (sh.cols - c0) >> 3);
-    const int nch = (int)sh.brows * cpr;
-
-    uint4 v[NV];
-    int64_t idx[NV];
-    bool ok[NV];
-#pragma unroll
-    for (int k = 0; k < NV; ++k) {
-        int ch = k * WG + tid;
-        int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
-        int cc = ch - r * cpr;
-        ok[k] = (ch < nch) && (r < rows_valid) && (cc < cols_valid);
-        idx[k] = (r0 + r) * row_stride + (c0 >> 3) + cc;
-        if (ok[k]) v[k] = in[idx[k]];
-    }
-
-    // pass 1 (registers): amax and min over non-zero magnitudes, FQ:407-485
-    float amax = 0.0f;
-    uint32_t amin_m1 = AMIN_INIT_M1;
-#pragma unroll
-    for (int k = 0; k < NV; ++k)
-        if (ok[k]) {
-            acc_amax(amax, v[k].x); acc_amax(amax, v[k].y); acc_amax(amax, v[k].z); acc_amax(amax, v[k].w);
-            if (qa.qmode == 1) { acc_amin(amin_m1, v[k].x); acc_amin(amin_m1, v[k].y); acc_amin(amin_m1, v[k].z); acc_amin(amin_m1, v[k].w); }
-        }
-    amax = group_max(amax, 64);
-    amin_m1 = group_umin(amin_m1, 64);
-    if (lane == 0) { s_f[0][wave] = amax; s_u[wave] = amin_m1; }
-    __syncthreads();
-    amax = fmaxf(fmaxf(s_f[0][0], s_f[0][1]), fmaxf(s_f[0][2], s_f[0][3]));
-    amin_m1 = min(min(s_u[0], s_u[1]), min(s_u[2], s_u[3]));
-    const float amin = u2f(amin_m1 + 1u);
-
-    int fmt = qa.fmt;
-    int meta_val = qa.meta_val;
-    float e4 = 0.0f, e5 = 0.0f;
-    if (qa.qmode == 1) {
-        int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
-        if (qt == Q_UNKNOWN) {
-            // pass 2 (registers): the two error sums, FQ:487-584.  amax > 0 here.
-            const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
-#pragma unroll
-            for (int k = 0; k < NV; ++k)
-                if (ok[k]) {
-                    const uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        err_terms<E8, EMU, HWCAST>(bf16_lo(w[j]), s4, s5, e4, e5);
-                        err_terms<E8, EMU, HWCAST>(bf16_hi(w[j]), s4, s5, e4, e5);
-                    }
-                }
-            e4 = wave_sum(e4);
-            e5 = wave_sum(e5);
-            __syncthreads();                     // s_f[0] was read by every wave above
-            if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
-            __syncthreads();
-            e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
-            e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
-            qt = mor_decide_error(amax, qa.clamp, e4, e5);
-        }
-        meta_val = qt;
-        fmt = mor_fmt_of(qt);
-    }
-    if (tid == 0) {
-        if (meta && meta_val >= 0) meta[bid] = meta_val;
-        if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
-    }
-    if (!out) return;
-
-    // pass 3 (registers): quantize and store, FQ:733-851
-    const bool copy = (fmt < 0) || !(amax > 0.0f);
-    const Scale sc = make_scale(copy ? 1.0f : fmax_of(fmt) / amax);
-    if (copy) {
-        if (out != in) {
-#pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = v[k];
-        }
-        return;
-    }
-    switch (fmt) {
-        case FMT_E4M3:
-#pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = fq_vec<FMT_E4M3, E8, EMU, HWCAST>(v[k], sc);
-            break;
-        case FMT_E5M2:
-#pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = fq_vec<FMT_E5M2, E8, EMU, HWCAST>(v[k], sc);
-            break;
-        case FMT_E3M2:
-#pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = fq_vec<FMT_E3M2, E8, EMU, HWCAST>(v[k], sc);
-            break;
-        default:
-#pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) out[idx[k]] = fq_vec<FMT_E2M3, E8, EMU, HWCAST>(v[k], sc);
-            break;
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
-// k_generic: any shape.  One workgroup per block, element i of the block at (i / bw, i % bw).
+// generic_block: one workgroup quantizes one block of any shape straight from memory with the exact arithmetic.
+// It is the body of k_generic and the fallback of k_wgblock for blocks outside the fast range.
 template <bool EMU>
-__global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* out,
-                                                int32_t* __restrict__ meta, float* __restrict__ stats,
-                                                Shape sh, QuantArgs qa, int e8) {
-    __shared__ float s_f[2][WAVES];
-    __shared__ uint32_t s_u[WAVES];
+__device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out, int32_t* meta, float* stats,
+                                              const Shape& sh, const QuantArgs& qa, bool e8, int64_t bid,
+                                              float (*s_f)[WAVES], uint32_t* s_u) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t bid = blockIdx.x;
     const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
     const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
     const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
@@ -305,6 +117,7 @@ __global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* ou
 
     float amax = 0.0f;
     uint32_t amin_m1 = AMIN_INIT_M1;
+#pragma unroll 1
     for (int64_t i = tid; i < nel; i += WG) {
         int64_t r = i / bw, c = i - r * bw;
         uint32_t a = ((uint32_t)in[(r0 + r) * sh.cols + c0 + c] << 16) & 0x7FFFFFFFu;
@@ -313,6 +126,7 @@ __global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* ou
     }
     amax = group_max(amax, 64);
     amin_m1 = group_umin(amin_m1, 64);
+    __syncthreads();
     if (lane == 0) { s_f[0][wave] = amax; s_u[wave] = amin_m1; }
     __syncthreads();
     amax = fmaxf(fmaxf(s_f[0][0], s_f[0][1]), fmaxf(s_f[0][2], s_f[0][3]));
@@ -326,11 +140,10 @@ __global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* ou
         int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
         if (qt == Q_UNKNOWN) {
             const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
+#pragma unroll 1
             for (int64_t i = tid; i < nel; i += WG) {
                 int64_t r = i / bw, c = i - r * bw;
-                float x = bf16_one(in[(r0 + r) * sh.cols + c0 + c]);
-                if (e8) err_terms<true, EMU, false>(x, s4, s5, e4, e5);
-                else err_terms<false, EMU, false>(x, s4, s5, e4, e5);
+                err_terms_exact<EMU>(bf16_one(in[(r0 + r) * sh.cols + c0 + c]), e8, s4, s5, e4, e5);
             }
             e4 = wave_sum(e4);
             e5 = wave_sum(e5);
@@ -352,12 +165,365 @@ __global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* ou
     const bool copy = (fmt < 0) || !(amax > 0.0f);
     if (copy && out == in) return;
     const Scale sc = make_scale(copy ? 1.0f : fmax_of(fmt) / amax);
+#pragma unroll 1
     for (int64_t i = tid; i < nel; i += WG) {
         int64_t r = i / bw, c = i - r * bw;
         int64_t at = (r0 + r) * sh.cols + c0 + c;
         uint16_t h = in[at];
-        if (!copy) h = e8 ? fq_one_exact<true, EMU>(h, fmt, sc) : fq_one_exact<false, EMU>(h, fmt, sc);
+        if (!copy) h = fq_one_exact<EMU>(h, fmt, e8, sc);
         out[at] = h;
+    }
+}
+
+template <bool EMU>
+__global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* out, int32_t* __restrict__ meta,
+                                                float* __restrict__ stats, Shape sh, QuantArgs qa, int e8) {
+    __shared__ float s_f[2][WAVES];
+    __shared__ uint32_t s_u[WAVES];
+    generic_block<EMU>(in, out, meta, stats, sh, qa, e8 != 0, blockIdx.x, s_f, s_u);
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_elementwise: modes 4 / 5 (FQ:825-842): every element uses the caller's scale; meta is a constant.
+// The host picks the fast kernel when the scale is in the fast range, else (or for the other flavours) the exact one.
+// EW_NV = 16-byte vectors per thread of the flat kernels (fewer for small tensors, so that every CU gets work)
+template <bool E8, int EW_NV>
+__global__ __launch_bounds__(WG) void k_elementwise_fast(const uint16_t* in, uint16_t* out, int32_t* __restrict__ meta,
+                                                         int64_t n, int64_t nvec, int64_t nmeta, int fmt, float scale, int meta_val) {
+    const Scale sc = make_scale(scale);
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    if (meta) for (int64_t i = gtid; i < nmeta; i += stride) meta[i] = meta_val;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    uint4* out4 = reinterpret_cast<uint4*>(out);
+    const int64_t base = (int64_t)blockIdx.x * (EW_NV * WG) + threadIdx.x;
+    uint4 v[EW_NV];
+#pragma unroll
+    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = in4[c]; }
+    if (fmt == FMT_E4M3) {
+#pragma unroll
+        for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) out4[c] = fq_vec_fast<FMT_E4M3, E8, true>(v[k], sc); }
+    } else {
+#pragma unroll
+        for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) out4[c] = fq_vec_fast<FMT_E5M2, E8, true>(v[k], sc); }
+    }
+#pragma unroll 1
+    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = fq_one_exact<false>(in[i], fmt, E8, sc);
+}
+
+template <bool EMU>
+__global__ __launch_bounds__(WG) void k_elementwise_exact(const uint16_t* in, uint16_t* out, int32_t* __restrict__ meta,
+                                                          int64_t n, int64_t nmeta, int fmt, int e8, float scale, int meta_val) {
+    const Scale sc = make_scale(scale);
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    if (meta) for (int64_t i = gtid; i < nmeta; i += stride) meta[i] = meta_val;
+#pragma unroll 1
+    for (int64_t i = gtid; i < n; i += stride) out[i] = fq_one_exact<EMU>(in[i], fmt, e8 != 0, sc);
+}
+
+__global__ __launch_bounds__(WG) void k_fill_i32(int32_t* p, int64_t n, int32_t v) {
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) p[i] = v;
+}
+
+// bf16 copy (mode 7 and the unused mode digits, FQ:1831-1833): 16-byte vectors and a scalar tail
+template <int EW_NV>
+__global__ __launch_bounds__(WG) void k_copy(const uint16_t* in, uint16_t* out, int64_t n, int64_t nvec) {
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    uint4* out4 = reinterpret_cast<uint4*>(out);
+    const int64_t base = (int64_t)blockIdx.x * (EW_NV * WG) + threadIdx.x;
+    uint4 v[EW_NV];
+#pragma unroll
+    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = in4[c]; }
+#pragma unroll
+    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) out4[c] = v[k]; }
+    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = in[i];
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_rowgroup: blocks of 1 x 8G elements; the tensor is a flat array of 16-byte chunks and a block is G
+// consecutive chunks held by G consecutive lanes.  A workgroup owns NV * 256 consecutive chunks and issues all of
+// its loads before it computes.  The main path is branch-free: the fast result is computed for every chunk and
+// replaced by the input for all-zero groups (FQ:802, 814) and for groups whose scale is outside the fast range; the
+// latter are redone by a second, non-unrolled exact loop.  GT > 0 fixes the group size at compile time; FULL means
+// nchunks is a multiple of NV * 256.
+template <int F, bool E8, int NV, int GT, bool FULL>
+__global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, int32_t* __restrict__ meta,
+                                                 int64_t nchunks, int G, int logG, int meta_val) {
+    if constexpr (GT > 0) { G = GT; }
+    const int64_t base = (int64_t)blockIdx.x * (NV * WG) + threadIdx.x;
+    uint4 v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        int64_t c = base + k * WG;
+        v[k] = make_uint4(0, 0, 0, 0);
+        if (FULL || c < nchunks) v[k] = in[c];
+    }
+    uint32_t slow = 0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        int64_t c = base + k * WG;
+        float amax = 0.0f;
+        acc_amax(amax, v[k].x); acc_amax(amax, v[k].y); acc_amax(amax, v[k].z); acc_amax(amax, v[k].w);
+        amax = group_max_t<GT>(amax, G);
+        Scale sc;
+        if constexpr (E8) sc = make_scale_e8<F>(amax);
+        else sc = make_scale(Fmt<F>::fmax / amax);
+        const bool quant = (amax > 0.0f) && sc.fast;
+        const uint4 q = fq_vec_fast<F, E8>(v[k], sc);
+        uint4 r;
+        r.x = quant ? q.x : v[k].x;
+        r.y = quant ? q.y : v[k].y;
+        r.z = quant ? q.z : v[k].z;
+        r.w = quant ? q.w : v[k].w;
+        if ((amax > 0.0f) && !sc.fast) slow |= 1u << k;
+        if (FULL || c < nchunks) {
+            out[c] = r;
+            if (meta_val >= 0 && (c & (G - 1)) == 0) meta[c >> logG] = meta_val;
+        }
+    }
+    if (slow) {
+#pragma unroll 1
+        for (int k = 0; k < NV; ++k) {
+            if (!((slow >> k) & 1u)) continue;
+            int64_t c = base + k * WG;
+            uint4 x = in[c];                    // when out == in this is the input again: it was stored back above
+            float amax = 0.0f;
+            acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
+            amax = group_max_t<GT>(amax, G);
+            const Scale sc = make_scale(Fmt<F>::fmax / amax);
+            uint4 r;
+            r.x = fq_pair_exact<F, E8, false>(x.x, sc);
+            r.y = fq_pair_exact<F, E8, false>(x.y, sc);
+            r.z = fq_pair_exact<F, E8, false>(x.z, sc);
+            r.w = fq_pair_exact<F, E8, false>(x.w, sc);
+            out[c] = r;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Per-block look-up tables in LDS for fp32 scales (E4M3 / E5M2, block in the fast range).
+// The descaled value of an element depends only on its 7-bit magnitude code, so q(code) = decode(code) / s is
+// computed once per block with the IEEE division and the per-element divisions of FQ:314 disappear.
+// Entries 0..127: E4M3 with s4 = 448 / amax; entries 128..255: E5M2 with s5 = 57344 / amax.
+__device__ __forceinline__ void build_luts(float* lut, int tid, float s4, float s5) {
+    if (tid < 128) lut[tid] = hw_unpack<FMT_E4M3, 0>((uint32_t)tid) / s4;
+    else lut[tid] = hw_unpack<FMT_E5M2, 0>((uint32_t)(tid - 128)) / s5;
+}
+
+// quantize one packed word through the table: |x| * s, hardware convert, table, round-half-up store, sign
+template <int F> __device__ __forceinline__ uint32_t fq_pair_lut(uint32_t w, float s, const float* lut) {
+    uint32_t p = hw_pack2<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s);
+    float q0 = lut[p & 0xFFu];
+    float q1 = lut[(p >> 8) & 0xFFu];
+    return store_pair<false>(q0, q1) | (w & 0x80008000u);
+}
+template <int F> __device__ __forceinline__ uint4 fq_vec_lut(uint4 v, float s, const float* lut) {
+    uint4 r;
+    r.x = fq_pair_lut<F>(v.x, s, lut);
+    r.y = fq_pair_lut<F>(v.y, s, lut);
+    r.z = fq_pair_lut<F>(v.z, s, lut);
+    r.w = fq_pair_lut<F>(v.w, s, lut);
+    return r;
+}
+
+// q / x for 0 < x, q >= 0, both far from the ends of the exponent range: reciprocal with one Newton step, one
+// quotient correction with an exact residual.  Equals the IEEE quotient except for rare last-place cases.
+__device__ __forceinline__ float refine_rcp(float x) {
+    float y = __builtin_amdgcn_rcpf(x);
+    return fmaf(fmaf(-x, y, 1.0f), y, y);
+}
+__device__ __forceinline__ float div_nr(float q, float x, float y) {
+    float r = q * y;
+    return fmaf(fmaf(-x, r, q), y, r);
+}
+
+// The two error terms of one packed word (FQ:504-542) on magnitudes; s5 = 128 * s4 exactly.
+template <bool E8>
+__device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, const float* lut, float& e4, float& e5) {
+    float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
+    float qa4, qb4, qa5, qb5;
+    if constexpr (E8) {
+        const int e84 = s4.e8, e85 = s4.e8 + 7;
+        uint32_t p4 = hw_pack2<FMT_E4M3>(ldexpf(a, e84), ldexpf(b, e84));
+        uint32_t p5 = hw_pack2<FMT_E5M2>(ldexpf(a, e85), ldexpf(b, e85));
+        qa4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p4)) - (e84 << 23), 0));
+        qb4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p4)) - (e84 << 23), 0));
+        qa5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 0>(p5)) - (e85 << 23), 0));
+        qb5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 1>(p5)) - (e85 << 23), 0));
+    } else {
+        float va = a * s4.s, vb = b * s4.s;
+        uint32_t p4 = hw_pack2<FMT_E4M3>(va, vb);
+        uint32_t p5 = hw_pack2<FMT_E5M2>(va * 128.0f, vb * 128.0f);
+        qa4 = lut[p4 & 0xFFu]; qb4 = lut[(p4 >> 8) & 0xFFu];
+        qa5 = lut[128u + (p5 & 0xFFu)]; qb5 = lut[128u + ((p5 >> 8) & 0xFFu)];
+    }
+    float ya = refine_rcp(a), yb = refine_rcp(b);
+    float ta4 = fabsf(div_nr(qa4, a, ya) - 1.0f), ta5 = fabsf(div_nr(qa5, a, ya) - 1.0f);
+    float tb4 = fabsf(div_nr(qb4, b, yb) - 1.0f), tb5 = fabsf(div_nr(qb5, b, yb) - 1.0f);
+    e4 += (a != 0.0f ? ta4 : 0.0f) + (b != 0.0f ? tb4 : 0.0f);
+    e5 += (a != 0.0f ? ta5 : 0.0f) + (b != 0.0f ? tb5 : 0.0f);
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_wgblock: one workgroup per quantization block, the block held in registers (NV 16-byte vectors per lane).
+// Chunk ch = k * 256 + tid of the block sits at block row ch / cpr, chunk column ch % cpr.
+// MOR: per-block format selection (FQ:610-682), else one forced format.  FULL: every block is complete and has
+// exactly NV * 256 chunks, so no predicates.  Blocks outside the fast range go through generic_block.
+template <bool MOR, bool E8, int NV, bool FULL>
+__global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
+                                                float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
+    constexpr bool LUT = !E8;
+    __shared__ float s_f[2][WAVES];
+    __shared__ uint32_t s_u[WAVES];
+    __shared__ float s_lut[LUT ? 256 : 1];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t bid = blockIdx.x;
+    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3);          // chunks per tensor row
+    const uint4* bin = in + (r0 * row_stride + (c0 >> 3));
+    uint4* bout = out ? out + (r0 * row_stride + (c0 >> 3)) : nullptr;
+    const int rows_valid = (int)min(sh.brows, sh.rows - r0);
+    const int cols_valid = (int)min((int64_t)cpr, (sh.cols - c0) >> 3);
+    const int nch = (int)sh.brows * cpr;
+
+    uint4 v[NV];
+    uint32_t off[NV];
+    bool ok[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        int ch = k * WG + tid;
+        int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
+        int cc = ch - r * cpr;
+        ok[k] = FULL || ((ch < nch) && (r < rows_valid) && (cc < cols_valid));
+        off[k] = (uint32_t)r * row_stride + (uint32_t)cc;
+        if (ok[k]) v[k] = bin[off[k]];
+    }
+
+    // pass 1 (registers): amax and min over non-zero magnitudes, FQ:407-485
+    float amax = 0.0f;
+    uint32_t amin_m1 = AMIN_INIT_M1;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+        if (ok[k]) {
+            acc_amax(amax, v[k].x); acc_amax(amax, v[k].y); acc_amax(amax, v[k].z); acc_amax(amax, v[k].w);
+            if constexpr (MOR) { acc_amin(amin_m1, v[k].x); acc_amin(amin_m1, v[k].y); acc_amin(amin_m1, v[k].z); acc_amin(amin_m1, v[k].w); }
+        }
+    amax = group_max(amax, 64);
+    if constexpr (MOR) amin_m1 = group_umin(amin_m1, 64);
+    if (lane == 0) { s_f[0][wave] = amax; s_u[wave] = amin_m1; }
+    __syncthreads();
+    amax = fmaxf(fmaxf(s_f[0][0], s_f[0][1]), fmaxf(s_f[0][2], s_f[0][3]));
+    amin_m1 = min(min(s_u[0], s_u[1]), min(s_u[2], s_u[3]));
+    const float amin = u2f(amin_m1 + 1u);
+
+    // scales of the two fp8 formats; the fp6 scales differ from s4 by 2^4 / 2^6, inside the margin of `fast`
+    const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
+    if (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90)) {           // uniform over the workgroup
+        generic_block<false>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
+                             sh, qa, E8, bid, s_f, s_u);
+        return;
+    }
+
+    int fmt = qa.fmt;
+    int meta_val = qa.meta_val;
+    float e4 = 0.0f, e5 = 0.0f;
+    bool lut_built = false;
+    if constexpr (MOR) {
+        int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
+        if (qt == Q_UNKNOWN) {
+            // pass 2 (registers): the two error sums, FQ:487-584.  amax > 0 here.
+            if constexpr (LUT) { build_luts(s_lut, tid, s4.s, s5.s); lut_built = true; }
+            __syncthreads();                     // tables written, s_f[0] read by every wave
+#pragma unroll
+            for (int k = 0; k < NV; ++k)
+                if (ok[k]) {
+                    err_pair_fast<E8>(v[k].x, s4, s_lut, e4, e5);
+                    err_pair_fast<E8>(v[k].y, s4, s_lut, e4, e5);
+                    err_pair_fast<E8>(v[k].z, s4, s_lut, e4, e5);
+                    err_pair_fast<E8>(v[k].w, s4, s_lut, e4, e5);
+                }
+            e4 = wave_sum(e4);
+            e5 = wave_sum(e5);
+            if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+            __syncthreads();
+            e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
+            e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+            if (!(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) {
+                // The sums above divide with a Newton step.  When they are too close for that to be trusted with
+                // the decision, repeat them with IEEE divisions (from memory, non-unrolled: this is rare).
+                const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in);
+                const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
+                e4 = 0.0f; e5 = 0.0f;
+#pragma unroll 1
+                for (int64_t i = tid; i < bh * bw; i += WG) {
+                    int64_t r = i / bw, c = i - r * bw;
+                    err_terms_exact<false>(bf16_one(in16[(r0 + r) * sh.cols + c0 + c]), E8, s4, s5, e4, e5);
+                }
+                e4 = wave_sum(e4);
+                e5 = wave_sum(e5);
+                __syncthreads();
+                if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+                __syncthreads();
+                e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
+                e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+            }
+            qt = mor_decide_error(amax, qa.clamp, e4, e5);
+        }
+        meta_val = qt;
+        fmt = mor_fmt_of(qt);
+    }
+    if (tid == 0) {
+        if (meta && meta_val >= 0) meta[bid] = meta_val;
+        if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+    }
+    if (!out) return;
+
+    // pass 3 (registers): quantize and store, FQ:733-851
+    if ((fmt < 0) || !(amax > 0.0f)) {
+        if (out != in) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = v[k];
+        }
+        return;
+    }
+    if constexpr (LUT) {
+        if (fmt == FMT_E4M3 || fmt == FMT_E5M2) {
+            if (!lut_built) { build_luts(s_lut, tid, s4.s, s5.s); __syncthreads(); }
+            if (fmt == FMT_E4M3) {
+#pragma unroll
+                for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_lut<FMT_E4M3>(v[k], s4.s, s_lut);
+            } else {
+#pragma unroll
+                for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_lut<FMT_E5M2>(v[k], s5.s, s_lut + 128);
+            }
+            return;
+        }
+    }
+    const Scale sc = make_scale(fmax_of(fmt) / amax);
+    switch (fmt) {
+        case FMT_E4M3:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_fast<FMT_E4M3, E8>(v[k], sc);
+            break;
+        case FMT_E5M2:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_fast<FMT_E5M2, E8>(v[k], sc);
+            break;
+        case FMT_E3M2:
+            if constexpr (!MOR) {
+#pragma unroll
+                for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_fast<FMT_E3M2, E8>(v[k], sc);
+            }
+            break;
+        default:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_fast<FMT_E2M3, E8>(v[k], sc);
+            break;
     }
 }
 
@@ -498,22 +664,44 @@ static int validate_shape(const void* input, int64_t rows, int64_t cols, int64_t
     return MOR_OK;
 }
 
-template <bool E8, bool EMU, bool HWCAST>
-static void launch_rowgroup(int fmt, const void* in, void* out, int32_t* meta, int64_t nchunks, int G, int meta_val, hipStream_t st) {
-    constexpr int U = 4;
-    int grid = grid_for(cdiv(nchunks, U), 16);
-    const uint4* i4 = static_cast<const uint4*>(in);
-    uint4* o4 = static_cast<uint4*>(out);
-    int lg = ilog2(G);
-    switch (fmt) {
-        case FMT_E4M3: k_rowgroup<FMT_E4M3, E8, EMU, HWCAST, U><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); break;
-        case FMT_E5M2: k_rowgroup<FMT_E5M2, E8, EMU, HWCAST, U><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); break;
-        case FMT_E3M2: k_rowgroup<FMT_E3M2, E8, EMU, HWCAST, U><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); break;
-        default:       k_rowgroup<FMT_E2M3, E8, EMU, HWCAST, U><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); break;
+template <int F, bool E8>
+static void launch_rowgroup_f(const uint4* i4, uint4* o4, int32_t* meta, int64_t nchunks, int G, int meta_val, hipStream_t st) {
+    // small tensors take fewer chunks per workgroup so that every CU still gets several workgroups
+    const int lg = ilog2(G);
+    if (nchunks >= 8ll * WG * 2048) {
+        constexpr int NV = 8;
+        const int grid = (int)cdiv(nchunks, (int64_t)NV * WG);
+        const bool full = nchunks % ((int64_t)NV * WG) == 0;
+        if (G == 4 && full) k_rowgroup<F, E8, NV, 4, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+        else if (G == 16 && full) k_rowgroup<F, E8, NV, 16, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+        else k_rowgroup<F, E8, NV, 0, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+    } else {
+        constexpr int NV = 2;
+        const int grid = (int)cdiv(nchunks, (int64_t)NV * WG);
+        k_rowgroup<F, E8, NV, 0, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
     }
 }
 
-template <bool E8, bool EMU, bool HWCAST>
+template <bool E8>
+static void launch_rowgroup(int fmt, const void* in, void* out, int32_t* meta, int64_t nchunks, int G, int meta_val, hipStream_t st) {
+    const uint4* i4 = static_cast<const uint4*>(in);
+    uint4* o4 = static_cast<uint4*>(out);
+    switch (fmt) {
+        case FMT_E4M3: launch_rowgroup_f<FMT_E4M3, E8>(i4, o4, meta, nchunks, G, meta_val, st); break;
+        case FMT_E5M2: launch_rowgroup_f<FMT_E5M2, E8>(i4, o4, meta, nchunks, G, meta_val, st); break;
+        case FMT_E3M2: launch_rowgroup_f<FMT_E3M2, E8>(i4, o4, meta, nchunks, G, meta_val, st); break;
+        default:       launch_rowgroup_f<FMT_E2M3, E8>(i4, o4, meta, nchunks, G, meta_val, st); break;
+    }
+}
+
+template <bool MOR, bool E8, int NV>
+static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, int32_t* meta, float* stats,
+                              const Shape& sh, const QuantArgs& qa, int cpr, int shift, hipStream_t st) {
+    if (full) k_wgblock<MOR, E8, NV, true><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    else k_wgblock<MOR, E8, NV, false><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+}
+
+template <bool MOR, bool E8>
 static void launch_wgblock(const void* in, void* out, int32_t* meta, float* stats, const Shape& sh, const QuantArgs& qa, hipStream_t st) {
     int cpr = (int)(sh.bcols / 8);
     int nch = (int)sh.brows * cpr;
@@ -522,31 +710,15 @@ static void launch_wgblock(const void* in, void* out, int32_t* meta, float* stat
     int grid = (int)(sh.gy * sh.gx);
     const uint4* i4 = static_cast<const uint4*>(in);
     uint4* o4 = static_cast<uint4*>(out);
-    if (nv <= 1)      k_wgblock<E8, EMU, HWCAST, 1><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
-    else if (nv <= 2) k_wgblock<E8, EMU, HWCAST, 2><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
-    else if (nv <= 4) k_wgblock<E8, EMU, HWCAST, 4><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
-    else              k_wgblock<E8, EMU, HWCAST, 8><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    int NVc = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
+    bool full = (sh.rows % sh.brows == 0) && (sh.cols % sh.bcols == 0) && (nch == NVc * WG);
+    switch (NVc) {
+        case 1: launch_wgblock_nv<MOR, E8, 1>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
+        case 2: launch_wgblock_nv<MOR, E8, 2>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
+        case 4: launch_wgblock_nv<MOR, E8, 4>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
+        default: launch_wgblock_nv<MOR, E8, 8>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
+    }
 }
-
-template <bool E8, bool EMU, bool HWCAST>
-static void launch_elementwise(const void* in, void* out, int32_t* meta, int64_t n, int64_t nmeta, int fmt, float scale, int meta_val, hipStream_t st) {
-    int64_t nvec = (aligned16(in) && aligned16(out)) ? n / 8 : 0;
-    int grid = grid_for(nvec > 0 ? nvec : n, 16);
-    k_elementwise<E8, EMU, HWCAST><<<grid, WG, 0, st>>>(static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), meta, n, nvec, nmeta, fmt, scale, meta_val);
-}
-
-#define DISPATCH3(FN, e8, emu, hw, ...)                                            \
-    do {                                                                           \
-        if (e8) {                                                                  \
-            if (emu) FN<true, true, false>(__VA_ARGS__);                           \
-            else if (hw) FN<true, false, true>(__VA_ARGS__);                       \
-            else FN<true, false, false>(__VA_ARGS__);                              \
-        } else {                                                                   \
-            if (emu) FN<false, true, false>(__VA_ARGS__);                          \
-            else if (hw) FN<false, false, true>(__VA_ARGS__);                      \
-            else FN<false, false, false>(__VA_ARGS__);                             \
-        }                                                                          \
-    } while (0)
 
 // Common driver of mor_fake_quantize / mor_block_format / mor_mor_stats.
 static int run_quantize(const void* input, void* output, int32_t* meta, float* stats,
@@ -554,25 +726,52 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
                         const QuantArgs& qa, bool e8, uint32_t flags, hipStream_t st) {
     Shape sh{rows, cols, brows, bcols, cdiv(rows, brows), cdiv(cols, bcols)};
     const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
-    const bool hw = !(flags & MOR_FLAG_SOFTWARE_CAST);
+    const bool fast_ok = !emu && !(flags & MOR_FLAG_SOFTWARE_CAST);
     const int64_t nblocks = sh.gy * sh.gx;
+    const uint16_t* in16 = static_cast<const uint16_t*>(input);
+    uint16_t* out16 = static_cast<uint16_t*>(output);
 
     if (qa.qmode == 4) {
-        DISPATCH3(launch_elementwise, e8, emu, hw, input, output, meta, rows * cols, nblocks, qa.fmt, qa.clamp, qa.meta_val, st);
+        const int64_t n = rows * cols;
+        uint32_t sbits;
+        memcpy(&sbits, &qa.clamp, 4);
+        const int e8v = (int)((sbits >> 23) & 0xFF) - 127;
+        if (fast_ok && e8v >= -100 && e8v <= 100) {
+            int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
+            if (nvec >= 8ll * WG * 2048) {
+                int grid = (int)cdiv(nvec, 8ll * WG);
+                if (e8) k_elementwise_fast<true, 8><<<grid, WG, 0, st>>>(in16, out16, meta, n, nvec, nblocks, qa.fmt, qa.clamp, qa.meta_val);
+                else k_elementwise_fast<false, 8><<<grid, WG, 0, st>>>(in16, out16, meta, n, nvec, nblocks, qa.fmt, qa.clamp, qa.meta_val);
+            } else {
+                int grid = nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16);
+                if (e8) k_elementwise_fast<true, 2><<<grid, WG, 0, st>>>(in16, out16, meta, n, nvec, nblocks, qa.fmt, qa.clamp, qa.meta_val);
+                else k_elementwise_fast<false, 2><<<grid, WG, 0, st>>>(in16, out16, meta, n, nvec, nblocks, qa.fmt, qa.clamp, qa.meta_val);
+            }
+        } else {
+            int grid = grid_for(n, 16);
+            if (emu) k_elementwise_exact<true><<<grid, WG, 0, st>>>(in16, out16, meta, n, nblocks, qa.fmt, e8, qa.clamp, qa.meta_val);
+            else k_elementwise_exact<false><<<grid, WG, 0, st>>>(in16, out16, meta, n, nblocks, qa.fmt, e8, qa.clamp, qa.meta_val);
+        }
         return check_launch("k_elementwise");
     }
-    const bool vec_ok = aligned16(input) && (!output || aligned16(output)) && cols % 8 == 0 && bcols % 8 == 0;
+    const bool vec_ok = fast_ok && aligned16(input) && (!output || aligned16(output)) && cols % 8 == 0 && bcols % 8 == 0
+                        && brows * (cols / 8) < 0x7FFFFFFFll;
     const int64_t G = bcols / 8;
     if (qa.qmode == 2 && !stats && output && vec_ok && brows == 1 && cols % bcols == 0 && is_pow2(G) && G <= 64) {
-        DISPATCH3(launch_rowgroup, e8, emu, hw, qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
+        if (e8) launch_rowgroup<true>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
+        else launch_rowgroup<false>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
         return check_launch("k_rowgroup");
     }
     if (vec_ok && brows * (bcols / 8) <= 8 * WG) {
-        DISPATCH3(launch_wgblock, e8, emu, hw, input, output, meta, stats, sh, qa, st);
+        if (qa.qmode == 1) {
+            if (e8) launch_wgblock<true, true>(input, output, meta, stats, sh, qa, st);
+            else launch_wgblock<true, false>(input, output, meta, stats, sh, qa, st);
+        } else {
+            if (e8) launch_wgblock<false, true>(input, output, meta, stats, sh, qa, st);
+            else launch_wgblock<false, false>(input, output, meta, stats, sh, qa, st);
+        }
         return check_launch("k_wgblock");
     }
-    const uint16_t* in16 = static_cast<const uint16_t*>(input);
-    uint16_t* out16 = static_cast<uint16_t*>(output);
     if (emu) k_generic<true><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, e8 ? 1 : 0);
     else k_generic<false><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, e8 ? 1 : 0);
     return check_launch("k_generic");
@@ -600,11 +799,13 @@ extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
             // FQ:1831-1833, 727-729, 843: bf16 copy, meta 3
             const int64_t nblocks = cdiv(rows, brows) * cdiv(cols, bcols);
             if (output != input) {
-                hipError_t e = hipMemcpyAsync(output, input, (size_t)rows * cols * 2, hipMemcpyDeviceToDevice, st);
-                if (e != hipSuccess) return fail(MOR_ERR_LAUNCH, "hipMemcpyAsync: %s", hipGetErrorString(e));
+                const int64_t n = rows * cols;
+                const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
+                if (nvec >= 8ll * WG * 2048) k_copy<8><<<(int)cdiv(nvec, 8ll * WG), WG, 0, st>>>(static_cast<const uint16_t*>(input), static_cast<uint16_t*>(output), n, nvec);
+                else k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(static_cast<const uint16_t*>(input), static_cast<uint16_t*>(output), n, nvec);
             }
             k_fill_i32<<<grid_for(nblocks), WG, 0, st>>>(meta, nblocks, 3);
-            return check_launch("k_fill_i32");
+            return check_launch("k_copy / k_fill_i32");
         }
     }
     return run_quantize(input, output, meta, nullptr, rows, cols, brows, bcols, qa, e8, flags, st);

@@ -414,7 +414,7 @@ int mor_oracle_fake_quantize(const uint16_t* in, uint16_t* out, int32_t* meta,
     int dynamic_range_mode = (mode / 100 > 0);
     int e8 = (sf_type == 2);
     int64_t gy = cdiv(rows, brows), gx = cdiv(cols, bcols);
-#pragma omp parallel for collapse(2) schedule(dynamic, 1)
+#pragma omp parallel for collapse(2) schedule(static)
     for (int64_t by = 0; by < gy; ++by)
         for (int64_t bx = 0; bx < gx; ++bx) {
             blk_t b = {in, rows, cols, brows, bcols, by * brows, 0, bx * bcols, 0};
