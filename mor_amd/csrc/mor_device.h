@@ -28,6 +28,26 @@ __host__ __device__ __forceinline__ float fmax_of(int fmt) {
     return fmt == FMT_E4M3 ? 448.0f : fmt == FMT_E5M2 ? 57344.0f : fmt == FMT_E3M2 ? 28.0f : 7.5f;
 }
 
+// ---------------------------------------------------------------- 16-byte global accesses
+// NT = streaming (non-temporal) access for tensors far larger than the last-level cache.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <bool NT> __device__ __forceinline__ uint4 load16(const uint4* p) {
+    if constexpr (NT) {
+        u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        return make_uint4(t.x, t.y, t.z, t.w);
+    } else {
+        return *p;
+    }
+}
+template <bool NT> __device__ __forceinline__ void store16(uint4* p, uint4 v) {
+    if constexpr (NT) {
+        u32x4 t = {v.x, v.y, v.z, v.w};
+        __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+    } else {
+        *p = v;
+    }
+}
+
 // ---------------------------------------------------------------- bf16 <-> fp32
 // FQ:38-44: a bf16 is the upper half of an fp32.
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }

@@ -16,6 +16,7 @@
 #include <stdio.h>
 #include <stdarg.h>
 #include <string.h>
+#include <algorithm>
 
 #include "mor_device.h"
 #include "../../include/mor_hip.h"
@@ -330,18 +331,11 @@ template <int F> __device__ __forceinline__ uint4 fq_vec_lut(uint4 v, float s, c
     return r;
 }
 
-// q / x for 0 < x, q >= 0, both far from the ends of the exponent range: reciprocal with one Newton step, one
-// quotient correction with an exact residual.  Equals the IEEE quotient except for rare last-place cases.
-__device__ __forceinline__ float refine_rcp(float x) {
-    float y = __builtin_amdgcn_rcpf(x);
-    return fmaf(fmaf(-x, y, 1.0f), y, y);
-}
-__device__ __forceinline__ float div_nr(float q, float x, float y) {
-    float r = q * y;
-    return fmaf(fmaf(-x, r, q), y, r);
-}
-
 // The two error terms of one packed word (FQ:504-542) on magnitudes; s5 = 128 * s4 exactly.
+// The reference computes |q / x - 1|; here |q - x| * (1 / x): q - x is exact in fp32 (q is within a factor 2 of
+// x, or 0), so each term carries one reciprocal's relative error (1e-7) instead of the absolute 6e-8 rounding of
+// a quotient near 1.  Both agree with the exact term far inside the 1e-6 tolerance on the sums; decisions that
+// would depend on less than 1e-5 are recomputed with the reference's divisions by the caller.
 template <bool E8>
 __device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, const float* lut, float& e4, float& e5) {
     float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
@@ -361,19 +355,21 @@ __device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, const
         qa4 = lut[p4 & 0xFFu]; qb4 = lut[(p4 >> 8) & 0xFFu];
         qa5 = lut[128u + (p5 & 0xFFu)]; qb5 = lut[128u + ((p5 >> 8) & 0xFFu)];
     }
-    float ya = refine_rcp(a), yb = refine_rcp(b);
-    float ta4 = fabsf(div_nr(qa4, a, ya) - 1.0f), ta5 = fabsf(div_nr(qa5, a, ya) - 1.0f);
-    float tb4 = fabsf(div_nr(qb4, b, yb) - 1.0f), tb5 = fabsf(div_nr(qb5, b, yb) - 1.0f);
-    e4 += (a != 0.0f ? ta4 : 0.0f) + (b != 0.0f ? tb4 : 0.0f);
-    e5 += (a != 0.0f ? ta5 : 0.0f) + (b != 0.0f ? tb5 : 0.0f);
+    float ya = (a != 0.0f) ? __builtin_amdgcn_rcpf(a) : 0.0f;
+    float yb = (b != 0.0f) ? __builtin_amdgcn_rcpf(b) : 0.0f;
+    e4 = fmaf(fabsf(qa4 - a), ya, e4);
+    e5 = fmaf(fabsf(qa5 - a), ya, e5);
+    e4 = fmaf(fabsf(qb4 - b), yb, e4);
+    e5 = fmaf(fabsf(qb5 - b), yb, e5);
 }
 
 // ------------------------------------------------------------------------------------------------
 // k_wgblock: one workgroup per quantization block, the block held in registers (NV 16-byte vectors per lane).
 // Chunk ch = k * 256 + tid of the block sits at block row ch / cpr, chunk column ch % cpr.
 // MOR: per-block format selection (FQ:610-682), else one forced format.  FULL: every block is complete and has
-// exactly NV * 256 chunks, so no predicates.  Blocks outside the fast range go through generic_block.
-template <bool MOR, bool E8, int NV, bool FULL>
+// exactly NV * 256 chunks, so no predicates.  NT: streaming loads and stores.  Blocks outside the fast range go
+// through generic_block.
+template <bool MOR, bool E8, int NV, bool FULL, bool NT>
 __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
     constexpr bool LUT = !E8;
@@ -401,7 +397,7 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
         int cc = ch - r * cpr;
         ok[k] = FULL || ((ch < nch) && (r < rows_valid) && (cc < cols_valid));
         off[k] = (uint32_t)r * row_stride + (uint32_t)cc;
-        if (ok[k]) v[k] = bin[off[k]];
+        if (ok[k]) v[k] = load16<NT>(bin + off[k]);
     }
 
     // pass 1 (registers): amax and min over non-zero magnitudes, FQ:407-485
@@ -487,7 +483,7 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
     if ((fmt < 0) || !(amax > 0.0f)) {
         if (out != in) {
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = v[k];
+            for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], v[k]);
         }
         return;
     }
@@ -496,10 +492,10 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
             if (!lut_built) { build_luts(s_lut, tid, s4.s, s5.s); __syncthreads(); }
             if (fmt == FMT_E4M3) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_lut<FMT_E4M3>(v[k], s4.s, s_lut);
+                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_lut<FMT_E4M3>(v[k], s4.s, s_lut));
             } else {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_lut<FMT_E5M2>(v[k], s5.s, s_lut + 128);
+                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_lut<FMT_E5M2>(v[k], s5.s, s_lut + 128));
             }
             return;
         }
@@ -508,21 +504,21 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
     switch (fmt) {
         case FMT_E4M3:
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_fast<FMT_E4M3, E8>(v[k], sc);
+            for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_fast<FMT_E4M3, E8>(v[k], sc));
             break;
         case FMT_E5M2:
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_fast<FMT_E5M2, E8>(v[k], sc);
+            for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_fast<FMT_E5M2, E8>(v[k], sc));
             break;
         case FMT_E3M2:
             if constexpr (!MOR) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_fast<FMT_E3M2, E8>(v[k], sc);
+                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_fast<FMT_E3M2, E8>(v[k], sc));
             }
             break;
         default:
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) bout[off[k]] = fq_vec_fast<FMT_E2M3, E8>(v[k], sc);
+            for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_fast<FMT_E2M3, E8>(v[k], sc));
             break;
     }
 }
@@ -697,8 +693,11 @@ static void launch_rowgroup(int fmt, const void* in, void* out, int32_t* meta, i
 template <bool MOR, bool E8, int NV>
 static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, int32_t* meta, float* stats,
                               const Shape& sh, const QuantArgs& qa, int cpr, int shift, hipStream_t st) {
-    if (full) k_wgblock<MOR, E8, NV, true><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
-    else k_wgblock<MOR, E8, NV, false><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    // tensors that cannot stay in the 256 MB last-level cache between the read and later uses are streamed
+    const bool nt = full && (sh.rows * sh.cols * 4 > (int64_t)512 << 20);
+    if (nt) k_wgblock<MOR, E8, NV, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    else if (full) k_wgblock<MOR, E8, NV, true, false><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    else k_wgblock<MOR, E8, NV, false, false><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
 }
 
 template <bool MOR, bool E8>
@@ -865,8 +864,523 @@ extern "C" int mor_selftest_hw_cast(uint64_t* mismatches, void* stream) {
     return check_launch("k_selftest_hw_cast");
 }
 
-// ---- temporary: filled in by the scaling ops ----
-extern "C" size_t mor_workspace_bytes(int, int64_t, int64_t, int64_t, int64_t) { return 0; }
-extern "C" int mor_block_scaling(const void*, void*, int32_t*, float*, int32_t*, float*, int64_t, int64_t, int64_t, int64_t,
-                                 double, int64_t, int, void*, size_t, uint32_t, void*) { return fail(MOR_ERR_INVALID_ARGUMENT, "not built"); }
-extern "C" int mor_e8mx(const void*, void*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, void*, size_t, uint32_t, void*) { return fail(MOR_ERR_INVALID_ARGUMENT, "not built"); }
+
+// ================================================================================================
+// Block / channel scaling (FQ:951-1241, 1459-1752, host FQ:2013-2230, 2431-2660) and e8mx (FQ:1243-1428).
+//
+// Workspace layout (32-bit words): [0] tensor amax bits, [1] non-zero count, [2] number of error partials,
+// [3] spare, [WS_PARTIALS .. +MAX_PARTIALS) per-workgroup error sums, then one float per block (amax, turned
+// into the block's scale in place).
+namespace mor {
+
+constexpr int WS_HEADER = 4;
+constexpr int MAX_PARTIALS = 8192;
+constexpr int WS_BLOCKS = WS_HEADER + MAX_PARTIALS;
+
+struct DivU32 {   // x / d for 32-bit x by multiply-shift (d >= 1)
+    uint32_t d, mul, shift;
+};
+static DivU32 make_div(uint32_t d) {
+    DivU32 r{d, 0, 0};
+    if (d <= 1) { r.mul = 0; r.shift = 0; return r; }
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;                       // ceil(log2 d)
+    r.mul = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    r.shift = l;
+    return r;
+}
+__device__ __forceinline__ uint32_t div_u32(uint32_t x, const DivU32& d) {
+    if (d.d <= 1) return x;
+    uint32_t t = __umulhi(x, d.mul);
+    return (t + ((x - t) >> 1)) >> (d.shift - 1);
+}
+
+__global__ void k_ws_init(uint32_t* ws, float* block_amax, int64_t nb, int zero_blocks) {
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    if (gtid < WS_HEADER) ws[gtid] = 0;
+    if (zero_blocks) for (int64_t i = gtid; i < nb; i += (int64_t)gridDim.x * WG) block_amax[i] = 0.0f;
+}
+
+__device__ __forceinline__ int nnz_word(uint32_t w) {
+    return ((w & 0x7FFFu) != 0) + ((w & 0x7FFF0000u) != 0);
+}
+
+// publish one workgroup's amax / nnz into the header (max and integer add are order independent)
+__device__ __forceinline__ void publish_global(uint32_t* ws, float amax, int nnz, float* s_f, int* s_i) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    amax = group_max(amax, 64);
+    nnz = wave_sum_i(nnz);
+    if (lane == 0) { s_f[wave] = amax; s_i[wave] = nnz; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float a = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        int n = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+        atomicMax(&ws[0], f2u(a));
+        if (n) atomicAdd(reinterpret_cast<int*>(&ws[1]), n);
+    }
+}
+
+// pass 1, blocks 1 x 8G as lane groups over the flat chunk array (FQ:1430-1457, 1611-1629)
+__global__ __launch_bounds__(WG) void k_bs_amax_rowgroup(const uint4* in, uint32_t* ws, float* block_amax,
+                                                         int64_t nchunks, int G, int logG) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    float gmax = 0.0f;
+    int nnz = 0;
+    for (int64_t c = (int64_t)blockIdx.x * WG + threadIdx.x; c < nchunks; c += (int64_t)gridDim.x * WG) {
+        uint4 v = in[c];
+        float amax = 0.0f;
+        acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
+        nnz += nnz_word(v.x) + nnz_word(v.y) + nnz_word(v.z) + nnz_word(v.w);
+        gmax = fmaxf(gmax, amax);
+        amax = group_max(amax, G);
+        if ((c & (G - 1)) == 0) block_amax[c >> logG] = amax;
+    }
+    publish_global(ws, gmax, nnz, s_f, s_i);
+}
+
+// pass 1, one workgroup per block of any shape (FQ:951-1015); vec: 16-byte loads (cols and bcols multiples of 8)
+__global__ __launch_bounds__(WG) void k_bs_amax_block(const uint16_t* in, uint32_t* ws, float* block_amax, Shape sh, int vec) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const int64_t bid = blockIdx.x;
+    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
+    float amax = 0.0f;
+    int nnz = 0;
+    if (vec) {
+        const uint4* in4 = reinterpret_cast<const uint4*>(in);
+        const int64_t row_stride = sh.cols >> 3, cpr = sh.bcols >> 3;
+        for (int64_t i = threadIdx.x; i < sh.brows * cpr; i += WG) {
+            int64_t r = i / cpr, cc = i - r * cpr;
+            uint4 v = in4[(r0 + r) * row_stride + (c0 >> 3) + cc];
+            acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
+            nnz += nnz_word(v.x) + nnz_word(v.y) + nnz_word(v.z) + nnz_word(v.w);
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < sh.brows * sh.bcols; i += WG) {
+            int64_t r = i / sh.bcols, c = i - r * sh.bcols;
+            uint32_t a = ((uint32_t)in[(r0 + r) * sh.cols + c0 + c] << 16) & 0x7FFFFFFFu;
+            amax = fmaxf(amax, u2f(a));
+            nnz += ((a & 0x7FFF0000u) != 0);
+        }
+    }
+    publish_global(ws, amax, nnz, s_f, s_i);       // also leaves the per-wave maxima in s_f
+    if (threadIdx.x == 0) block_amax[bid] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+}
+
+// pass 1, column blocks N x 1 (FQ:1538-1610): a thread owns 8 adjacent columns over a segment of rows and merges
+// into the (zero-initialised) per-block maxima with atomicMax on the bit patterns of non-negative floats.
+__global__ __launch_bounds__(WG) void k_bs_amax_col(const uint16_t* in, uint32_t* ws, float* block_amax, Shape sh,
+                                                    int rows_per_wg, int vec) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const int64_t by = blockIdx.z;                                   // block row
+    const int64_t r_begin = by * sh.brows + (int64_t)blockIdx.y * rows_per_wg;
+    const int64_t r_end = min(r_begin + rows_per_wg, (by + 1) * sh.brows);
+    const int64_t col0 = ((int64_t)blockIdx.x * WG + threadIdx.x) * 8;
+    float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int nnz = 0;
+    if (col0 < sh.cols) {
+        if (vec) {
+            const uint4* in4 = reinterpret_cast<const uint4*>(in);
+            for (int64_t r = r_begin; r < r_end; ++r) {
+                uint4 v = in4[(r * sh.cols + col0) >> 3];
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    m[2 * j] = fmaxf(m[2 * j], fabsf(bf16_lo(w[j])));
+                    m[2 * j + 1] = fmaxf(m[2 * j + 1], fabsf(bf16_hi(w[j])));
+                    nnz += nnz_word(w[j]);
+                }
+            }
+        } else {
+            const int ncol = (int)min((int64_t)8, sh.cols - col0);
+            for (int64_t r = r_begin; r < r_end; ++r)
+                for (int j = 0; j < ncol; ++j) {
+                    uint32_t a = ((uint32_t)in[r * sh.cols + col0 + j] << 16) & 0x7FFFFFFFu;
+                    m[j] = fmaxf(m[j], u2f(a));
+                    nnz += (a != 0);
+                }
+        }
+        const int ncol = (int)min((int64_t)8, sh.cols - col0);
+        for (int j = 0; j < ncol; ++j)
+            if (m[j] > 0.0f) atomicMax(reinterpret_cast<uint32_t*>(&block_amax[by * sh.cols + col0 + j]), f2u(m[j]));
+    }
+    float gmax = fmaxf(fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3])), fmaxf(fmaxf(m[4], m[5]), fmaxf(m[6], m[7])));
+    publish_global(ws, gmax, nnz, s_f, s_i);
+}
+
+// FQ:1059-1093
+__device__ __forceinline__ float scaling_factor(float global_amax, float block_amax, int ss_mode) {
+    float sf = 1.0f;
+    const float fmax = 448.0f;
+    if (block_amax < 1e-35f) block_amax = 1e-35f;
+    switch (ss_mode) {
+        case 1: {
+            float ratio = fmax / global_amax;
+            uint32_t gman = f2u(ratio) & 0x007FFFFFu;
+            float bsf = fmax / block_amax;
+            uint32_t bb = f2u(bsf);
+            float adj = u2f((bb & 0xFF800000u) | gman);
+            sf = (gman <= (bb & 0x007FFFFFu)) ? adj : adj / 2.0f;
+            break;
+        }
+        case 2:
+        case 3: sf = fmax / block_amax; break;
+        case 4: if (global_amax > 0.0f) sf = fmax / global_amax; break;
+        default: break;
+    }
+    return sf;
+}
+
+// pass 1.5: block amax -> block scale, in place
+__global__ __launch_bounds__(WG) void k_bs_scales(const uint32_t* ws, float* block_amax, int64_t nb, int ss_mode) {
+    const float gamax = u2f(ws[0]);
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < nb; i += (int64_t)gridDim.x * WG)
+        block_amax[i] = scaling_factor(gamax, block_amax[i], ss_mode);
+}
+
+// One element of FQ:1133-1162: zeros give +0 and no error; others E4M3 through the hardware-cast model.
+// The power-of-two path is taken for ss_mode 2 (the reference tests the strategy against SF_E8 = 2, FQ:1138).
+template <bool E8, bool EMU>
+__device__ __forceinline__ float bs_element(float x, const Scale& sc, float& err) {
+    if (x == 0.0f) return EMU ? x : 0.0f;
+    float dq = sqdd_exact<FMT_E4M3, E8, EMU>(x, sc);
+    err += fabsf((dq - x) / x);
+    return dq;
+}
+// Fast version on magnitudes for scales in the fast range: hardware convert; q = c / s by a reciprocal-multiply
+// with one exact-residual correction (r = 1 / s correctly rounded, the result is then the rounded quotient);
+// error term |q - x| / x through the hardware reciprocal (relative 1e-7, tolerance on the sum 1e-6).
+template <bool E8>
+__device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, float rs, float& err) {
+    float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
+    float qa, qb;
+    if constexpr (E8) {
+        const int e8s = sc.e8 << 23;
+        uint32_t p = hw_pack2<FMT_E4M3>(ldexpf(a, sc.e8), ldexpf(b, sc.e8));
+        qa = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p)) - e8s, 0));
+        qb = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p)) - e8s, 0));
+    } else {
+        uint32_t p = hw_pack2<FMT_E4M3>(a * sc.s, b * sc.s);
+        float ca = hw_unpack<FMT_E4M3, 0>(p), cb = hw_unpack<FMT_E4M3, 1>(p);
+        float ta = ca * rs, tb = cb * rs;
+        qa = fmaf(fmaf(-ta, sc.s, ca), rs, ta);
+        qb = fmaf(fmaf(-tb, sc.s, cb), rs, tb);
+    }
+    const bool za = (a == 0.0f), zb = (b == 0.0f);
+    float ya = za ? 0.0f : __builtin_amdgcn_rcpf(a);
+    float yb = zb ? 0.0f : __builtin_amdgcn_rcpf(b);
+    err = fmaf(fabsf(qa - a), ya, err);
+    err = fmaf(fabsf(qb - b), yb, err);
+    // zero inputs come back as +0 (FQ:1133-1134); everything else keeps the input's sign
+    uint32_t lo = za ? 0u : ((rhu_bits(qa) >> 16) | (w & 0x8000u));
+    uint32_t hi = zb ? 0u : ((rhu_bits(qb) & 0xFFFF0000u) | (w & 0x80000000u));
+    return lo | hi;
+}
+
+// pass 2 / pass 4: quantize every element with its block's scale (looked up per chunk, or per column in column
+// mode), accumulate the relative error, optionally write.  GATE > 0: run only if meta[0] == GATE.
+template <bool E8, bool EMU, bool COL, bool WRITE, bool ERR>
+__global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* out, uint32_t* ws, const float* scales,
+                                                 const int32_t* meta, int gate, Shape sh, int vec, DivU32 d_rowchunks,
+                                                 DivU32 d_brows, DivU32 d_bchunks, DivU32 d_bcols) {
+    __shared__ float s_f[WAVES];
+    if (gate > 0 && meta[0] != gate) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float err = 0.0f;
+    if (vec) {
+        const uint32_t row_chunks = (uint32_t)(sh.cols >> 3);
+        const uint32_t nchunks = (uint32_t)sh.rows * row_chunks;
+        const uint4* in4 = reinterpret_cast<const uint4*>(in);
+        uint4* out4 = reinterpret_cast<uint4*>(out);
+        for (uint32_t c = blockIdx.x * WG + threadIdx.x; c < nchunks; c += gridDim.x * WG) {
+            const uint32_t row = div_u32(c, d_rowchunks), cc = c - row * row_chunks;
+            const uint32_t by = div_u32(row, d_brows);
+            uint4 v = in4[c];
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            if constexpr (COL) {
+                const float* sp = scales + (int64_t)by * sh.cols + (int64_t)cc * 8;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const Scale s0 = make_scale(sp[2 * j]), s1 = make_scale(sp[2 * j + 1]);
+                    float q0 = bs_element<E8, EMU>(bf16_lo(w[j]), s0, err);
+                    float q1 = bs_element<E8, EMU>(bf16_hi(w[j]), s1, err);
+                    w[j] = store_pair<EMU>(q0, q1);
+                }
+            } else {
+                const uint32_t bx = div_u32(cc, d_bchunks);
+                const Scale sc = make_scale(scales[(int64_t)by * sh.gx + bx]);
+                if (!EMU && sc.fast) {
+                    const float rs = 1.0f / sc.s;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) w[j] = bs_pair_fast<E8>(w[j], sc, rs, err);
+                } else {
+#pragma unroll 1
+                    for (int j = 0; j < 4; ++j) {
+                        float q0 = bs_element<E8, EMU>(bf16_lo(w[j]), sc, err);
+                        float q1 = bs_element<E8, EMU>(bf16_hi(w[j]), sc, err);
+                        w[j] = store_pair<EMU>(q0, q1);
+                    }
+                }
+            }
+            if constexpr (WRITE) out4[c] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    } else {
+        const int64_t n = sh.rows * sh.cols;
+        for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) {
+            const int64_t row = i / sh.cols, col = i - row * sh.cols;
+            const int64_t by = row / sh.brows, bx = col / sh.bcols;
+            const Scale sc = make_scale(scales[by * sh.gx + bx]);
+            float q = bs_element<E8, EMU>(bf16_one(in[i]), sc, err);
+            if constexpr (WRITE) out[i] = store_bf16<EMU>(q);
+        }
+    }
+    if constexpr (ERR) {
+        err = wave_sum(err);
+        if (lane == 0) s_f[wave] = err;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            reinterpret_cast<float*>(ws)[WS_HEADER + blockIdx.x] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+            if (blockIdx.x == 0) ws[2] = gridDim.x;
+        }
+    }
+}
+
+// pass 3 (FQ:1178-1241): total error (fixed summation order), the bf16 decision, the scalar outputs
+__global__ __launch_bounds__(WG) void k_bs_finalize(const uint32_t* ws, int npartials, float threshold, int32_t* meta,
+                                                    float* gamax_o, int32_t* gnnz_o, float* gerr_o) {
+    __shared__ float s_f[WAVES];
+    const float* part = reinterpret_cast<const float*>(ws) + WS_HEADER;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float acc = 0.0f;
+    for (int i = threadIdx.x; i < npartials; i += WG) acc += part[i];
+    acc = wave_sum(acc);
+    if (lane == 0) s_f[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float gerr = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+        const int gnnz = (int)ws[1];
+        const float avg = gerr / (float)gnnz;        // 0 / 0 = NaN on an all-zero tensor: not above the threshold
+        meta[0] = (avg > threshold) ? 3 : 1;
+        gamax_o[0] = u2f(ws[0]);
+        gnnz_o[0] = gnnz;
+        gerr_o[0] = gerr;
+    }
+}
+
+// pass 4 for the out-of-place ops (FQ:1217-1235): copy the input over the quantized output when meta[0] == 3
+__global__ __launch_bounds__(WG) void k_copy_if(const uint16_t* in, uint16_t* out, const int32_t* meta, int gate, int64_t n, int64_t nvec) {
+    if (meta[0] != gate) return;
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    uint4* out4 = reinterpret_cast<uint4*>(out);
+    for (int64_t c = gtid; c < nvec; c += stride) out4[c] = in4[c];
+    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = in[i];
+}
+
+// global amax only (e8mx, FQ:2292-2293)
+__global__ __launch_bounds__(WG) void k_global_amax(const uint16_t* in, uint32_t* ws, int64_t n, int64_t nvec) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    float amax = 0.0f;
+    for (int64_t c = gtid; c < nvec; c += stride) {
+        uint4 v = in4[c];
+        acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
+    }
+    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) amax = fmaxf(amax, fabsf(bf16_one(in[i])));
+    publish_global(ws, amax, 0, s_f, s_i);
+}
+
+// FQ:1243-1327: keep MB mantissa bits by comparing the 23-bit mantissa with the reference's threshold tables
+// (on bf16 inputs they are the midpoints with ties to even; on scaled inputs, whose low 16 bits are not zero,
+// they are what they are).  Exponent 0 loses its mantissa, exponent 255 is left alone, a carry out of exponent
+// 254 saturates.
+template <int MB> __device__ __forceinline__ float quant_e8m(float v) {
+    uint32_t b = f2u(v);
+    uint32_t sign = b & 0x80000000u;
+    uint32_t e = (b >> 23) & 0xFF, m = b & 0x7FFFFFu;
+    if (e == 0) m = 0;
+    else if (e != 255) {
+        // threshold j: even j -> midpoint (j << (7-MB)) + half, odd j -> next midpoint - 1, in units of 2^16
+        uint32_t k = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < (1u << MB); ++j) {
+            const uint32_t half = 1u << (6 - MB);
+            const uint32_t t = (j & 1u) ? (((j + 1u) << (7 - MB)) - half - 1u) : ((j << (7 - MB)) + half);
+            k += (m > (t << 16)) ? 1u : 0u;
+        }
+        if (k == (1u << MB)) {
+            m = 0; e++;
+            if (e == 255) { e = 254; m = ((1u << MB) - 1u) << (23 - MB); }
+        } else m = k << (23 - MB);
+    }
+    return u2f(sign | (e << 23) | m);
+}
+
+// FQ:1335-1359
+template <int MB> __device__ __forceinline__ float e8mx_scale(float gamax, int strategy) {
+    if (strategy != 1) return 1.0f;
+    uint32_t y = f2u(gamax);
+    uint32_t e = (y >> 23) + 1;
+    float fp_max = u2f((e << 23) | (((1u << MB) - 1u) << (23 - MB)));
+    float sf = fp_max / gamax;
+    if (sf >= 2.0f) sf /= 2.0f;
+    return sf;
+}
+
+template <int MB, bool EMU> __device__ __forceinline__ float e8mx_element(float x, float sf) {
+    float v = x * sf;
+    float dq = 0.0f;
+    if (v != 0.0f) dq = quant_e8m<MB>(v);
+    return dq / sf;
+}
+
+// FQ:1361-1428
+template <int MB, bool EMU>
+__global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, const uint32_t* ws, int strategy, int64_t n, int64_t nvec) {
+    const float sf = e8mx_scale<MB>(u2f(ws[0]), strategy);
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    uint4* out4 = reinterpret_cast<uint4*>(out);
+    for (int64_t c = gtid; c < nvec; c += stride) {
+        uint4 v = in4[c];
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            w[j] = store_pair<EMU>(e8mx_element<MB, EMU>(bf16_lo(w[j]), sf), e8mx_element<MB, EMU>(bf16_hi(w[j]), sf));
+        out4[c] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = store_bf16<EMU>(e8mx_element<MB, EMU>(bf16_one(in[i]), sf));
+}
+
+}  // namespace mor
+
+extern "C" size_t mor_workspace_bytes(int op, int64_t rows, int64_t cols, int64_t brows, int64_t bcols) {
+    if (rows <= 0 || cols <= 0 || brows <= 0 || bcols <= 0) return 0;
+    switch (op) {
+        case MOR_OP_BLOCK_SCALING:
+        case MOR_OP_CHANNEL_SCALING:
+            return (size_t)(WS_BLOCKS + cdiv(rows, brows) * cdiv(cols, bcols)) * 4;
+        case MOR_OP_E8MX:
+            return (size_t)WS_HEADER * 4;
+        default:
+            return 0;
+    }
+}
+
+template <bool E8, bool EMU, bool COL>
+static void launch_bs_quant(bool write, bool err, int grid, hipStream_t st, const uint16_t* in, uint16_t* out, uint32_t* ws,
+                            const float* scales, const int32_t* meta, int gate, const Shape& sh, int vec,
+                            DivU32 d0, DivU32 d1, DivU32 d2, DivU32 d3) {
+    if (write && err) k_bs_quant<E8, EMU, COL, true, true><<<grid, WG, 0, st>>>(in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3);
+    else if (write) k_bs_quant<E8, EMU, COL, true, false><<<grid, WG, 0, st>>>(in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3);
+    else k_bs_quant<E8, EMU, COL, false, true><<<grid, WG, 0, st>>>(in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3);
+}
+
+static void dispatch_bs_quant(bool e8, bool emu, bool col, bool write, bool err, int grid, hipStream_t st, const uint16_t* in,
+                              uint16_t* out, uint32_t* ws, const float* scales, const int32_t* meta, int gate, const Shape& sh,
+                              int vec, DivU32 d0, DivU32 d1, DivU32 d2, DivU32 d3) {
+#define BSQ(E8, EMU, COL) launch_bs_quant<E8, EMU, COL>(write, err, grid, st, in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3)
+    if (e8) {
+        if (emu) { if (col) BSQ(true, true, true); else BSQ(true, true, false); }
+        else { if (col) BSQ(true, false, true); else BSQ(true, false, false); }
+    } else {
+        if (emu) { if (col) BSQ(false, true, true); else BSQ(false, true, false); }
+        else { if (col) BSQ(false, false, true); else BSQ(false, false, false); }
+    }
+#undef BSQ
+}
+
+extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
+                                 float* global_amax, int32_t* global_non_zero, float* global_error,
+                                 int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                                 double e4m3_threshold, int64_t ss_mode, int channel,
+                                 void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+    if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
+    if (!output || !meta || !global_amax || !global_non_zero || !global_error) return fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
+    if (rows % brows != 0 || cols % bcols != 0)      // FQ:2019-2020, 2437-2438
+        return fail(MOR_ERR_INVALID_ARGUMENT, "block dims %lld x %lld do not divide the tensor %lld x %lld", (long long)brows, (long long)bcols, (long long)rows, (long long)cols);
+    if (ss_mode < 1 || ss_mode > 4) return fail(MOR_ERR_INVALID_ARGUMENT, "ss_mode must be 1..4 (got %lld)", (long long)ss_mode);
+    if (channel && brows != 1 && bcols != 1)         // FQ:2501
+        return fail(MOR_ERR_INVALID_ARGUMENT, "channel scaling needs block_rows == 1 or block_cols == 1");
+    if (rows * cols >= (1ll << 34)) return fail(MOR_ERR_INVALID_ARGUMENT, "tensor too large");
+    const size_t need = mor_workspace_bytes(MOR_OP_BLOCK_SCALING, rows, cols, brows, bcols);
+    if (!workspace || workspace_bytes < need) return fail(MOR_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
+    Shape sh{rows, cols, brows, bcols, rows / brows, cols / bcols};
+    const int64_t nb = sh.gy * sh.gx;
+    uint32_t* ws = static_cast<uint32_t*>(workspace);
+    float* blocks = reinterpret_cast<float*>(ws + WS_BLOCKS);
+    const uint16_t* in16 = static_cast<const uint16_t*>(input);
+    uint16_t* out16 = static_cast<uint16_t*>(output);
+    const bool inplace = (input == output);
+    const int vec = (aligned16(input) && aligned16(output) && cols % 8 == 0) ? 1 : 0;
+    const bool col = (bcols == 1 && brows > 1);
+
+    // pass 1: per-block amax, tensor amax, non-zero count
+    k_ws_init<<<col ? grid_for(nb) : 1, WG, 0, st>>>(ws, blocks, nb, col ? 1 : 0);
+    const int64_t G = bcols / 8;
+    if (col) {
+        const int rows_per_wg = (int)std::min<int64_t>(brows, 128);
+        dim3 grid((unsigned)cdiv(cdiv(cols, 8), WG), (unsigned)cdiv(brows, rows_per_wg), (unsigned)sh.gy);
+        k_bs_amax_col<<<grid, WG, 0, st>>>(in16, ws, blocks, sh, rows_per_wg, vec);
+    } else if (vec && brows == 1 && bcols % 8 == 0 && is_pow2(G) && G <= 64) {
+        k_bs_amax_rowgroup<<<grid_for(rows * cols / 8, 16), WG, 0, st>>>(static_cast<const uint4*>(input), ws, blocks, rows * cols / 8, (int)G, ilog2(G));
+    } else {
+        k_bs_amax_block<<<(int)nb, WG, 0, st>>>(in16, ws, blocks, sh, (vec && bcols % 8 == 0) ? 1 : 0);
+    }
+    // pass 1.5: scales
+    k_bs_scales<<<grid_for(nb), WG, 0, st>>>(ws, blocks, nb, (int)ss_mode);
+    // pass 2: quantize (out of place: write now; in place: error only), error partials
+    const bool vec2 = vec && (col || bcols % 8 == 0);
+    const int64_t work = vec2 ? rows * cols / 8 : rows * cols;
+    const int grid2 = (int)std::min<int64_t>(std::max<int64_t>(cdiv(work, WG), 1), MAX_PARTIALS);
+    DivU32 d0 = make_div((uint32_t)std::max<int64_t>(cols / 8, 1)), d1 = make_div((uint32_t)brows),
+           d2 = make_div((uint32_t)std::max<int64_t>(bcols / 8, 1)), d3 = make_div((uint32_t)bcols);
+    const bool e8 = (ss_mode == 2);
+    dispatch_bs_quant(e8, emu, col, !inplace, true, grid2, st, in16, out16, ws, blocks, meta, 0, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
+    // pass 3: decision and scalars
+    k_bs_finalize<<<1, WG, 0, st>>>(ws, grid2, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+    // pass 4: bf16 fallback (out of place: copy if meta == 3) or the quantized write (in place: only if meta == 1)
+    if (inplace) {
+        dispatch_bs_quant(e8, emu, col, true, false, grid2, st, in16, out16, ws, blocks, meta, 1, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
+    } else {
+        const int64_t n = rows * cols, nvec = vec ? n / 8 : 0;
+        k_copy_if<<<grid_for(nvec > 0 ? nvec : n, 16), WG, 0, st>>>(in16, out16, meta, 3, n, nvec);
+    }
+    return check_launch("mor_block_scaling");
+}
+
+extern "C" int mor_e8mx(const void* input, void* output, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                        int64_t quantize_type, int64_t scaling_strategy, void* workspace, size_t workspace_bytes,
+                        uint32_t flags, void* stream) {
+    if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
+    if (!output) return fail(MOR_ERR_INVALID_ARGUMENT, "output is NULL");
+    if (quantize_type < 1 || quantize_type > 3) return fail(MOR_ERR_INVALID_ARGUMENT, "quantize_type must be 1..3 (got %lld)", (long long)quantize_type);
+    const size_t need = mor_workspace_bytes(MOR_OP_E8MX, rows, cols, brows, bcols);
+    if (!workspace || workspace_bytes < need) return fail(MOR_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
+    uint32_t* ws = static_cast<uint32_t*>(workspace);
+    const uint16_t* in16 = static_cast<const uint16_t*>(input);
+    uint16_t* out16 = static_cast<uint16_t*>(output);
+    const int64_t n = rows * cols;
+    const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
+    const int grid = grid_for(nvec > 0 ? nvec : n, 16);
+    const int strategy = (int)scaling_strategy;
+    k_ws_init<<<1, WG, 0, st>>>(ws, nullptr, 0, 0);
+    if (strategy == 1) k_global_amax<<<grid, WG, 0, st>>>(in16, ws, n, nvec);
+#define E8MX(MB) do { if (emu) k_e8mx<MB, true><<<grid, WG, 0, st>>>(in16, out16, ws, strategy, n, nvec); \
+                      else k_e8mx<MB, false><<<grid, WG, 0, st>>>(in16, out16, ws, strategy, n, nvec); } while (0)
+    if (quantize_type == 1) E8MX(1); else if (quantize_type == 2) E8MX(2); else E8MX(3);
+#undef E8MX
+    return check_launch("mor_e8mx");
+}

@@ -71,3 +71,54 @@ def block_stats(a_u16, block_x, block_y, fmax):
     _cabi.check(L.mor_block_stats(x.data_ptr(), rows, cols, block_x, block_y, float(fmax), amax.data_ptr(), scale.data_ptr(), e8.data_ptr(), stream_ptr()))
     torch.cuda.synchronize()
     return amax.cpu().numpy(), scale.cpu().numpy(), e8.cpu().numpy()
+
+
+def block_scaling(a_u16, block_x, block_y, threshold, ss_mode, channel=False, flags=0, inplace=False):
+    """-> (out bits, meta, global_amax, global_non_zero, global_error) through mor_block_scaling"""
+    L = _cabi.lib()
+    rows, cols = a_u16.shape
+    x = to_dev_u16(a_u16)
+    out = x if inplace else torch.full_like(x, 7.0)
+    meta = torch.full((1,), -7, dtype=torch.int32, device=dev())
+    gamax = torch.zeros(1, dtype=torch.float32, device=dev())
+    gnnz = torch.zeros(1, dtype=torch.int32, device=dev())
+    gerr = torch.zeros(1, dtype=torch.float32, device=dev())
+    op = _cabi.OP_CHANNEL_SCALING if channel else _cabi.OP_BLOCK_SCALING
+    nbytes = L.mor_workspace_bytes(op, rows, cols, block_x, block_y)
+    ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev())
+    _cabi.check(L.mor_block_scaling(x.data_ptr(), out.data_ptr(), meta.data_ptr(), gamax.data_ptr(), gnnz.data_ptr(),
+                                    gerr.data_ptr(), rows, cols, block_x, block_y, float(threshold), ss_mode,
+                                    int(channel), ws.data_ptr(), nbytes, flags, stream_ptr()))
+    torch.cuda.synchronize()
+    return to_host_u16(out), meta.cpu().numpy(), gamax.cpu().numpy(), gnnz.cpu().numpy(), gerr.cpu().numpy()
+
+
+def e8mx(a_u16, block_x, block_y, quantize_type, scaling_strategy, flags=0, inplace=False):
+    L = _cabi.lib()
+    rows, cols = a_u16.shape
+    x = to_dev_u16(a_u16)
+    out = x if inplace else torch.empty_like(x)
+    nbytes = L.mor_workspace_bytes(_cabi.OP_E8MX, rows, cols, block_x, block_y)
+    ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev())
+    _cabi.check(L.mor_e8mx(x.data_ptr(), out.data_ptr(), rows, cols, block_x, block_y, quantize_type, scaling_strategy,
+                           ws.data_ptr(), nbytes, flags, stream_ptr()))
+    torch.cuda.synchronize()
+    return to_host_u16(out)
+
+
+def quant_dequant(x_f32, fmt):
+    L = _cabi.lib()
+    x = torch.from_numpy(np.ascontiguousarray(x_f32, dtype=np.float32)).to(dev())
+    out = torch.empty_like(x)
+    _cabi.check(L.mor_quant_dequant(x.data_ptr(), out.data_ptr(), x.numel(), fmt, stream_ptr()))
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def e4m3_with_e8_scale(x_f32, rne):
+    L = _cabi.lib()
+    x = torch.from_numpy(np.ascontiguousarray(x_f32, dtype=np.float32)).to(dev())
+    out = torch.empty_like(x)
+    _cabi.check(L.mor_e4m3_with_e8_scale(x.data_ptr(), out.data_ptr(), x.numel(), int(rne), stream_ptr()))
+    torch.cuda.synchronize()
+    return out.cpu().numpy()

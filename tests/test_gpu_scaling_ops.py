@@ -1,0 +1,137 @@
+"""GPU parity of mor_block_scaling (block and channel), mor_e8mx and the fp32 test ops against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mor_oracle as O
+import data_gen
+import torch_emulation as E
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    assert torch.cuda.is_available()
+    return gpu_util
+
+
+def uniform_bits(seed, rows, cols, lo, hi):
+    g = torch.Generator().manual_seed(seed)
+    return E.bf16_to_bits(torch.empty(rows, cols).uniform_(lo, hi, generator=g).to(torch.bfloat16))
+
+
+def check_scaling(G, a, br, bc, thr, ss, channel, flags=0, inplace=False):
+    print("scaling", a.shape, br, bc, thr, ss, channel, flags, inplace, flush=True)
+    out, meta, gamax, gnnz, gerr = G.block_scaling(a, br, bc, thr, ss, channel=channel, flags=flags, inplace=inplace)
+    want, wmeta, wamax, wnnz, werr = O.block_scaling(a, br, bc, thr, ss, channel=channel, flavour=O.EMU if flags & 1 else O.KERNEL)
+    assert gamax[0] == wamax[0] and gnnz[0] == wnnz[0]
+    np.testing.assert_allclose(gerr[0], werr[0], rtol=1e-6, atol=0)       # error sums: 1e-6 relative
+    avg = werr[0] / max(wnnz[0], 1)
+    if abs(avg - thr) > 1e-5 * thr:                                        # decision not within the tolerance of the sum
+        assert meta[0] == wmeta[0]
+    if meta[0] == wmeta[0]:
+        bad = np.argwhere(out != want)
+        assert len(bad) == 0, f"{len(bad)} differ, first {bad[0]} got {out[tuple(bad[0])]:#06x} want {want[tuple(bad[0])]:#06x}"
+    return meta[0]
+
+
+@pytest.mark.parametrize("ss", [1, 2, 3, 4])
+@pytest.mark.parametrize("shape", [(256, 256, 128, 128, False), (256, 256, 1, 256, True), (256, 256, 256, 1, True),
+                                   (64, 512, 1, 32, True), (96, 80, 32, 16, False), (60, 36, 20, 12, False),
+                                   (512, 40, 128, 1, True)])
+def test_scaling_fixture_and_random(G, ss, shape):
+    rows, cols, br, bc, channel = shape
+    if rows == 256 and cols == 256:
+        a = E.fixture_words(256, 256)
+        assert check_scaling(G, a, br, bc, 0.045, ss, channel) == 1
+        a = E.fixture_words(256, 256, [(0, 70, 21000, 53768)])
+        check_scaling(G, a, br, bc, 0.045, ss, channel)
+    a = uniform_bits(rows + ss, rows, cols, -448.0, 448.0)
+    a[1, :8] = 0
+    a[3, 5] = 0x8000
+    check_scaling(G, a, br, bc, 0.045, ss, channel)
+    check_scaling(G, a, br, bc, 0.02, ss, channel)       # low threshold: bf16 fallback copies the input
+    b = data_gen.c3_weights(rows, cols, seed=rows * 3 + ss)
+    check_scaling(G, b, br, bc, 0.045, ss, channel)
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 128, 128, False), (128, 512, 1, 512, True), (256, 64, 256, 1, True)])
+@pytest.mark.parametrize("thr", [0.045, 0.001])
+def test_scaling_inplace_and_flavour(G, shape, thr):
+    rows, cols, br, bc, channel = shape
+    a = uniform_bits(9, rows, cols, -53768.0, 53768.0)
+    for ss in (1, 3):
+        check_scaling(G, a, br, bc, thr, ss, channel, inplace=True)
+        check_scaling(G, a, br, bc, thr, ss, channel, flags=1)
+
+
+def test_scaling_reference_bf16_fallback_known_answer(G):
+    """test_fake_quantize_block_scaling.py:138-175: the 1.46e11 outlier gives meta 3 and output == input."""
+    a = E.fixture_words(256, 256, [(0, 70, 21000, 53768)])
+    out, meta, gamax, gnnz, gerr = G.block_scaling(a, 128, 128, 0.045, 1)
+    assert meta[0] == 3 and np.array_equal(out, a)
+    t = E.bits_to_bf16(a)
+    assert gamax[0] == t.float().abs().max().item() and gnnz[0] == int(torch.count_nonzero(t))
+
+
+def test_scaling_all_zero_tensor_does_not_trap(G):
+    z = np.zeros((128, 128), np.uint16)
+    out, meta, gamax, gnnz, gerr = G.block_scaling(z, 64, 64, 0.045, 1)
+    assert meta[0] == 1 and gamax[0] == 0 and gnnz[0] == 0 and np.array_equal(out, z)
+
+
+def test_scaling_rejects_bad_arguments(G):
+    a = np.zeros((100, 256), np.uint16)
+    with pytest.raises(RuntimeError):
+        G.block_scaling(a, 128, 128, 0.045, 1)
+    with pytest.raises(RuntimeError):
+        G.block_scaling(np.zeros((128, 128), np.uint16), 64, 64, 0.045, 5)
+    with pytest.raises(RuntimeError):
+        G.block_scaling(np.zeros((128, 128), np.uint16), 64, 64, 0.045, 1, channel=True)
+
+
+@pytest.mark.parametrize("qt", [1, 2, 3])
+@pytest.mark.parametrize("strategy", [1, 3])
+def test_e8mx(G, qt, strategy):
+    a = E.fixture_words(256, 256, [(0, 70, 21000, 53768)])
+    b = data_gen.c2_student_t(67, 93, seed=qt)
+    every = np.arange(0x0000, 0x10000, dtype=np.uint32).astype(np.uint16).reshape(256, 256)
+    every = every[(every & 0x7F80) != 0x7F80].reshape(-1, 64)      # all finite bf16 values
+    for x in (a, b, every):
+        print("e8mx", qt, strategy, x.shape, flush=True)
+        want = O.e8mx(x, 128, 128, qt, strategy)
+        assert np.array_equal(G.e8mx(x, 128, 128, qt, strategy), want)
+        assert np.array_equal(G.e8mx(x, 128, 128, qt, strategy, inplace=True), want)
+    if strategy == 3:
+        small = E.fixture_words(64, 64, [(0, 30, 21000, 53768)])
+        assert np.array_equal(G.e8mx(small, 32, 32, qt, 3), E.e8mx_tensor(small, qt))
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2, O.E3M2, O.E2M3])
+def test_quant_dequant_ops(G, fmt):
+    rng = np.random.default_rng(fmt)
+    lim = O.FMAX[fmt]
+    x = np.concatenate([rng.uniform(-lim * 1.2, lim * 1.2, 200000), rng.standard_normal(100000) * lim / 50,
+                        rng.standard_normal(50000) * 1e-3, [463, 464, 465, 0.0, -0.0, 1e30, -1e30]]).astype(np.float32)
+    print("quant_dequant", fmt, flush=True)
+    got, want = G.quant_dequant(x, fmt), O.quant_dequant(x, fmt)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    if fmt in (O.E4M3, O.E5M2):
+        dt = torch.float8_e4m3fn if fmt == O.E4M3 else torch.float8_e5m2
+        inr = np.abs(x) <= (448 if fmt == O.E4M3 else 57344)
+        ref = torch.from_numpy(x[inr]).to(dt).float().numpy()
+        assert np.array_equal(got[inr], ref)
+
+
+@pytest.mark.parametrize("rne", [False, True])
+def test_e4m3_with_e8_scale_ops(G, rne):
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-1000, 1000, 300000).astype(np.float32)
+    x = x[x != 0]
+    print("e4m3_with_e8_scale", rne, flush=True)
+    got, want = G.e4m3_with_e8_scale(x, rne), O.e4m3_with_e8_scale(x, rne)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
