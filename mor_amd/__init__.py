@@ -1,0 +1,9 @@
+"""MI355X (gfx950) implementation of the MoR fake-quantization path.
+
+`mor_amd._cabi` binds the C ABI of libmor_hip.so (include/mor_hip.h); `mor_amd.ops` registers the `torch.ops.mor.*`
+operators on top of it and mirrors the reference's `mor.ops` Python API.  `import mor` gives the drop-in name.
+"""
+from . import _cabi  # noqa: F401
+from . import ops  # noqa: F401
+
+__all__ = ["ops"]
