@@ -78,19 +78,33 @@ class Launcher:
 
 
 def time_launches(torch, fn, steps, warmup):
-    """-> (mean ms per launch from per-launch HIP events, wall ms per launch)"""
+    """-> (mean ms per launch from one pair of HIP events around `steps` back-to-back launches, wall ms per launch)"""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    for a, b in ev:
-        a.record()
+    a.record()
+    for _ in range(steps):
         fn()
-        b.record()
+    b.record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    return sum(a.elapsed_time(b) for a, b in ev) / steps, wall
+    return a.elapsed_time(b) / steps, wall
+
+
+def read_traffic(kernel):
+    """HBM bytes per launch of `kernel` from the committed counter summary (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
+    each scaled by the same counter's reading for the library's plain copy kernel); None when there is no summary."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")
+    try:
+        for line in open(path):
+            f = line.split()
+            if len(f) >= 3 and f[0] == "traffic_bytes" and f[1] == kernel:
+                return int(f[2])
+    except OSError:
+        pass
+    return None
 
 
 def main():
@@ -121,22 +135,24 @@ def main():
     ]
     bytes_per_step = sum(b for _, _, b in launches)
 
-    def step(events=None):
-        for i, (_, fn, _) in enumerate(launches):
-            if events is not None:
-                events[i][0].record()
+    def step():
+        for _, fn, _ in launches:
             fn()
-            if events is not None:
-                events[i][1].record()
 
     for _ in range(W):
         step()
     torch.cuda.synchronize()
-    evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in launches] for _ in range(K)]
+    # The timed region holds exactly K steps of work.  Its launches are grouped by format (K x E4M3, K x E5M2,
+    # K x E2M3) so that one pair of HIP events brackets the K launches of each kernel: an event between every two
+    # launches would add its own few microseconds to 45-microsecond kernels.
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(len(launches) + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for k in range(K):
-        step(evs[k])
+    marks[0].record()
+    for i, (_, fn, _) in enumerate(launches):
+        for _ in range(K):
+            fn()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / K
@@ -144,12 +160,12 @@ def main():
 
     per_kernel = {}
     for i, (name, _, nbytes) in enumerate(launches):
-        ms = sum(evs[k][i][0].elapsed_time(evs[k][i][1]) for k in range(K)) / K
+        ms = marks[i].elapsed_time(marks[i + 1]) / K
         per_kernel[name] = {"ms": round(ms, 5), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                             "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "bytes": nbytes}
     dom = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
     roofline = {"bound": "hbm", "kernel": dom, "achieved": per_kernel[dom]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": per_kernel[dom]["frac"], "traffic": None, "per_kernel": per_kernel}
+                "frac": per_kernel[dom]["frac"], "traffic": read_traffic(dom), "per_kernel": per_kernel}
 
     extra = {}
     if not args.no_extra:
