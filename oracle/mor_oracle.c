@@ -347,14 +347,16 @@ static void block_error(const blk_t* b, float amax, int e8, int flavour, float* 
     int64_t nthreads = tbx * tby;
     if (nthreads <= 0 || nthreads % 32 != 0 || nthreads > 1024) geom = 0;
     if (!geom) {
-        float s4 = 0.0f, s5 = 0.0f;
+        /* no reference launch geometry exists for this shape, hence no reference order: the fp32 terms are
+         * added in double and rounded once */
+        double s4 = 0.0, s5 = 0.0;
         for (int64_t r = b->r0; r < b->r1; ++r)
             for (int64_t c = b->c0; c < b->c1; ++c) {
                 float e4, e5;
                 err_terms(ld(b, r, c), amax, e8, flavour, &e4, &e5);
                 s4 += e4; s5 += e5;
             }
-        *e4_o = s4; *e5_o = s5;
+        *e4_o = (float)s4; *e5_o = (float)s5;
         return;
     }
     float p4[1024], p5[1024];
@@ -591,16 +593,49 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
     int32_t gnnz = 0;
     for (int64_t k = 0; k < nb; ++k) { gamax = max_nn(gamax, bamax[k]); gnnz += bnnz[k]; }
 
-    /* FQ:1095-1176 / FQ:1633-1752 */
+    /* FQ:1095-1176 / FQ:1633-1752.  The per-element arithmetic does not depend on the launch geometry; the
+     * order of the fp32 additions of the error sum does.  Three geometries of the reference are reproduced:
+     *   block op, 32x32 threads per block (needs bcols % 64 == 0, brows % 32 == 0);
+     *   channel op, row blocks 1 x N with N >= 128, N % 128 == 0: 64 threads per block (FQ:2502, 2399-2415);
+     *   channel op, column blocks rows x 1 (one block row) with cols % 64 == 0: 32x16 threads per 64 columns,
+     *     the sum of a thread block goes to its first column, the other 63 get 0 (FQ:2503, 1750-1751).
+     * For any other shape the reference has no working launch, hence no order: terms are added in double. */
+    const int geom_block = !channel && (bcols % 64 == 0) && (brows % 32 == 0);
+    const int geom_row = channel && brows == 1 && bcols >= 128 && (bcols % 128 == 0);
+    const int geom_col = channel && bcols == 1 && brows == rows && (cols % 64 == 0) && (rows % 16 == 0);
+    if (geom_col) {
+        for (int64_t k = 0; k < nb; ++k) berr[k] = 0.0f;
+#pragma omp parallel for schedule(static)
+        for (int64_t tb = 0; tb < cols / 64; ++tb) {
+            float partial[512];
+            for (int ty = 0; ty < 16; ++ty)
+                for (int tx = 0; tx < 32; ++tx) {
+                    int64_t c1 = tb * 64 + 2 * tx + 1, c2 = c1 - 1;       /* high half = odd column */
+                    float sf1 = mor_oracle_scaling_factor(gamax, bamax[c1], (int)ss_mode);
+                    float sf2 = mor_oracle_scaling_factor(gamax, bamax[c2], (int)ss_mode);
+                    float e1 = 0.0f, e2 = 0.0f;
+                    for (int64_t r = ty; r < rows; r += 16) {
+                        float t1, t2;
+                        float x1 = mor_oracle_bf16_to_fp32(in[r * cols + c1]), x2 = mor_oracle_bf16_to_fp32(in[r * cols + c2]);
+                        float q1 = bs_element(x1, sf1, ss_mode, flavour, &t1);
+                        float q2 = bs_element(x2, sf2, ss_mode, flavour, &t2);
+                        if (x1 != 0.0f) e1 += t1;
+                        if (x2 != 0.0f) e2 += t2;
+                        tmp[r * cols + c1] = (uint16_t)store_bf16(q1, flavour);
+                        tmp[r * cols + c2] = (uint16_t)store_bf16(q2, flavour);
+                    }
+                    partial[ty * 32 + tx] = e1 + e2;
+                }
+            berr[tb * 64] = block_tree_sum(partial, 512);
+        }
+    } else {
 #pragma omp parallel for schedule(static)
     for (int64_t k = 0; k < nb; ++k) {
         int64_t by = k / gx, bx = k % gx;
         float sf = mor_oracle_scaling_factor(gamax, bamax[k], (int)ss_mode);
         int64_t r0 = by * brows, c0 = bx * bcols;
-        int geom = !channel && (bcols % 64 == 0) && (brows % 32 == 0);
         float partial[1024];
-        float seq = 0.0f;
-        if (geom) {
+        if (geom_block) {
             /* 32x32 threads over packed columns, r outer / c inner, high half first */
             for (int ty = 0; ty < 32; ++ty)
                 for (int tx = 0; tx < 32; ++tx) {
@@ -609,17 +644,37 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
                         for (int64_t pc = tx; pc < bcols / 2; pc += 32) {
                             float e1, e2;
                             int64_t i1 = (r0 + r) * cols + c0 + 2 * pc + 1, i2 = i1 - 1;
-                            float q1 = bs_element(mor_oracle_bf16_to_fp32(in[i1]), sf, ss_mode, flavour, &e1);
-                            float q2 = bs_element(mor_oracle_bf16_to_fp32(in[i2]), sf, ss_mode, flavour, &e2);
-                            if (mor_oracle_bf16_to_fp32(in[i1]) != 0.0f) acc += e1;
-                            if (mor_oracle_bf16_to_fp32(in[i2]) != 0.0f) acc += e2;
+                            float x1 = mor_oracle_bf16_to_fp32(in[i1]), x2 = mor_oracle_bf16_to_fp32(in[i2]);
+                            float q1 = bs_element(x1, sf, ss_mode, flavour, &e1);
+                            float q2 = bs_element(x2, sf, ss_mode, flavour, &e2);
+                            if (x1 != 0.0f) acc += e1;
+                            if (x2 != 0.0f) acc += e2;
                             tmp[i1] = (uint16_t)store_bf16(q1, flavour);
                             tmp[i2] = (uint16_t)store_bf16(q2, flavour);
                         }
                     partial[ty * 32 + tx] = acc;
                 }
             berr[k] = block_tree_sum(partial, 1024);
+        } else if (geom_row) {
+            /* 64 threads along the row, one packed column each per step; odd and even columns summed apart */
+            for (int tx = 0; tx < 64; ++tx) {
+                float e1 = 0.0f, e2 = 0.0f;
+                for (int64_t pc = tx; pc < bcols / 2; pc += 64) {
+                    float t1, t2;
+                    int64_t i1 = r0 * cols + c0 + 2 * pc + 1, i2 = i1 - 1;
+                    float x1 = mor_oracle_bf16_to_fp32(in[i1]), x2 = mor_oracle_bf16_to_fp32(in[i2]);
+                    float q1 = bs_element(x1, sf, ss_mode, flavour, &t1);
+                    float q2 = bs_element(x2, sf, ss_mode, flavour, &t2);
+                    if (x1 != 0.0f) e1 += t1;
+                    if (x2 != 0.0f) e2 += t2;
+                    tmp[i1] = (uint16_t)store_bf16(q1, flavour);
+                    tmp[i2] = (uint16_t)store_bf16(q2, flavour);
+                }
+                partial[tx] = e1 + e2;
+            }
+            berr[k] = block_tree_sum(partial, 64);
         } else {
+            double seq = 0.0;
             for (int64_t r = r0; r < r0 + brows; ++r)
                 for (int64_t c = c0; c < c0 + bcols; ++c) {
                     float e;
@@ -628,8 +683,9 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
                     if (x != 0.0f) seq += e;
                     tmp[r * cols + c] = (uint16_t)store_bf16(q, flavour);
                 }
-            berr[k] = seq;
+            berr[k] = (float)seq;
         }
+    }
     }
     /* FQ:1178-1201: 1024 threads stride over the block errors, then the tree */
     float gerr;
