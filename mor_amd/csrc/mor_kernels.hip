@@ -868,14 +868,18 @@ extern "C" int mor_selftest_hw_cast(uint64_t* mismatches, void* stream) {
 // ================================================================================================
 // Block / channel scaling (FQ:951-1241, 1459-1752, host FQ:2013-2230, 2431-2660) and e8mx (FQ:1243-1428).
 //
-// Workspace layout (32-bit words): [0] tensor amax bits, [1] non-zero count, [2] number of error partials,
-// [3] spare, [WS_PARTIALS .. +MAX_PARTIALS) per-workgroup error sums, then one float per block (amax, turned
-// into the block's scale in place).
+// Workspace layout (32-bit words): [0] tensor amax bits, [1] non-zero count, [2..3] spare, then three arrays of
+// MAX_PARTIALS per-workgroup partials (error sums of pass 2; amax and non-zero counts of pass 1), then one float
+// per block (amax, turned into the block's scale in place).  Nothing is accumulated with atomics except the
+// per-column maxima of the column kernel, so all results are independent of scheduling.
 namespace mor {
 
 constexpr int WS_HEADER = 4;
 constexpr int MAX_PARTIALS = 8192;
-constexpr int WS_BLOCKS = WS_HEADER + MAX_PARTIALS;
+constexpr int WS_ERR = WS_HEADER;
+constexpr int WS_PAMAX = WS_HEADER + MAX_PARTIALS;
+constexpr int WS_PNNZ = WS_HEADER + 2 * MAX_PARTIALS;
+constexpr int WS_BLOCKS = WS_HEADER + 3 * MAX_PARTIALS;
 
 struct DivU32 {   // x / d for 32-bit x by multiply-shift (d >= 1)
     uint32_t d, mul, shift;
@@ -895,97 +899,158 @@ __device__ __forceinline__ uint32_t div_u32(uint32_t x, const DivU32& d) {
     return (t + ((x - t) >> 1)) >> (d.shift - 1);
 }
 
-__global__ void k_ws_init(uint32_t* ws, float* block_amax, int64_t nb, int zero_blocks) {
-    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
-    if (gtid < WS_HEADER) ws[gtid] = 0;
-    if (zero_blocks) for (int64_t i = gtid; i < nb; i += (int64_t)gridDim.x * WG) block_amax[i] = 0.0f;
+__global__ void k_zero_f32(float* p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) p[i] = 0.0f;
 }
 
 __device__ __forceinline__ int nnz_word(uint32_t w) {
     return ((w & 0x7FFFu) != 0) + ((w & 0x7FFF0000u) != 0);
 }
+__device__ __forceinline__ void acc_amax_nnz(float& amax, int& nnz, uint4 v) {
+    acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
+    nnz += nnz_word(v.x) + nnz_word(v.y) + nnz_word(v.z) + nnz_word(v.w);
+}
 
-// publish one workgroup's amax / nnz into the header (max and integer add are order independent)
-__device__ __forceinline__ void publish_global(uint32_t* ws, float amax, int nnz, float* s_f, int* s_i) {
+// one workgroup's amax / nnz -> its slot of the partial arrays; returns the workgroup amax to every thread
+__device__ __forceinline__ float publish_partial(uint32_t* ws, float amax, int nnz, float* s_f, int* s_i) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     amax = group_max(amax, 64);
     nnz = wave_sum_i(nnz);
+    __syncthreads();
     if (lane == 0) { s_f[wave] = amax; s_i[wave] = nnz; }
     __syncthreads();
+    const float a = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
     if (threadIdx.x == 0) {
-        float a = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
-        int n = s_i[0] + s_i[1] + s_i[2] + s_i[3];
-        atomicMax(&ws[0], f2u(a));
-        if (n) atomicAdd(reinterpret_cast<int*>(&ws[1]), n);
+        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = a;
+        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = s_i[0] + s_i[1] + s_i[2] + s_i[3];
     }
+    return a;
 }
 
-// pass 1, blocks 1 x 8G as lane groups over the flat chunk array (FQ:1430-1457, 1611-1629)
-__global__ __launch_bounds__(WG) void k_bs_amax_rowgroup(const uint4* in, uint32_t* ws, float* block_amax,
-                                                         int64_t nchunks, int G, int logG) {
+// tensor amax from the pass-1 partials (every thread of the workgroup gets it)
+__device__ __forceinline__ float reduce_partial_amax(const uint32_t* ws, int npart, float* s_f) {
+    const float* pa = reinterpret_cast<const float*>(ws) + WS_PAMAX;
+    float a = 0.0f;
+#pragma unroll 8
+    for (int i = threadIdx.x; i < npart; i += WG) a = fmaxf(a, pa[i]);
+    a = group_max(a, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s_f[threadIdx.x >> 6] = a;
+    __syncthreads();
+    return fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+}
+
+// pass 1, blocks 1 x 8G as lane groups over the flat chunk array (FQ:1430-1457, 1611-1629).  A workgroup takes
+// tiles of 8 * 256 consecutive chunks, all loads of a tile in flight at once.  block_amax may be NULL (e8mx).
+__global__ __launch_bounds__(WG) void k_bs_amax_flat(const uint4* in, uint32_t* ws, float* block_amax,
+                                                     int64_t nchunks, int G, int logG) {
     __shared__ float s_f[WAVES];
     __shared__ int s_i[WAVES];
+    constexpr int NV = 8;
     float gmax = 0.0f;
     int nnz = 0;
-    for (int64_t c = (int64_t)blockIdx.x * WG + threadIdx.x; c < nchunks; c += (int64_t)gridDim.x * WG) {
-        uint4 v = in[c];
-        float amax = 0.0f;
-        acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
-        nnz += nnz_word(v.x) + nnz_word(v.y) + nnz_word(v.z) + nnz_word(v.w);
-        gmax = fmaxf(gmax, amax);
-        amax = group_max(amax, G);
-        if ((c & (G - 1)) == 0) block_amax[c >> logG] = amax;
+    const int64_t ntiles = (nchunks + NV * WG - 1) / (NV * WG);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t base = tile * (NV * WG) + threadIdx.x;
+        uint4 v[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            v[k] = make_uint4(0, 0, 0, 0);
+            if (base + k * WG < nchunks) v[k] = in[base + k * WG];
+        }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int64_t c = base + k * WG;
+            float amax = 0.0f;
+            acc_amax_nnz(amax, nnz, v[k]);
+            gmax = fmaxf(gmax, amax);
+            if (block_amax) {
+                amax = group_max(amax, G);
+                if (c < nchunks && (c & (G - 1)) == 0) block_amax[c >> logG] = amax;
+            }
+        }
     }
-    publish_global(ws, gmax, nnz, s_f, s_i);
+    publish_partial(ws, gmax, nnz, s_f, s_i);
 }
 
-// pass 1, one workgroup per block of any shape (FQ:951-1015); vec: 16-byte loads (cols and bcols multiples of 8)
-__global__ __launch_bounds__(WG) void k_bs_amax_block(const uint16_t* in, uint32_t* ws, float* block_amax, Shape sh, int vec) {
+// tensor amax of an unaligned or odd-sized buffer, element by element (e8mx only needs the tensor amax)
+__global__ __launch_bounds__(WG) void k_amax_scalar(const uint16_t* in, uint32_t* ws, int64_t n) {
     __shared__ float s_f[WAVES];
     __shared__ int s_i[WAVES];
-    const int64_t bid = blockIdx.x;
-    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
-    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
     float amax = 0.0f;
-    int nnz = 0;
-    if (vec) {
-        const uint4* in4 = reinterpret_cast<const uint4*>(in);
-        const int64_t row_stride = sh.cols >> 3, cpr = sh.bcols >> 3;
-        for (int64_t i = threadIdx.x; i < sh.brows * cpr; i += WG) {
-            int64_t r = i / cpr, cc = i - r * cpr;
-            uint4 v = in4[(r0 + r) * row_stride + (c0 >> 3) + cc];
-            acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
-            nnz += nnz_word(v.x) + nnz_word(v.y) + nnz_word(v.z) + nnz_word(v.w);
-        }
-    } else {
-        for (int64_t i = threadIdx.x; i < sh.brows * sh.bcols; i += WG) {
-            int64_t r = i / sh.bcols, c = i - r * sh.bcols;
-            uint32_t a = ((uint32_t)in[(r0 + r) * sh.cols + c0 + c] << 16) & 0x7FFFFFFFu;
-            amax = fmaxf(amax, u2f(a));
-            nnz += ((a & 0x7FFF0000u) != 0);
-        }
-    }
-    publish_global(ws, amax, nnz, s_f, s_i);       // also leaves the per-wave maxima in s_f
-    if (threadIdx.x == 0) block_amax[bid] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG)
+        amax = fmaxf(amax, fabsf(bf16_one(in[i])));
+    publish_partial(ws, amax, 0, s_f, s_i);
 }
 
-// pass 1, column blocks N x 1 (FQ:1538-1610): a thread owns 8 adjacent columns over a segment of rows and merges
+// pass 1, one workgroup per block of any shape (FQ:951-1015), blocks taken grid-stride;
+// vec: 16-byte loads (cols and bcols multiples of 8, aligned base)
+__global__ __launch_bounds__(WG) void k_bs_amax_block(const uint16_t* in, uint32_t* ws, float* block_amax, Shape sh, int vec,
+                                                      DivU32 d_gx, DivU32 d_cpr) {
+    __shared__ float s_f[WAVES];
+    __shared__ float s_b[WAVES];
+    __shared__ int s_i[WAVES];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t nb = (uint32_t)(sh.gy * sh.gx);
+    float gmax = 0.0f;
+    int nnz = 0;
+    for (uint32_t bid = blockIdx.x; bid < nb; bid += gridDim.x) {
+        const uint32_t by = div_u32(bid, d_gx), bx = bid - by * (uint32_t)sh.gx;
+        const int64_t r0 = (int64_t)by * sh.brows, c0 = (int64_t)bx * sh.bcols;
+        float amax = 0.0f;
+        if (vec) {
+            const uint32_t row_stride = (uint32_t)(sh.cols >> 3), cpr = (uint32_t)(sh.bcols >> 3);
+            const uint4* bin = reinterpret_cast<const uint4*>(in) + (r0 * row_stride + (c0 >> 3));
+            const uint32_t nch = (uint32_t)sh.brows * cpr;
+#pragma unroll 4
+            for (uint32_t i = threadIdx.x; i < nch; i += WG) {
+                const uint32_t r = div_u32(i, d_cpr), cc = i - r * cpr;
+                acc_amax_nnz(amax, nnz, bin[r * row_stride + cc]);
+            }
+        } else {
+            for (int64_t i = threadIdx.x; i < sh.brows * sh.bcols; i += WG) {
+                int64_t r = i / sh.bcols, c = i - r * sh.bcols;
+                uint32_t a = ((uint32_t)in[(r0 + r) * sh.cols + c0 + c] << 16) & 0x7FFFFFFFu;
+                amax = fmaxf(amax, u2f(a));
+                nnz += ((a & 0x7FFF0000u) != 0);
+            }
+        }
+        amax = group_max(amax, 64);
+        __syncthreads();
+        if (lane == 0) s_b[wave] = amax;
+        __syncthreads();
+        amax = fmaxf(fmaxf(s_b[0], s_b[1]), fmaxf(s_b[2], s_b[3]));
+        if (threadIdx.x == 0) block_amax[bid] = amax;
+        gmax = fmaxf(gmax, amax);
+    }
+    publish_partial(ws, gmax, nnz, s_f, s_i);
+}
+
+// pass 1, column blocks N x 1 (FQ:1538-1610): a workgroup covers 256 adjacent columns (32 groups of 8) with 8 row
+// lanes; a thread takes every 8th row of a row segment, the 8 row lanes meet in LDS and one thread per column merges
 // into the (zero-initialised) per-block maxima with atomicMax on the bit patterns of non-negative floats.
 __global__ __launch_bounds__(WG) void k_bs_amax_col(const uint16_t* in, uint32_t* ws, float* block_amax, Shape sh,
                                                     int rows_per_wg, int vec) {
+    __shared__ float s_m[8][32 * 8 + 8];
     __shared__ float s_f[WAVES];
     __shared__ int s_i[WAVES];
-    const int64_t by = blockIdx.z;                                   // block row
-    const int64_t r_begin = by * sh.brows + (int64_t)blockIdx.y * rows_per_wg;
-    const int64_t r_end = min(r_begin + rows_per_wg, (by + 1) * sh.brows);
-    const int64_t col0 = ((int64_t)blockIdx.x * WG + threadIdx.x) * 8;
-    float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int cg = threadIdx.x & 31, rl = threadIdx.x >> 5;
+    const int64_t col0 = ((int64_t)blockIdx.x * 32 + cg) * 8;
+    const int64_t segs_per_block = (sh.brows + rows_per_wg - 1) / rows_per_wg;
+    const int ncol = (int)max((int64_t)0, min((int64_t)8, sh.cols - col0));
+    float gmax = 0.0f;
     int nnz = 0;
-    if (col0 < sh.cols) {
-        if (vec) {
+    // row segments of all block rows, taken grid-stride along y
+    for (int64_t seg = blockIdx.y; seg < sh.gy * segs_per_block; seg += gridDim.y) {
+        const int64_t by = seg / segs_per_block;
+        const int64_t r_begin = by * sh.brows + (seg - by * segs_per_block) * rows_per_wg;
+        const int64_t r_end = min(r_begin + rows_per_wg, (by + 1) * sh.brows);
+        float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (vec && ncol == 8) {
             const uint4* in4 = reinterpret_cast<const uint4*>(in);
-            for (int64_t r = r_begin; r < r_end; ++r) {
-                uint4 v = in4[(r * sh.cols + col0) >> 3];
+#pragma unroll 8
+            for (int64_t r = r_begin + rl; r < r_end; r += 8) {
+                const uint4 v = in4[(r * sh.cols + col0) >> 3];
                 const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -995,20 +1060,36 @@ __global__ __launch_bounds__(WG) void k_bs_amax_col(const uint16_t* in, uint32_t
                 }
             }
         } else {
-            const int ncol = (int)min((int64_t)8, sh.cols - col0);
-            for (int64_t r = r_begin; r < r_end; ++r)
-                for (int j = 0; j < ncol; ++j) {
-                    uint32_t a = ((uint32_t)in[r * sh.cols + col0 + j] << 16) & 0x7FFFFFFFu;
-                    m[j] = fmaxf(m[j], u2f(a));
-                    nnz += (a != 0);
-                }
+            for (int64_t r = r_begin + rl; r < r_end; r += 8)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (j < ncol) {
+                        const uint32_t a = ((uint32_t)in[r * sh.cols + col0 + j] << 16) & 0x7FFFFFFFu;
+                        m[j] = fmaxf(m[j], u2f(a));
+                        nnz += (a != 0);
+                    }
         }
-        const int ncol = (int)min((int64_t)8, sh.cols - col0);
-        for (int j = 0; j < ncol; ++j)
-            if (m[j] > 0.0f) atomicMax(reinterpret_cast<uint32_t*>(&block_amax[by * sh.cols + col0 + j]), f2u(m[j]));
+        __syncthreads();                       // the previous segment's readers are done
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s_m[rl][cg * 8 + j] = m[j];
+        __syncthreads();
+        float cm = s_m[0][threadIdx.x];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) cm = fmaxf(cm, s_m[k][threadIdx.x]);
+        const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        if (c < sh.cols && cm > 0.0f) atomicMax(reinterpret_cast<uint32_t*>(&block_amax[by * sh.cols + c]), f2u(cm));
+        gmax = fmaxf(gmax, cm);
     }
-    float gmax = fmaxf(fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3])), fmaxf(fmaxf(m[4], m[5]), fmaxf(m[6], m[7])));
-    publish_global(ws, gmax, nnz, s_f, s_i);
+    const uint32_t slot = blockIdx.x + gridDim.x * blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    gmax = group_max(gmax, 64);
+    nnz = wave_sum_i(nnz);
+    if (lane == 0) { s_f[wave] = gmax; s_i[wave] = nnz; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        reinterpret_cast<float*>(ws)[WS_PAMAX + slot] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        reinterpret_cast<int*>(ws)[WS_PNNZ + slot] = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    }
 }
 
 // FQ:1059-1093
@@ -1034,9 +1115,22 @@ __device__ __forceinline__ float scaling_factor(float global_amax, float block_a
     return sf;
 }
 
-// pass 1.5: block amax -> block scale, in place
-__global__ __launch_bounds__(WG) void k_bs_scales(const uint32_t* ws, float* block_amax, int64_t nb, int ss_mode) {
-    const float gamax = u2f(ws[0]);
+// pass 1.5 (FQ:1017-1049 + the scale of every block): tensor amax and non-zero count from the partials into the
+// header, block amax -> block scale in place
+__global__ __launch_bounds__(WG) void k_bs_scales(uint32_t* ws, float* block_amax, int64_t nb, int ss_mode, int npart) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const float gamax = reduce_partial_amax(ws, npart, s_f);
+    if (blockIdx.x == 0) {
+        const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
+        int n = 0;
+#pragma unroll 8
+        for (int i = threadIdx.x; i < npart; i += WG) n += pn[i];
+        n = wave_sum_i(n);
+        if ((threadIdx.x & 63) == 0) s_i[threadIdx.x >> 6] = n;
+        __syncthreads();
+        if (threadIdx.x == 0) { ws[0] = f2u(gamax); ws[1] = (uint32_t)(s_i[0] + s_i[1] + s_i[2] + s_i[3]); }
+    }
     for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < nb; i += (int64_t)gridDim.x * WG)
         block_amax[i] = scaling_factor(gamax, block_amax[i], ss_mode);
 }
@@ -1142,9 +1236,94 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
         if (lane == 0) s_f[wave] = err;
         __syncthreads();
         if (threadIdx.x == 0) {
-            reinterpret_cast<float*>(ws)[WS_HEADER + blockIdx.x] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
-            if (blockIdx.x == 0) ws[2] = gridDim.x;
+            reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
         }
+    }
+}
+
+// pass 2 / pass 4 for column blocks N x 1 with aligned rows (the geometry of k_bs_amax_col): a thread owns 8 adjacent
+// columns over a segment of rows, so its 8 scales and their reciprocals are computed once.  Threads whose scales are
+// not all in the fast range use the exact arithmetic.
+template <bool WRITE, bool ERR>
+__global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_t* out, uint32_t* ws, const float* scales,
+                                                     const int32_t* meta, int gate, Shape sh, int rows_per_wg) {
+    __shared__ float s_f[WAVES];
+    if (gate > 0 && meta[0] != gate) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t col0 = ((int64_t)blockIdx.x * WG + threadIdx.x) * 8;
+    const int64_t segs_per_block = (sh.brows + rows_per_wg - 1) / rows_per_wg;
+    const int64_t row_stride = sh.cols >> 3;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    uint4* out4 = reinterpret_cast<uint4*>(out);
+    float err = 0.0f;
+    if (col0 < sh.cols) {
+        for (int64_t seg = blockIdx.y; seg < sh.gy * segs_per_block; seg += gridDim.y) {
+            const int64_t by = seg / segs_per_block;
+            const int64_t r_begin = by * sh.brows + (seg - by * segs_per_block) * rows_per_wg;
+            const int64_t r_end = min(r_begin + rows_per_wg, (by + 1) * sh.brows);
+            const float* sp = scales + by * sh.cols + col0;
+            Scale sc[8];
+            float rs[8];
+            bool fast = true;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { sc[j] = make_scale(sp[j]); rs[j] = 1.0f / sc[j].s; fast = fast && sc[j].fast; }
+            if (fast) {
+#pragma unroll 1
+                for (int64_t r = r_begin; r < r_end; r += 4) {
+                    uint4 v[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        v[k] = make_uint4(0, 0, 0, 0);
+                        if (r + k < r_end) v[k] = in4[(r + k) * row_stride + (col0 >> 3)];
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+                        float row_err = 0.0f;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const float a = fabsf(bf16_lo(w[j])), b = fabsf(bf16_hi(w[j]));
+                            const uint32_t p = hw_pack2<FMT_E4M3>(a * sc[2 * j].s, b * sc[2 * j + 1].s);
+                            const float ca = hw_unpack<FMT_E4M3, 0>(p), cb = hw_unpack<FMT_E4M3, 1>(p);
+                            const float ta = ca * rs[2 * j], tb = cb * rs[2 * j + 1];
+                            const float qa = fmaf(fmaf(-ta, sc[2 * j].s, ca), rs[2 * j], ta);
+                            const float qb = fmaf(fmaf(-tb, sc[2 * j + 1].s, cb), rs[2 * j + 1], tb);
+                            const bool za = (a == 0.0f), zb = (b == 0.0f);
+                            row_err = fmaf(fabsf(qa - a), za ? 0.0f : __builtin_amdgcn_rcpf(a), row_err);
+                            row_err = fmaf(fabsf(qb - b), zb ? 0.0f : __builtin_amdgcn_rcpf(b), row_err);
+                            const uint32_t lo = za ? 0u : ((rhu_bits(qa) >> 16) | (w[j] & 0x8000u));
+                            const uint32_t hi = zb ? 0u : ((rhu_bits(qb) & 0xFFFF0000u) | (w[j] & 0x80000000u));
+                            w[j] = lo | hi;
+                        }
+                        err += row_err;
+                        if constexpr (WRITE) {
+                            if (r + k < r_end) out4[(r + k) * row_stride + (col0 >> 3)] = make_uint4(w[0], w[1], w[2], w[3]);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll 1
+                for (int64_t r = r_begin; r < r_end; ++r) {
+                    const uint4 v = in4[r * row_stride + (col0 >> 3)];
+                    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float s0 = sp[2 * j], s1 = sp[2 * j + 1];
+                        float q0 = bs_element<false, false>(bf16_lo(w[j]), make_scale(s0), err);
+                        float q1 = bs_element<false, false>(bf16_hi(w[j]), make_scale(s1), err);
+                        w[j] = store_pair<false>(q0, q1);
+                    }
+                    if constexpr (WRITE) out4[r * row_stride + (col0 >> 3)] = make_uint4(w[0], w[1], w[2], w[3]);
+                }
+            }
+        }
+    }
+    if constexpr (ERR) {
+        err = wave_sum(err);
+        if (lane == 0) s_f[wave] = err;
+        __syncthreads();
+        if (threadIdx.x == 0)
+            reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x + gridDim.x * blockIdx.y] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
     }
 }
 
@@ -1152,9 +1331,10 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
 __global__ __launch_bounds__(WG) void k_bs_finalize(const uint32_t* ws, int npartials, float threshold, int32_t* meta,
                                                     float* gamax_o, int32_t* gnnz_o, float* gerr_o) {
     __shared__ float s_f[WAVES];
-    const float* part = reinterpret_cast<const float*>(ws) + WS_HEADER;
+    const float* part = reinterpret_cast<const float*>(ws) + WS_ERR;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float acc = 0.0f;
+#pragma unroll 8
     for (int i = threadIdx.x; i < npartials; i += WG) acc += part[i];
     acc = wave_sum(acc);
     if (lane == 0) s_f[wave] = acc;
@@ -1181,22 +1361,6 @@ __global__ __launch_bounds__(WG) void k_copy_if(const uint16_t* in, uint16_t* ou
     for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = in[i];
 }
 
-// global amax only (e8mx, FQ:2292-2293)
-__global__ __launch_bounds__(WG) void k_global_amax(const uint16_t* in, uint32_t* ws, int64_t n, int64_t nvec) {
-    __shared__ float s_f[WAVES];
-    __shared__ int s_i[WAVES];
-    const int64_t stride = (int64_t)gridDim.x * WG;
-    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
-    const uint4* in4 = reinterpret_cast<const uint4*>(in);
-    float amax = 0.0f;
-    for (int64_t c = gtid; c < nvec; c += stride) {
-        uint4 v = in4[c];
-        acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
-    }
-    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) amax = fmaxf(amax, fabsf(bf16_one(in[i])));
-    publish_global(ws, amax, 0, s_f, s_i);
-}
-
 // FQ:1243-1327: keep MB mantissa bits by comparing the 23-bit mantissa with the reference's threshold tables
 // (on bf16 inputs they are the midpoints with ties to even; on scaled inputs, whose low 16 bits are not zero,
 // they are what they are).  Exponent 0 loses its mantissa, exponent 255 is left alone, a carry out of exponent
@@ -1207,14 +1371,14 @@ template <int MB> __device__ __forceinline__ float quant_e8m(float v) {
     uint32_t e = (b >> 23) & 0xFF, m = b & 0x7FFFFFu;
     if (e == 0) m = 0;
     else if (e != 255) {
-        // threshold j: even j -> midpoint (j << (7-MB)) + half, odd j -> next midpoint - 1, in units of 2^16
-        uint32_t k = 0;
-#pragma unroll
-        for (uint32_t j = 0; j < (1u << MB); ++j) {
-            const uint32_t half = 1u << (6 - MB);
-            const uint32_t t = (j & 1u) ? (((j + 1u) << (7 - MB)) - half - 1u) : ((j << (7 - MB)) + half);
-            k += (m > (t << 16)) ? 1u : 0u;
-        }
+        // The reference's thresholds, in units of 2^16: even j -> j*S + S/2, odd j -> j*S + S/2 - 1 with S = 2^(7-MB);
+        // k = number of thresholds below the mantissa.  With h = mantissa >> 16 plus one if any lower bit is set and
+        // u = h - S/2 this count is floor(u / S) plus one if that quotient is odd or the division leaves a remainder
+        // (nearest even on bf16 inputs, the same tables on inputs with low bits).
+        constexpr int S = 1 << (7 - MB);
+        const int u = (int)(m >> 16) + ((m & 0xFFFFu) != 0 ? 1 : 0) - S / 2;
+        const uint32_t q = (uint32_t)max(u, 0) >> (7 - MB);
+        const uint32_t k = (u < 0) ? 0u : q + (((q & 1u) | (((uint32_t)u & (S - 1)) != 0 ? 1u : 0u)));
         if (k == (1u << MB)) {
             m = 0; e++;
             if (e == 255) { e = 254; m = ((1u << MB) - 1u) << (23 - MB); }
@@ -1234,30 +1398,53 @@ template <int MB> __device__ __forceinline__ float e8mx_scale(float gamax, int s
     return sf;
 }
 
-template <int MB, bool EMU> __device__ __forceinline__ float e8mx_element(float x, float sf) {
-    float v = x * sf;
-    float dq = 0.0f;
-    if (v != 0.0f) dq = quant_e8m<MB>(v);
-    return dq / sf;
+// One element of FQ:1399-1419.  UNIT: the scale is 1 (no tensor-amax strategy), so the multiply and the divide are
+// exact no-ops.  Otherwise dq / sf is a reciprocal-multiply with one exact-residual correction (rs = 1 / sf correctly
+// rounded), which gives the rounded quotient when the operands are well inside the exponent range and the
+// significand of sf is not all ones; the IEEE division covers the rest.
+template <int MB, bool UNIT> __device__ __forceinline__ float e8mx_element(float x, float sf, float rs, bool markstein_ok) {
+    if constexpr (UNIT) {
+        return (x != 0.0f) ? quant_e8m<MB>(x) : 0.0f;
+    } else {
+        float v = x * sf;
+        float dq = 0.0f;
+        if (v != 0.0f) dq = quant_e8m<MB>(v);
+        const uint32_t e = (f2u(dq) >> 23) & 0xFF;
+        if (markstein_ok && e > 30 && e < 225) {
+            float t = dq * rs;
+            return fmaf(fmaf(-t, sf, dq), rs, t);
+        }
+        return dq / sf;
+    }
 }
 
 // FQ:1361-1428
-template <int MB, bool EMU>
-__global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, const uint32_t* ws, int strategy, int64_t n, int64_t nvec) {
-    const float sf = e8mx_scale<MB>(u2f(ws[0]), strategy);
+template <int MB, bool EMU, bool UNIT>
+__global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, const uint32_t* ws, int npart, int strategy, int64_t n, int64_t nvec) {
+    __shared__ float s_f[WAVES];
+    const float gamax = (!UNIT && strategy == 1) ? reduce_partial_amax(ws, npart, s_f) : 0.0f;
+    const float sf = UNIT ? 1.0f : e8mx_scale<MB>(gamax, strategy);
+    const float rs = 1.0f / sf;
+    const bool mk = (f2u(sf) & 0x7FFFFFu) != 0x7FFFFFu;
     const int64_t stride = (int64_t)gridDim.x * WG;
     const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
     const uint4* in4 = reinterpret_cast<const uint4*>(in);
     uint4* out4 = reinterpret_cast<uint4*>(out);
-    for (int64_t c = gtid; c < nvec; c += stride) {
-        uint4 v = in4[c];
-        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    constexpr int NV = 4;
+    for (int64_t c0 = gtid; c0 < nvec; c0 += stride * NV) {
+        uint4 v[NV];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            w[j] = store_pair<EMU>(e8mx_element<MB, EMU>(bf16_lo(w[j]), sf), e8mx_element<MB, EMU>(bf16_hi(w[j]), sf));
-        out4[c] = make_uint4(w[0], w[1], w[2], w[3]);
+        for (int k = 0; k < NV; ++k) { v[k] = make_uint4(0, 0, 0, 0); if (c0 + k * stride < nvec) v[k] = in4[c0 + k * stride]; }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                w[j] = store_pair<EMU>(e8mx_element<MB, UNIT>(bf16_lo(w[j]), sf, rs, mk), e8mx_element<MB, UNIT>(bf16_hi(w[j]), sf, rs, mk));
+            if (c0 + k * stride < nvec) out4[c0 + k * stride] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
     }
-    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = store_bf16<EMU>(e8mx_element<MB, EMU>(bf16_one(in[i]), sf));
+    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = store_bf16<EMU>(e8mx_element<MB, UNIT>(bf16_one(in[i]), sf, rs, mk));
 }
 
 }  // namespace mor
@@ -1269,7 +1456,7 @@ extern "C" size_t mor_workspace_bytes(int op, int64_t rows, int64_t cols, int64_
         case MOR_OP_CHANNEL_SCALING:
             return (size_t)(WS_BLOCKS + cdiv(rows, brows) * cdiv(cols, bcols)) * 4;
         case MOR_OP_E8MX:
-            return (size_t)WS_HEADER * 4;
+            return (size_t)WS_BLOCKS * 4;
         default:
             return 0;
     }
@@ -1325,35 +1512,56 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
     const int vec = (aligned16(input) && aligned16(output) && cols % 8 == 0) ? 1 : 0;
     const bool col = (bcols == 1 && brows > 1);
 
-    // pass 1: per-block amax, tensor amax, non-zero count
-    k_ws_init<<<col ? grid_for(nb) : 1, WG, 0, st>>>(ws, blocks, nb, col ? 1 : 0);
+    // pass 1: per-block amax, per-workgroup partials of the tensor amax and the non-zero count
     const int64_t G = bcols / 8;
+    int npart;
     if (col) {
-        const int rows_per_wg = (int)std::min<int64_t>(brows, 128);
-        dim3 grid((unsigned)cdiv(cdiv(cols, 8), WG), (unsigned)cdiv(brows, rows_per_wg), (unsigned)sh.gy);
-        k_bs_amax_col<<<grid, WG, 0, st>>>(in16, ws, blocks, sh, rows_per_wg, vec);
+        k_zero_f32<<<grid_for(nb), WG, 0, st>>>(blocks, nb);
+        const int rows_per_wg = (int)std::min<int64_t>(brows, 256);
+        const unsigned gx = (unsigned)cdiv(cols, 256);
+        const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
+        if ((int64_t)gx > MAX_PARTIALS) return fail(MOR_ERR_INVALID_ARGUMENT, "too many columns (%lld)", (long long)cols);
+        const unsigned gy = (unsigned)std::min<int64_t>(segs, std::max<int64_t>(MAX_PARTIALS / gx, 1));
+        npart = (int)(gx * gy);
+        k_bs_amax_col<<<dim3(gx, gy), WG, 0, st>>>(in16, ws, blocks, sh, rows_per_wg, vec);
     } else if (vec && brows == 1 && bcols % 8 == 0 && is_pow2(G) && G <= 64) {
-        k_bs_amax_rowgroup<<<grid_for(rows * cols / 8, 16), WG, 0, st>>>(static_cast<const uint4*>(input), ws, blocks, rows * cols / 8, (int)G, ilog2(G));
+        const int64_t nchunks = rows * cols / 8;
+        npart = (int)std::min<int64_t>(cdiv(nchunks, 8 * WG), MAX_PARTIALS);
+        k_bs_amax_flat<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, blocks, nchunks, (int)G, ilog2(G));
     } else {
-        k_bs_amax_block<<<(int)nb, WG, 0, st>>>(in16, ws, blocks, sh, (vec && bcols % 8 == 0) ? 1 : 0);
+        const int v1 = (vec && bcols % 8 == 0 && brows * (cols / 8) < 0x7FFFFFFFll) ? 1 : 0;
+        npart = (int)std::min<int64_t>(nb, MAX_PARTIALS);
+        k_bs_amax_block<<<npart, WG, 0, st>>>(in16, ws, blocks, sh, v1, make_div((uint32_t)sh.gx),
+                                              make_div((uint32_t)std::max<int64_t>(bcols / 8, 1)));
     }
-    // pass 1.5: scales
-    k_bs_scales<<<grid_for(nb), WG, 0, st>>>(ws, blocks, nb, (int)ss_mode);
+    // pass 1.5: tensor amax and non-zero count into the header, block scales
+    k_bs_scales<<<(int)std::min<int64_t>(cdiv(nb, WG), 256), WG, 0, st>>>(ws, blocks, nb, (int)ss_mode, npart);
     // pass 2: quantize (out of place: write now; in place: error only), error partials
-    const bool vec2 = vec && (col || bcols % 8 == 0);
-    const int64_t work = vec2 ? rows * cols / 8 : rows * cols;
-    const int grid2 = (int)std::min<int64_t>(std::max<int64_t>(cdiv(work, WG), 1), MAX_PARTIALS);
-    DivU32 d0 = make_div((uint32_t)std::max<int64_t>(cols / 8, 1)), d1 = make_div((uint32_t)brows),
-           d2 = make_div((uint32_t)std::max<int64_t>(bcols / 8, 1)), d3 = make_div((uint32_t)bcols);
-    const bool e8 = (ss_mode == 2);
-    dispatch_bs_quant(e8, emu, col, !inplace, true, grid2, st, in16, out16, ws, blocks, meta, 0, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
     // pass 3: decision and scalars
-    k_bs_finalize<<<1, WG, 0, st>>>(ws, grid2, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
     // pass 4: bf16 fallback (out of place: copy if meta == 3) or the quantized write (in place: only if meta == 1)
-    if (inplace) {
-        dispatch_bs_quant(e8, emu, col, true, false, grid2, st, in16, out16, ws, blocks, meta, 1, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
+    const bool e8 = (ss_mode == 2);
+    const int64_t n = rows * cols;
+    if (col && vec && !emu && !e8) {
+        const int rows_per_wg = (int)std::min<int64_t>(brows, 16);
+        const unsigned gx = (unsigned)cdiv(cdiv(cols, 8), WG);
+        const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
+        const dim3 grid(gx, (unsigned)std::min<int64_t>(segs, std::max<int64_t>(MAX_PARTIALS / gx, 1)));
+        if (inplace) k_bs_quant_col<false, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 0, sh, rows_per_wg);
+        else k_bs_quant_col<true, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 0, sh, rows_per_wg);
+        k_bs_finalize<<<1, WG, 0, st>>>(ws, (int)(grid.x * grid.y), (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        if (inplace) k_bs_quant_col<true, false><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 1, sh, rows_per_wg);
     } else {
-        const int64_t n = rows * cols, nvec = vec ? n / 8 : 0;
+        const bool vec2 = vec && (col || bcols % 8 == 0) && n / 8 < 0xFFFFFFFFll;
+        const int64_t work = vec2 ? n / 8 : n;
+        const int grid2 = (int)std::min<int64_t>(std::max<int64_t>(cdiv(work, WG), 1), MAX_PARTIALS);
+        DivU32 d0 = make_div((uint32_t)std::max<int64_t>(cols / 8, 1)), d1 = make_div((uint32_t)brows),
+               d2 = make_div((uint32_t)std::max<int64_t>(bcols / 8, 1)), d3 = make_div((uint32_t)bcols);
+        dispatch_bs_quant(e8, emu, col, !inplace, true, grid2, st, in16, out16, ws, blocks, meta, 0, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
+        k_bs_finalize<<<1, WG, 0, st>>>(ws, grid2, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        if (inplace) dispatch_bs_quant(e8, emu, col, true, false, grid2, st, in16, out16, ws, blocks, meta, 1, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
+    }
+    if (!inplace) {
+        const int64_t nvec = vec ? n / 8 : 0;
         k_copy_if<<<grid_for(nvec > 0 ? nvec : n, 16), WG, 0, st>>>(in16, out16, meta, 3, n, nvec);
     }
     return check_launch("mor_block_scaling");
@@ -1376,10 +1584,21 @@ extern "C" int mor_e8mx(const void* input, void* output, int64_t rows, int64_t c
     const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
     const int grid = grid_for(nvec > 0 ? nvec : n, 16);
     const int strategy = (int)scaling_strategy;
-    k_ws_init<<<1, WG, 0, st>>>(ws, nullptr, 0, 0);
-    if (strategy == 1) k_global_amax<<<grid, WG, 0, st>>>(in16, ws, n, nvec);
-#define E8MX(MB) do { if (emu) k_e8mx<MB, true><<<grid, WG, 0, st>>>(in16, out16, ws, strategy, n, nvec); \
-                      else k_e8mx<MB, false><<<grid, WG, 0, st>>>(in16, out16, ws, strategy, n, nvec); } while (0)
+    int npart = 0;
+    if (strategy == 1) {
+        if (nvec > 0 && nvec * 8 == n) {
+            npart = (int)std::min<int64_t>(cdiv(nvec, 8 * WG), 1024);
+            k_bs_amax_flat<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, nullptr, nvec, 1, 0);
+        } else {
+            npart = (int)std::min<int64_t>(cdiv(n, WG), 1024);
+            k_amax_scalar<<<npart, WG, 0, st>>>(in16, ws, n);
+        }
+    }
+#define E8MX(MB) do { \
+        if (strategy != 1) { if (emu) k_e8mx<MB, true, true><<<grid, WG, 0, st>>>(in16, out16, ws, npart, strategy, n, nvec); \
+                             else k_e8mx<MB, false, true><<<grid, WG, 0, st>>>(in16, out16, ws, npart, strategy, n, nvec); } \
+        else { if (emu) k_e8mx<MB, true, false><<<grid, WG, 0, st>>>(in16, out16, ws, npart, strategy, n, nvec); \
+               else k_e8mx<MB, false, false><<<grid, WG, 0, st>>>(in16, out16, ws, npart, strategy, n, nvec); } } while (0)
     if (quantize_type == 1) E8MX(1); else if (quantize_type == 2) E8MX(2); else E8MX(3);
 #undef E8MX
     return check_launch("mor_e8mx");
