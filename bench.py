@@ -77,6 +77,22 @@ class Launcher:
         self.cabi.check(self.L.mor_block_format(x.data_ptr(), out.data_ptr(), r, c, br, bc, fmt, sf, 0, self.stream()))
 
 
+    def scaling_state(self, rows, cols, br, bc, channel):
+        """Scalar outputs and the workspace of one mor_block_scaling call (allocated once, outside the timed region)."""
+        t = self.torch
+        op = self.cabi.OP_CHANNEL_SCALING if channel else self.cabi.OP_BLOCK_SCALING
+        nbytes = self.L.mor_workspace_bytes(op, rows, cols, br, bc)
+        return {"meta": t.empty(1, dtype=t.int32, device="cuda"), "amax": t.empty(1, dtype=t.float32, device="cuda"),
+                "nnz": t.empty(1, dtype=t.int32, device="cuda"), "err": t.empty(1, dtype=t.float32, device="cuda"),
+                "ws": t.empty(max(nbytes, 4), dtype=t.uint8, device="cuda"), "nbytes": nbytes, "channel": int(channel)}
+
+    def block_scaling(self, x, out, st, br, bc, thr, ss_mode):
+        r, c = x.shape
+        self.cabi.check(self.L.mor_block_scaling(x.data_ptr(), out.data_ptr(), st["meta"].data_ptr(), st["amax"].data_ptr(),
+                                                 st["nnz"].data_ptr(), st["err"].data_ptr(), r, c, br, bc, float(thr), ss_mode,
+                                                 st["channel"], st["ws"].data_ptr(), st["nbytes"], 0, self.stream()))
+
+
 def time_launches(torch, fn, steps, warmup):
     """-> (mean ms per launch from one pair of HIP events around `steps` back-to-back launches, wall ms per launch)"""
     for _ in range(warmup):
@@ -213,6 +229,9 @@ def other_configs(torch, run, cabi, K, W):
     m1 = torch.empty((32, 32), dtype=torch.int32, device="cuda")
     scale = float(448.0 / x1.float().abs().max().item())
     add("c1_per_tensor_e4m3_4096x4096", lambda: run.fake_quantize(x1, o1, m1, 128, 128, scale, 4, 1), x1.numel() * 4, x1.numel())
+    # C1 with the tensor amax found on the GPU: block-scaling op, ss_mode 4 (two reads + one write: 6 B/element)
+    st1 = run.scaling_state(4096, 4096, 128, 128, False)
+    add("c1_per_tensor_e4m3_4096x4096_gpu_amax_ss4", lambda: run.block_scaling(x1, o1, st1, 128, 128, 0.045, 4), x1.numel() * 6, x1.numel())
     del x, out, x1, o1
     # C3: per-row fp32 scale, 16384x4096
     g = torch.Generator(device="cuda").manual_seed(1003)
@@ -225,6 +244,8 @@ def other_configs(torch, run, cabi, K, W):
     mw = torch.empty((16384, 1), dtype=torch.int32, device="cuda")
     add("c3_per_row_e4m3_16384x4096", lambda: run.fake_quantize(w, ow, mw, 1, 4096, 0.0, 2, 1), w.numel() * 4 + 16384 * 4, w.numel())
     add("c3_per_row_e5m2_16384x4096", lambda: run.fake_quantize(w, ow, mw, 1, 4096, 0.0, 3, 1), w.numel() * 4 + 16384 * 4, w.numel())
+    st3 = run.scaling_state(16384, 4096, 1, 4096, True)
+    add("c3_per_row_e4m3_16384x4096_channel_op_ss3", lambda: run.block_scaling(w, ow, st3, 1, 4096, 0.045, 3), w.numel() * 6, w.numel())
     del w, ow
     # C4: MoR 128x128 on the 16384x14336 mixture
     x4 = gen_c4_gpu(torch, 16384, 14336)
@@ -234,6 +255,8 @@ def other_configs(torch, run, cabi, K, W):
     torch.cuda.synchronize()
     hist = torch.bincount(m4.flatten(), minlength=13).tolist()
     res["c4_mor_128x128_16384x14336_mixture"]["meta_histogram"] = {str(i): h for i, h in enumerate(hist) if h}
+    del x4, o4
+    res["c5_llama3_8b_layer"] = c5_sweep(torch, run, max(3, K // 4), 2)
     # launch overhead: a 1x32 tensor
     xs = torch.randn(1, 32, device="cuda").to(torch.bfloat16)
     os_ = torch.empty_like(xs)
@@ -241,6 +264,70 @@ def other_configs(torch, run, cabi, K, W):
     ms, wall = time_launches(torch, lambda: run.fake_quantize(xs, os_, ms_, 1, 32, 0.0, 2, 2), 200, 20)
     res["tiny_1x32"] = {"us_per_call_events": round(ms * 1e3, 2), "us_per_call_wall": round(wall * 1e3, 2)}
     return res
+
+
+def c5_sweep(torch, run, K, W):
+    """Every tensor one Llama-3-8B layer quantizes in a forward + backward pass at 16384 tokens: activations and
+    output gradients N(0,1), weights N(0,0.02).  Three families: MoR 128x128, block E4M3 128x128, and per-channel
+    (row-wise for fprop / dgrad, column-wise blocks N x 1 through the channel-scaling op for wgrad).  Per family:
+    total algorithmic bytes / total kernel time; per shape: microseconds and GB/s.  Plus the ragged 4097 x 4095."""
+    T, D, KV, F = 16384, 4096, 1024, 14336
+    acts = [("x_qkv", T, D), ("attn_out", T, D), ("x_mlp", T, D), ("h_down", T, F)]
+    weights = [("wq", D, D), ("wk", KV, D), ("wv", KV, D), ("wo", D, D), ("w_gate", F, D), ("w_up", F, D), ("w_down", D, F)]
+    grads = [("dy_q", T, D), ("dy_o", T, D), ("dy_down", T, D), ("dy_k", T, KV), ("dy_v", T, KV), ("dy_gate", T, F), ("dy_up", T, F)]
+    g = torch.Generator(device="cuda").manual_seed(1005)
+    big = torch.randn(T * F, device="cuda", generator=g).to(torch.bfloat16)
+    small = (torch.randn(F * D, device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+    obuf = torch.empty_like(big)
+    mbuf = torch.empty(T * F // 32, dtype=torch.int32, device="cuda")
+    cache = {}
+
+    def timed(key, fn):
+        if key not in cache:
+            cache[key] = time_launches(torch, fn, K, W)[0]
+        return cache[key]
+
+    def view(src, r, c):
+        return src[: r * c].view(r, c)
+
+    fam = {}
+
+    def family(name, entries):
+        tot_b = tot_ms = 0.0
+        shapes = {}
+        for tname, r, c, src, kind in entries:
+            x, o = view(src, r, c), view(obuf, r, c)
+            tag = "w" if src is small else "a"
+            if kind == "mor":
+                ms = timed((tag, r, c, kind), lambda: run.fake_quantize(x, o, mbuf, 128, 128, 1e-15, 1, 1))
+                nb = r * c * 4 + (r // 128) * (c // 128) * 4
+            elif kind == "block":
+                ms = timed((tag, r, c, kind), lambda: run.fake_quantize(x, o, mbuf, 128, 128, 0.0, 2, 1))
+                nb = r * c * 4 + (r // 128) * (c // 128) * 4
+            elif kind == "row":
+                ms = timed((tag, r, c, kind), lambda: run.fake_quantize(x, o, mbuf, 1, c, 0.0, 2, 1))
+                nb = r * c * 4 + r * 4
+            else:                                   # column blocks r x 1: channel-scaling op, fp32 scale per column
+                st = run.scaling_state(r, c, r, 1, True)
+                ms = timed((tag, r, c, kind), lambda: run.block_scaling(x, o, st, r, 1, 0.045, 3))
+                nb = r * c * 6
+            tot_b += nb
+            tot_ms += ms
+            shapes[f"{r}x{c}_{tag}_{kind}"] = {"us": round(ms * 1e3, 1), "GBps": round(nb / (ms * 1e-3) / 1e9, 1)}
+        fam[name] = {"launches": len(entries), "total_ms": round(tot_ms, 4), "total_GB": round(tot_b / 1e9, 3),
+                     "GBps": round(tot_b / (tot_ms * 1e-3) / 1e9, 1), "frac": round(tot_b / (tot_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "shapes": shapes}
+
+    every = [(n, r, c, big) for n, r, c in acts + grads] + [(n, r, c, small) for n, r, c in weights]
+    family("mor_128x128", [(n, r, c, s, "mor") for n, r, c, s in every])
+    family("block_e4m3_128x128", [(n, r, c, s, "block") for n, r, c, s in every])
+    family("per_channel_rows_and_columns", [(n, r, c, s, "row") for n, r, c, s in every]
+           + [(n, r, c, big, "col") for n, r, c in acts + grads])
+    # ragged, odd column count (scalar kernel): a shape the reference rejects
+    xr, orr = view(big, 4097, 4095), view(obuf, 4097, 4095)
+    ms = time_launches(torch, lambda: run.fake_quantize(xr, orr, mbuf, 128, 128, 1e-15, 1, 1), K, W)[0]
+    fam["ragged_4097x4095_mor_128x128"] = {"us": round(ms * 1e3, 1), "GBps": round(4097 * 4095 * 4 / (ms * 1e-3) / 1e9, 1)}
+    return fam
 
 
 def cpu_baseline(torch, x_gpu):

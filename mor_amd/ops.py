@@ -195,6 +195,36 @@ _lib.impl("fake_quantize_e8mx_inplace", _e8mx_inplace_impl, "CUDA")
 
 
 # ----------------------------------------------------------------------------------------------------------------------
+# Shape / dtype propagation (fake and meta tensors), so that the ops trace under torch.compile and torch.export.  The
+# reference registers none; the output shapes are those of FQ:1852-1857, 2065-2078, 2256.
+def _fake_meta(i, block_x, block_y, dim_x, dim_y):
+    return i.new_empty((_cdiv(dim_x, block_x), _cdiv(dim_y, block_y)), dtype=torch.int32)
+
+
+def _fake_scalars(i):
+    return [i.new_empty((1,), dtype=torch.int32), i.new_empty((1,), dtype=torch.float32),
+            i.new_empty((1,), dtype=torch.int32), i.new_empty((1,), dtype=torch.float32)]
+
+
+def _fake_like(i):
+    return torch.empty_like(i, memory_format=torch.contiguous_format)
+
+
+torch.library.register_fake("mor::fake_quantize")(
+    lambda i, x, y, bx, by, c, m, s: [_fake_like(i), _fake_meta(i, bx, by, x, y)])
+torch.library.register_fake("mor::fake_quantize_no_alloc")(
+    lambda i, x, y, bx, by, c, m, s, result: _fake_meta(i, bx, by, x, y))
+for _name in ("fake_quantize_block_scaling", "fake_quantize_channel_scaling"):
+    torch.library.register_fake(f"mor::{_name}")(lambda i, x, y, bx, by, t, s: [_fake_like(i)] + _fake_scalars(i))
+    torch.library.register_fake(f"mor::{_name}_inplace")(lambda i, x, y, bx, by, t, s: _fake_scalars(i))
+torch.library.register_fake("mor::fake_quantize_e8mx")(lambda i, x, y, bx, by, q, s: _fake_like(i))
+torch.library.register_fake("mor::fake_quantize_e8mx_inplace")(lambda i, x, y, bx, by, q, s, result: None)
+for _name in ("quant_dequant_e4m3", "quant_dequant_e5m2", "quant_dequant_e3m2", "quant_dequant_e2m3",
+              "e4m3_with_e8_scale_rne", "e4m3_with_e8_scale_rz"):
+    torch.library.register_fake(f"mor::{_name}")(lambda i, x, y, bx, by: _fake_like(i))
+
+
+# ----------------------------------------------------------------------------------------------------------------------
 # Python API and straight-through autograd: mor/ops.py:11-156
 def _noop_setup_context(ctx, inputs, output):
     pass

@@ -219,3 +219,53 @@ def test_errors_and_autograd(mor):
     o1, _ = mor.ops.fake_quantize(t, 256, 256, 128, 128, 1e-15, 1, 1)
     o2, _ = mor.ops.fake_quantize(t.contiguous(), 256, 256, 128, 128, 1e-15, 1, 1)
     assert o1.equal(o2)
+
+
+def test_ops_replay_in_a_hip_graph(mor):
+    """The library allocates nothing and clears its workspace with kernels, so the ops can be captured: every replay,
+    with eager work and synchronizations between replays and fresh input each time, equals the eager result."""
+    x = torch.empty(512, 1024, dtype=torch.bfloat16, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(7)
+
+    def body(t):
+        o1, m1 = mor.ops.fake_quantize(t, 512, 1024, 128, 128, clamp_threshold=1e-15, mode=1, sf_type=1)
+        o2, m2 = mor.ops.fake_quantize(t, 512, 1024, 1, 32, clamp_threshold=0.0, mode=2, sf_type=2)
+        r = mor.ops.fake_quantize_channel_scaling(t, 512, 1024, 512, 1, e4m3_threshold=0.045, ss_mode=1)
+        e = mor.ops.fake_quantize_e8mx(t, 512, 1024, 128, 128, quantize_type=2, scaling_strategy=1)
+        return [o1, m1, o2, m2, e] + list(r)
+
+    x.copy_(torch.randn(512, 1024, device="cuda", generator=g))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        body(x)                                            # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = body(x)
+    for rep in range(4):
+        x.copy_(torch.randn(512, 1024, device="cuda", generator=g) * (10.0 ** rep))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = body(x)                                     # eager work between the replays
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), rep
+
+
+def test_ops_trace_under_torch_compile(mor):
+    """aot_eager traces forward and backward through the fake kernels and the straight-through autograd."""
+    def f(t):
+        q = mor.ops.fake_quantize(t * 1.0, 256, 512, 128, 128, 1e-15, 1, 1)[0]
+        return mor.ops.fake_quantize_e8mx(q, 256, 512, 128, 128, 3, 1).float().sum()
+
+    w = torch.randn(256, 512, device="cuda").to(torch.bfloat16).requires_grad_(True)
+    want = f(w)
+    want.backward()
+    g_eager = w.grad.clone()
+    w.grad = None
+    got = torch.compile(f, backend="aot_eager", fullgraph=True)(w)
+    got.backward()
+    assert torch.equal(got, want) and torch.equal(w.grad, g_eager) and torch.all(g_eager == 1)

@@ -60,3 +60,31 @@ def test_cpu_tensors_are_rejected_as_in_the_reference():
     x = torch.zeros(4, 8, dtype=torch.bfloat16)
     with pytest.raises((NotImplementedError, RuntimeError)):
         mor.ops.fake_quantize(x, 4, 8, 4, 8, 0.0, 2, 1)
+
+
+def test_fake_tensor_shapes_without_a_gpu():
+    """Shape propagation (what torch.compile / export trace through) needs no device: meta and fake tensors."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    x = torch.empty(300, 520, dtype=torch.bfloat16, device="meta")
+    out, meta = mor.ops.fake_quantize(x, 300, 520, 128, 128, clamp_threshold=1e-15, mode=1, sf_type=1)
+    assert out.shape == x.shape and out.dtype == torch.bfloat16
+    assert meta.shape == (3, 5) and meta.dtype == torch.int32
+    assert mor.ops.fake_quantize_no_alloc(x, 300, 520, 1, 32, 0.0, 2, 2, output=x).shape == (300, 17)
+    for op in (mor.ops.fake_quantize_block_scaling, mor.ops.fake_quantize_channel_scaling):
+        res = op(x, 300, 520, 1, 520, e4m3_threshold=0.045, ss_mode=3)
+        assert [tuple(t.shape) for t in res] == [(300, 520), (1,), (1,), (1,), (1,)]
+        assert [t.dtype for t in res] == [torch.bfloat16, torch.int32, torch.float32, torch.int32, torch.float32]
+    for op in (mor.ops.fake_quantize_block_scaling_inplace, mor.ops.fake_quantize_channel_scaling_inplace):
+        res = op(x, 300, 520, 1, 520, 0.045, 3)
+        assert [t.dtype for t in res] == [torch.int32, torch.float32, torch.int32, torch.float32]
+    assert mor.ops.fake_quantize_e8mx(x, 300, 520, 128, 128, quantize_type=2, scaling_strategy=1).shape == x.shape
+    assert mor.ops.fake_quantize_e8mx_inplace(x, 300, 520, 128, 128, 2, 1, x) is None
+    f = torch.empty(16, 32, dtype=torch.float32, device="meta")
+    for name in ("quant_dequant_e4m3", "quant_dequant_e5m2", "quant_dequant_e2m3", "quant_dequant_e3m2",
+                 "e4m3_with_e8_scale_rne", "e4m3_with_e8_scale_rz"):
+        r = getattr(mor.ops, name)(f, 16, 32, 16, 32)
+        assert r.shape == f.shape and r.dtype == torch.float32
+    with FakeTensorMode():
+        y = torch.empty(256, 256, dtype=torch.bfloat16, device="cuda")
+        out, meta = mor.ops.fake_quantize(y, 256, 256, 128, 128, 1e-15, 1, 1)
+        assert out.device.type == "cuda" and meta.shape == (2, 2)
