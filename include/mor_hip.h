@@ -128,6 +128,38 @@ int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t block_r
  */
 int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
 
+/*
+ * MX wire format: the quantized tensor itself instead of its dequantized bf16 image.
+ *
+ * No counterpart in the reference, whose ops all return bf16 (FQ:1839-1871).  For blocks of 32
+ * elements these entries emit what its MX block quantization (block modes with sf_type 2,
+ * FQ:801-823; E2M3 branch FQ:758-770) computes between "quantize" and "dequantize":
+ *   e8      = exponent field of fl32(fmax / amax) - 127 (FQ:251-252), limited to [-127, 127]
+ *   code    = cast(x * 2^e8) in the element format, nearest even, sign of x kept
+ *   scale   = one byte per block, 127 - e8: the E8M0 encoding of the multiplier 2^-e8
+ * so that decode(code) * 2^(scale - 127) equals the tensor mor_fake_quantize / mor_block_format
+ * return with MOR_FLAG_TORCH_EMULATION for 1 x 32 blocks and sf_type 2.  A zero block has scale
+ * byte 127.  FP8 payload: one byte per element (OCP E4M3 / E5M2 encodings).  FP6 payload (E2M3 /
+ * E3M2): 32 codes packed little-endian into 24 bytes, element i in bits [6i, 6i + 6) of its block.
+ * cols must be a multiple of 32; tensors and payloads 16-byte aligned, scales 4-byte aligned.
+ */
+size_t mor_mx_payload_bytes(int64_t rows, int64_t cols, int fmt);
+
+/* Blocks of 32 along rows.  payload: [rows, cols * bits / 8] bytes, scales: [rows, cols / 32]. */
+int mor_mx_quantize(const void* input, void* payload, void* scales, int64_t rows, int64_t cols,
+                    int fmt, void* stream);
+
+/* Both orientations from one read of the tensor (rows and cols multiples of 32): the row-wise
+ * result as above and the column-wise one (blocks of 32 along columns) stored transposed, i.e. what
+ * mor_mx_quantize returns for the transposed tensor: col_payload [cols, rows * bits / 8],
+ * col_scales [cols, rows / 32].  This is the pair a linear layer needs for dgrad and wgrad. */
+int mor_mx_quantize_dual(const void* input, void* row_payload, void* row_scales, void* col_payload,
+                         void* col_scales, int64_t rows, int64_t cols, int fmt, void* stream);
+
+/* payload + scales -> bf16 [rows, cols] (blocks of 32 along rows). */
+int mor_mx_dequantize(const void* payload, const void* scales, void* output, int64_t rows,
+                      int64_t cols, int fmt, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

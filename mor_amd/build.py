@@ -3,7 +3,7 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = [os.path.join(_HERE, "csrc", "mor_kernels.hip")]
+SOURCES = [os.path.join(_HERE, "csrc", "mor_kernels.hip"), os.path.join(_HERE, "csrc", "mor_wire.hip")]
 OUT = os.path.join(_HERE, "lib", "libmor_hip.so")
 
 HIPCC_FLAGS = [

@@ -19,6 +19,7 @@
 #include <algorithm>
 
 #include "mor_device.h"
+#include "mor_host.h"
 #include "../../include/mor_hip.h"
 
 namespace mor {
@@ -622,7 +623,7 @@ using namespace mor;
 
 static thread_local char g_err[512] = "";
 
-static int fail(int code, const char* fmt, ...) {
+int mor_fail(int code, const char* fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof g_err, fmt, ap);
@@ -630,9 +631,9 @@ static int fail(int code, const char* fmt, ...) {
     return code;
 }
 
-static int check_launch(const char* what) {
+int mor_check_launch(const char* what) {
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fail(MOR_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    if (e != hipSuccess) return mor_fail(MOR_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
     return MOR_OK;
 }
 
@@ -653,10 +654,10 @@ extern "C" const char* mor_last_error(void) { return g_err; }
 extern "C" const char* mor_version(void) { return "mor_hip 0.1 (gfx950)"; }
 
 static int validate_shape(const void* input, int64_t rows, int64_t cols, int64_t brows, int64_t bcols) {
-    if (!input) return fail(MOR_ERR_INVALID_ARGUMENT, "input is NULL");
-    if (rows <= 0 || cols <= 0) return fail(MOR_ERR_INVALID_ARGUMENT, "rows and cols must be positive (got %lld x %lld)", (long long)rows, (long long)cols);
-    if (brows <= 0 || bcols <= 0) return fail(MOR_ERR_INVALID_ARGUMENT, "block dims must be positive (got %lld x %lld)", (long long)brows, (long long)bcols);
-    if (cdiv(rows, brows) * cdiv(cols, bcols) > 0x7FFFFFFFll) return fail(MOR_ERR_INVALID_ARGUMENT, "too many blocks");
+    if (!input) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "input is NULL");
+    if (rows <= 0 || cols <= 0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "rows and cols must be positive (got %lld x %lld)", (long long)rows, (long long)cols);
+    if (brows <= 0 || bcols <= 0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "block dims must be positive (got %lld x %lld)", (long long)brows, (long long)bcols);
+    if (cdiv(rows, brows) * cdiv(cols, bcols) > 0x7FFFFFFFll) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many blocks");
     return MOR_OK;
 }
 
@@ -751,7 +752,7 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
             if (emu) k_elementwise_exact<true><<<grid, WG, 0, st>>>(in16, out16, meta, n, nblocks, qa.fmt, e8, qa.clamp, qa.meta_val);
             else k_elementwise_exact<false><<<grid, WG, 0, st>>>(in16, out16, meta, n, nblocks, qa.fmt, e8, qa.clamp, qa.meta_val);
         }
-        return check_launch("k_elementwise");
+        return mor_check_launch("k_elementwise");
     }
     const bool vec_ok = fast_ok && aligned16(input) && (!output || aligned16(output)) && cols % 8 == 0 && bcols % 8 == 0
                         && brows * (cols / 8) < 0x7FFFFFFFll;
@@ -759,7 +760,7 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
     if (qa.qmode == 2 && !stats && output && vec_ok && brows == 1 && cols % bcols == 0 && is_pow2(G) && G <= 64) {
         if (e8) launch_rowgroup<true>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
         else launch_rowgroup<false>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
-        return check_launch("k_rowgroup");
+        return mor_check_launch("k_rowgroup");
     }
     if (vec_ok && brows * (bcols / 8) <= 8 * WG) {
         if (qa.qmode == 1) {
@@ -769,11 +770,11 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
             if (e8) launch_wgblock<false, true>(input, output, meta, stats, sh, qa, st);
             else launch_wgblock<false, false>(input, output, meta, stats, sh, qa, st);
         }
-        return check_launch("k_wgblock");
+        return mor_check_launch("k_wgblock");
     }
     if (emu) k_generic<true><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, e8 ? 1 : 0);
     else k_generic<false><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, e8 ? 1 : 0);
-    return check_launch("k_generic");
+    return mor_check_launch("k_generic");
 }
 
 extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
@@ -781,7 +782,7 @@ extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
                                  double clamp_threshold, int64_t mode, int64_t sf_type,
                                  uint32_t flags, void* stream) {
     if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
-    if (!output || !meta) return fail(MOR_ERR_INVALID_ARGUMENT, "output / meta is NULL");
+    if (!output || !meta) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output / meta is NULL");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int qmode = (int)(mode % 10);                 // FQ:1774
     QuantArgs qa{};
@@ -804,7 +805,7 @@ extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
                 else k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(static_cast<const uint16_t*>(input), static_cast<uint16_t*>(output), n, nvec);
             }
             k_fill_i32<<<grid_for(nblocks), WG, 0, st>>>(meta, nblocks, 3);
-            return check_launch("k_copy / k_fill_i32");
+            return mor_check_launch("k_copy / k_fill_i32");
         }
     }
     return run_quantize(input, output, meta, nullptr, rows, cols, brows, bcols, qa, e8, flags, st);
@@ -814,8 +815,8 @@ extern "C" int mor_block_format(const void* input, void* output,
                                 int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
                                 int fmt, int64_t sf_type, uint32_t flags, void* stream) {
     if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
-    if (!output) return fail(MOR_ERR_INVALID_ARGUMENT, "output is NULL");
-    if (fmt < 0 || fmt > 3) return fail(MOR_ERR_INVALID_ARGUMENT, "unknown format %d", fmt);
+    if (!output) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output is NULL");
+    if (fmt < 0 || fmt > 3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "unknown format %d", fmt);
     QuantArgs qa{};
     qa.qmode = 2; qa.fmt = fmt; qa.meta_val = -1;
     return run_quantize(input, output, nullptr, nullptr, rows, cols, brows, bcols, qa, sf_type == 2, flags, static_cast<hipStream_t>(stream));
@@ -824,7 +825,7 @@ extern "C" int mor_block_format(const void* input, void* output,
 extern "C" int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
                              double clamp_threshold, int64_t mode, int64_t sf_type, float* stats, void* stream) {
     if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
-    if (!stats) return fail(MOR_ERR_INVALID_ARGUMENT, "stats is NULL");
+    if (!stats) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "stats is NULL");
     QuantArgs qa{};
     qa.qmode = 1; qa.fmt = -1; qa.meta_val = -1;
     qa.clamp = (float)clamp_threshold;
@@ -835,33 +836,33 @@ extern "C" int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int6
 extern "C" int mor_block_stats(const void* input, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
                                float fmax, float* amax, float* scale, int32_t* e8m0, void* stream) {
     if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
-    if (!amax || !scale || !e8m0) return fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
+    if (!amax || !scale || !e8m0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
     Shape sh{rows, cols, brows, bcols, cdiv(rows, brows), cdiv(cols, bcols)};
     k_block_stats<<<(int)(sh.gy * sh.gx), WG, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const uint16_t*>(input), sh, fmax, amax, scale, e8m0);
-    return check_launch("k_block_stats");
+    return mor_check_launch("k_block_stats");
 }
 
 extern "C" int mor_quant_dequant(const float* input, float* output, int64_t n, int fmt, void* stream) {
-    if (!input || !output || n < 0) return fail(MOR_ERR_INVALID_ARGUMENT, "bad pointer or size");
-    if (fmt < 0 || fmt > 3) return fail(MOR_ERR_INVALID_ARGUMENT, "unknown format %d", fmt);
+    if (!input || !output || n < 0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "bad pointer or size");
+    if (fmt < 0 || fmt > 3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "unknown format %d", fmt);
     if (n == 0) return MOR_OK;
     k_quant_dequant<<<grid_for(n, 16), WG, 0, static_cast<hipStream_t>(stream)>>>(input, output, n, fmt);
-    return check_launch("k_quant_dequant");
+    return mor_check_launch("k_quant_dequant");
 }
 
 extern "C" int mor_e4m3_with_e8_scale(const float* input, float* output, int64_t n, int rne, void* stream) {
-    if (!input || !output || n < 0) return fail(MOR_ERR_INVALID_ARGUMENT, "bad pointer or size");
+    if (!input || !output || n < 0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "bad pointer or size");
     if (n == 0) return MOR_OK;
     k_e4m3_e8_scale<<<grid_for(n, 16), WG, 0, static_cast<hipStream_t>(stream)>>>(input, output, n, rne);
-    return check_launch("k_e4m3_e8_scale");
+    return mor_check_launch("k_e4m3_e8_scale");
 }
 
 extern "C" int mor_selftest_hw_cast(uint64_t* mismatches, void* stream) {
-    if (!mismatches) return fail(MOR_ERR_INVALID_ARGUMENT, "mismatches is NULL");
+    if (!mismatches) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mismatches is NULL");
     hipStream_t st = static_cast<hipStream_t>(stream);
     k_fill_i32<<<1, WG, 0, st>>>(reinterpret_cast<int32_t*>(mismatches), 4, 0);
     k_selftest_hw_cast<<<256 * 16, WG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
-    return check_launch("k_selftest_hw_cast");
+    return mor_check_launch("k_selftest_hw_cast");
 }
 
 
@@ -1491,15 +1492,15 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
                                  double e4m3_threshold, int64_t ss_mode, int channel,
                                  void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
     if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
-    if (!output || !meta || !global_amax || !global_non_zero || !global_error) return fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
+    if (!output || !meta || !global_amax || !global_non_zero || !global_error) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
     if (rows % brows != 0 || cols % bcols != 0)      // FQ:2019-2020, 2437-2438
-        return fail(MOR_ERR_INVALID_ARGUMENT, "block dims %lld x %lld do not divide the tensor %lld x %lld", (long long)brows, (long long)bcols, (long long)rows, (long long)cols);
-    if (ss_mode < 1 || ss_mode > 4) return fail(MOR_ERR_INVALID_ARGUMENT, "ss_mode must be 1..4 (got %lld)", (long long)ss_mode);
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "block dims %lld x %lld do not divide the tensor %lld x %lld", (long long)brows, (long long)bcols, (long long)rows, (long long)cols);
+    if (ss_mode < 1 || ss_mode > 4) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "ss_mode must be 1..4 (got %lld)", (long long)ss_mode);
     if (channel && brows != 1 && bcols != 1)         // FQ:2501
-        return fail(MOR_ERR_INVALID_ARGUMENT, "channel scaling needs block_rows == 1 or block_cols == 1");
-    if (rows * cols >= (1ll << 34)) return fail(MOR_ERR_INVALID_ARGUMENT, "tensor too large");
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "channel scaling needs block_rows == 1 or block_cols == 1");
+    if (rows * cols >= (1ll << 34)) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor too large");
     const size_t need = mor_workspace_bytes(MOR_OP_BLOCK_SCALING, rows, cols, brows, bcols);
-    if (!workspace || workspace_bytes < need) return fail(MOR_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    if (!workspace || workspace_bytes < need) return mor_fail(MOR_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
     Shape sh{rows, cols, brows, bcols, rows / brows, cols / bcols};
@@ -1520,7 +1521,7 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
         const int rows_per_wg = (int)std::min<int64_t>(brows, 256);
         const unsigned gx = (unsigned)cdiv(cols, 256);
         const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
-        if ((int64_t)gx > MAX_PARTIALS) return fail(MOR_ERR_INVALID_ARGUMENT, "too many columns (%lld)", (long long)cols);
+        if ((int64_t)gx > MAX_PARTIALS) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many columns (%lld)", (long long)cols);
         const unsigned gy = (unsigned)std::min<int64_t>(segs, std::max<int64_t>(MAX_PARTIALS / gx, 1));
         npart = (int)(gx * gy);
         k_bs_amax_col<<<dim3(gx, gy), WG, 0, st>>>(in16, ws, blocks, sh, rows_per_wg, vec);
@@ -1564,17 +1565,17 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
         const int64_t nvec = vec ? n / 8 : 0;
         k_copy_if<<<grid_for(nvec > 0 ? nvec : n, 16), WG, 0, st>>>(in16, out16, meta, 3, n, nvec);
     }
-    return check_launch("mor_block_scaling");
+    return mor_check_launch("mor_block_scaling");
 }
 
 extern "C" int mor_e8mx(const void* input, void* output, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
                         int64_t quantize_type, int64_t scaling_strategy, void* workspace, size_t workspace_bytes,
                         uint32_t flags, void* stream) {
     if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
-    if (!output) return fail(MOR_ERR_INVALID_ARGUMENT, "output is NULL");
-    if (quantize_type < 1 || quantize_type > 3) return fail(MOR_ERR_INVALID_ARGUMENT, "quantize_type must be 1..3 (got %lld)", (long long)quantize_type);
+    if (!output) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output is NULL");
+    if (quantize_type < 1 || quantize_type > 3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "quantize_type must be 1..3 (got %lld)", (long long)quantize_type);
     const size_t need = mor_workspace_bytes(MOR_OP_E8MX, rows, cols, brows, bcols);
-    if (!workspace || workspace_bytes < need) return fail(MOR_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    if (!workspace || workspace_bytes < need) return mor_fail(MOR_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
     uint32_t* ws = static_cast<uint32_t*>(workspace);
@@ -1601,5 +1602,5 @@ extern "C" int mor_e8mx(const void* input, void* output, int64_t rows, int64_t c
                else k_e8mx<MB, false, false><<<grid, WG, 0, st>>>(in16, out16, ws, npart, strategy, n, nvec); } } while (0)
     if (quantize_type == 1) E8MX(1); else if (quantize_type == 2) E8MX(2); else E8MX(3);
 #undef E8MX
-    return check_launch("mor_e8mx");
+    return mor_check_launch("mor_e8mx");
 }

@@ -1,0 +1,311 @@
+// MX wire format for MI355X (gfx950): element codes + one E8M0 scale byte per 32 elements.
+//
+// The reference ("FQ" = mor/csrc/cuda/fake_quantize.cu) only returns the dequantized bf16 tensor.  These kernels
+// emit what its MX block quantization (block modes with SF_E8, FQ:801-823, E2M3 branch FQ:758-770) holds between
+// "quantize" and "dequantize": per block of 32 elements, e8 = exponent field of fl32(fmax / amax) - 127 (FQ:251-252),
+// code = cast(x * 2^e8), scale byte = 127 - e8 (the E8M0 encoding of the multiplier 2^-e8 that decodes the block).
+//   k_mx_quantize    blocks along rows: a lane owns 8 elements, 4 lanes a block (amax by DPP), 8 or 6 bytes per lane
+//   k_mx_dual        one read of a 128 x 128 tile gives both orientations: blocks along rows from registers, blocks
+//                    along columns through an LDS copy of the tile, written transposed ([cols, rows] payload) so that
+//                    the reduction dimension of a weight-gradient GEMM is contiguous
+//   k_mx_dequantize  payload + scales -> bf16
+// FP8 codes come from the gfx950 converts; FP6 codes (E2M3 / E3M2) are computed in integer arithmetic and packed
+// little-endian, 32 codes in 24 bytes.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <algorithm>
+
+#include "mor_device.h"
+#include "mor_host.h"
+#include "../../include/mor_hip.h"
+
+namespace mor {
+
+constexpr int WWG = 256;
+
+template <int F> struct Wire {
+    static constexpr int bits = Fmt<F>::hw ? 8 : 6;
+    static constexpr int bias = (F == FMT_E4M3) ? 7 : (F == FMT_E5M2) ? 15 : (F == FMT_E3M2) ? 3 : 1;
+};
+
+// Exponent of the block scale, limited to the finite E8M0 range.  The integer form needs a normal amax; the
+// division covers subnormal amax and the far ends of the exponent range.
+template <int F> __device__ __forceinline__ int wire_e8(float amax) {
+    if (!(amax > 0.0f)) return 0;
+    const Scale sc = make_scale_e8<F>(amax);
+    int e8 = sc.e8;
+    if (!sc.fast) e8 = (int)((f2u(Fmt<F>::fmax / amax) >> 23) & 0xFF) - 127;
+    return min(max(e8, -127), 127);
+}
+
+// 6-bit code (without sign) of a non-negative value on the grid of F
+template <int F> __device__ __forceinline__ uint32_t fp6_code(float r) {
+    constexpr int mb = Fmt<F>::mbits, bias = Wire<F>::bias;
+    const uint32_t b = f2u(r);
+    const int e = (int)(b >> 23) - 127;
+    const uint32_t normal = ((uint32_t)(e + bias) << mb) | ((b >> (23 - mb)) & ((1u << mb) - 1u));
+    const uint32_t sub = (uint32_t)(r * (float)(1 << (mb + bias - 1)));
+    return (e < 1 - bias) ? sub : normal;
+}
+
+template <int F> __device__ __forceinline__ float fp6_value(uint32_t mag) {
+    constexpr int mb = Fmt<F>::mbits, bias = Wire<F>::bias;
+    const uint32_t e = mag >> mb, m = mag & ((1u << mb) - 1u);
+    const float sub = (float)m * (1.0f / (float)(1 << (mb + bias - 1)));
+    const float normal = u2f(((e + 127u - bias) << 23) | (m << (23 - mb)));
+    return e == 0 ? sub : normal;
+}
+
+// codes of the two elements of a packed word, in bits 0..bits-1 and bits..2*bits-1
+template <int F> __device__ __forceinline__ uint32_t code_pair(uint32_t w, int e8) {
+    if constexpr (Fmt<F>::hw) {
+        return hw_pack2<F>(ldexpf(bf16_lo(w), e8), ldexpf(bf16_hi(w), e8)) & 0xFFFFu;
+    } else {
+        const uint32_t a = fp6_code<F>(round_mag_sat<F>(ldexpf(fabsf(bf16_lo(w)), e8))) | ((w >> 10) & 0x20u);
+        const uint32_t b = fp6_code<F>(round_mag_sat<F>(ldexpf(fabsf(bf16_hi(w)), e8))) | ((w >> 26) & 0x20u);
+        return a | (b << 6);
+    }
+}
+
+// the 8 codes of a 16-byte chunk: 64 bits (FP8) or 48 bits (FP6)
+template <int F> __device__ __forceinline__ uint64_t code_chunk(uint4 v, int e8) {
+    constexpr int pb = 2 * Wire<F>::bits;
+    return (uint64_t)code_pair<F>(v.x, e8) | ((uint64_t)code_pair<F>(v.y, e8) << pb) |
+           ((uint64_t)code_pair<F>(v.z, e8) << (2 * pb)) | ((uint64_t)code_pair<F>(v.w, e8) << (3 * pb));
+}
+
+__device__ __forceinline__ float chunk_amax(uint4 v) {
+    float amax = 0.0f;
+    acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
+    return amax;
+}
+
+// Stores the codes of one chunk.  `c` is the chunk's index in the payload's own row-major order (4 chunks = 1 block).
+// FP8: 8 bytes per lane.  FP6: the 4 lanes of a block hold 4 x 48 bits = 24 bytes; lanes 0..2 store 8 bytes each,
+// built from their own bits and the next lane's.
+template <int F> __device__ __forceinline__ void store_codes(uint8_t* payload, int64_t c, uint64_t codes, bool ok) {
+    if constexpr (Fmt<F>::hw) {
+        if (ok) *reinterpret_cast<uint2*>(payload + c * 8) = make_uint2((uint32_t)codes, (uint32_t)(codes >> 32));
+    } else {
+        constexpr int NEXT = 0xF9;                               // quad_perm [1,2,3,3]: lane i reads lane i + 1
+        const uint32_t nlo = dpp_u<NEXT>((uint32_t)codes), nhi = dpp_u<NEXT>((uint32_t)(codes >> 32));
+        const uint64_t next = (uint64_t)nlo | ((uint64_t)nhi << 32);
+        const int j = (int)(c & 3);
+        const uint64_t word = (codes >> (16 * j)) | (next << (48 - 16 * j));
+        if (ok && j < 3) *reinterpret_cast<uint2*>(payload + (c >> 2) * 24 + j * 8) = make_uint2((uint32_t)word, (uint32_t)(word >> 32));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// blocks of 32 along rows; the tensor is a flat array of 16-byte chunks (cols % 32 == 0)
+template <int F, int NV>
+__global__ __launch_bounds__(WWG) void k_mx_quantize(const uint4* in, uint8_t* payload, uint8_t* scales, int64_t nchunks) {
+    const int64_t base = (int64_t)blockIdx.x * (NV * WWG) + threadIdx.x;
+    uint4 v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int64_t c = base + k * WWG;
+        v[k] = make_uint4(0, 0, 0, 0);
+        if (c < nchunks) v[k] = in[c];
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int64_t c = base + k * WWG;
+        const float amax = group_max_t<4>(chunk_amax(v[k]), 4);
+        const int e8 = wire_e8<F>(amax);
+        store_codes<F>(payload, c, code_chunk<F>(v[k], e8), c < nchunks);
+        // the scale bytes of 4 consecutive blocks (16 lanes) leave as one 32-bit store
+        const uint32_t sb = (uint32_t)(127 - e8);
+        const uint32_t s4 = sb | (__shfl_down(sb, 4, 16) << 8) | (__shfl_down(sb, 8, 16) << 16) | (__shfl_down(sb, 12, 16) << 24);
+        if (c < nchunks && (c & 15) == 0) {
+            if (c + 16 <= nchunks) *reinterpret_cast<uint32_t*>(scales + (c >> 2)) = s4;
+            else
+                for (int64_t b = 0; b < ((nchunks - c) >> 2); ++b) scales[(c >> 2) + b] = (uint8_t)(s4 >> (8 * b));
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// both orientations from one read.  Tile 128 x 128; rows % 32 == 0 and cols % 32 == 0.
+constexpr int TILE = 128;
+constexpr int LDS_PITCH = TILE + 8;              // in bf16 elements; keeps 16-byte alignment of the row starts
+
+template <int F>
+__global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_payload, uint8_t* row_scales,
+                                                 uint8_t* col_payload, uint8_t* col_scales, int64_t rows, int64_t cols) {
+    __shared__ __attribute__((aligned(16))) uint16_t tile[TILE * LDS_PITCH];
+    const int tid = threadIdx.x;
+    const int64_t tiles_x = (cols + TILE - 1) / TILE;
+    const int64_t ty = blockIdx.x / tiles_x, tx = blockIdx.x - ty * tiles_x;
+    const int64_t R0 = ty * TILE, C0 = tx * TILE;
+    const int rows_valid = (int)min((int64_t)TILE, rows - R0), cols_valid = (int)min((int64_t)TILE, cols - C0);
+    const int64_t row_chunks = cols >> 3;
+
+    // phase A: blocks along rows, from registers
+    uint4 v[8];
+    bool ok[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+        ok[k] = (r < rows_valid) && (cc * 8 < cols_valid);
+        v[k] = make_uint4(0, 0, 0, 0);
+        if (ok[k]) v[k] = in[(R0 + r) * row_chunks + (C0 >> 3) + cc];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+        *reinterpret_cast<uint4*>(&tile[r * LDS_PITCH + cc * 8]) = v[k];
+        const float amax = group_max_t<4>(chunk_amax(v[k]), 4);
+        const int e8 = wire_e8<F>(amax);
+        const int64_t c = (R0 + r) * row_chunks + (C0 >> 3) + cc;          // chunk index in the row-major payload
+        store_codes<F>(row_payload, c, code_chunk<F>(v[k], e8), ok[k]);
+        if (ok[k] && (cc & 3) == 0) row_scales[c >> 2] = (uint8_t)(127 - e8);
+    }
+    __syncthreads();
+
+    // phase B: blocks along columns from the LDS copy; a thread owns one column and two row blocks of 32
+    const int c = tid & (TILE - 1);
+    if (c < cols_valid) {
+        constexpr int blk_bytes = 32 * Wire<F>::bits / 8;
+        const int64_t col_row_bytes = rows / 32 * blk_bytes;             // bytes per column in the transposed payload
+#pragma unroll 1
+        for (int h = 0; h < 2; ++h) {
+            const int rb = (tid >> 7) * 2 + h;
+            if (rb * 32 >= rows_valid) break;
+            uint32_t w[16];
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                w[i] = (uint32_t)tile[(rb * 32 + 2 * i) * LDS_PITCH + c] | ((uint32_t)tile[(rb * 32 + 2 * i + 1) * LDS_PITCH + c] << 16);
+                acc_amax(amax, w[i]);
+            }
+            const int e8 = wire_e8<F>(amax);
+            uint8_t* dst = col_payload + (C0 + c) * col_row_bytes + (R0 / 32 + rb) * blk_bytes;
+            if constexpr (Fmt<F>::hw) {
+                uint32_t q[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = code_pair<F>(w[2 * i], e8) | (code_pair<F>(w[2 * i + 1], e8) << 16);
+                *reinterpret_cast<uint4*>(dst) = make_uint4(q[0], q[1], q[2], q[3]);
+                *reinterpret_cast<uint4*>(dst + 16) = make_uint4(q[4], q[5], q[6], q[7]);
+            } else {
+#pragma unroll
+                for (int g = 0; g < 3; ++g) {                                // 3 x 64 bits = 32 codes
+                    uint64_t acc = 0;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int lo_bit = 12 * i - 64 * g;                      // position of pair i in this 64-bit word
+                        if (lo_bit > -12 && lo_bit < 64) {
+                            const uint64_t p = code_pair<F>(w[i], e8);
+                            acc |= lo_bit >= 0 ? (p << lo_bit) : (p >> (-lo_bit));
+                        }
+                    }
+                    *reinterpret_cast<uint2*>(dst + 8 * g) = make_uint2((uint32_t)acc, (uint32_t)(acc >> 32));
+                }
+            }
+            col_scales[(C0 + c) * (rows / 32) + R0 / 32 + rb] = (uint8_t)(127 - e8);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+template <int F>
+__global__ __launch_bounds__(WWG) void k_mx_dequantize(const uint8_t* payload, const uint8_t* scales, uint4* out, int64_t nchunks) {
+    for (int64_t c = (int64_t)blockIdx.x * WWG + threadIdx.x; c < nchunks; c += (int64_t)gridDim.x * WWG) {
+        const int de = (int)scales[c >> 2] - 127;
+        float x[8];
+        if constexpr (Fmt<F>::hw) {
+            const uint2 q = *reinterpret_cast<const uint2*>(payload + c * 8);
+            x[0] = hw_unpack<F, 0>(q.x); x[1] = hw_unpack<F, 1>(q.x); x[2] = hw_unpack<F, 2>(q.x); x[3] = hw_unpack<F, 3>(q.x);
+            x[4] = hw_unpack<F, 0>(q.y); x[5] = hw_unpack<F, 1>(q.y); x[6] = hw_unpack<F, 2>(q.y); x[7] = hw_unpack<F, 3>(q.y);
+        } else {
+            const uint16_t* p = reinterpret_cast<const uint16_t*>(payload + (c >> 2) * 24 + (c & 3) * 6);
+            const uint64_t bits = (uint64_t)p[0] | ((uint64_t)p[1] << 16) | ((uint64_t)p[2] << 32);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t code = (uint32_t)(bits >> (6 * i)) & 0x3Fu;
+                x[i] = u2f(f2u(fp6_value<F>(code & 0x1Fu)) | ((code & 0x20u) << 26));
+            }
+        }
+        uint4 r;
+        r.x = store_pair<true>(ldexpf(x[0], de), ldexpf(x[1], de));
+        r.y = store_pair<true>(ldexpf(x[2], de), ldexpf(x[3], de));
+        r.z = store_pair<true>(ldexpf(x[4], de), ldexpf(x[5], de));
+        r.w = store_pair<true>(ldexpf(x[6], de), ldexpf(x[7], de));
+        out[c] = r;
+    }
+}
+
+}  // namespace mor
+
+using namespace mor;
+
+static int validate_wire(const void* a, const void* b, const void* c, int64_t rows, int64_t cols, int fmt, int64_t row_multiple) {
+    if (!a || !b || !c) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "NULL tensor pointer");
+    if (rows <= 0 || cols <= 0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "rows and cols must be positive (got %lld x %lld)", (long long)rows, (long long)cols);
+    if (cols % 32 || rows % row_multiple)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "MX blocks need cols %% 32 == 0 and rows %% %lld == 0 (got %lld x %lld)", (long long)row_multiple, (long long)rows, (long long)cols);
+    if (fmt < MOR_FMT_E4M3 || fmt > MOR_FMT_E2M3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "unknown element format %d", fmt);
+    if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor and payload must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(c) & 3u) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "scales must be 4-byte aligned");
+    return MOR_OK;
+}
+
+extern "C" size_t mor_mx_payload_bytes(int64_t rows, int64_t cols, int fmt) {
+    if (rows <= 0 || cols <= 0) return 0;
+    return (size_t)rows * (size_t)cols * ((fmt == MOR_FMT_E4M3 || fmt == MOR_FMT_E5M2) ? 8 : 6) / 8;
+}
+
+extern "C" int mor_mx_quantize(const void* input, void* payload, void* scales, int64_t rows, int64_t cols, int fmt, void* stream) {
+    if (int rc = validate_wire(input, payload, scales, rows, cols, fmt, 1)) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t nchunks = rows * cols / 8;
+    constexpr int NV = 4;
+    const unsigned grid = (unsigned)((nchunks + NV * WWG - 1) / (NV * WWG));
+    const uint4* in = static_cast<const uint4*>(input);
+    uint8_t* p = static_cast<uint8_t*>(payload);
+    uint8_t* s = static_cast<uint8_t*>(scales);
+    switch (fmt) {
+        case MOR_FMT_E4M3: k_mx_quantize<FMT_E4M3, NV><<<grid, WWG, 0, st>>>(in, p, s, nchunks); break;
+        case MOR_FMT_E5M2: k_mx_quantize<FMT_E5M2, NV><<<grid, WWG, 0, st>>>(in, p, s, nchunks); break;
+        case MOR_FMT_E3M2: k_mx_quantize<FMT_E3M2, NV><<<grid, WWG, 0, st>>>(in, p, s, nchunks); break;
+        default: k_mx_quantize<FMT_E2M3, NV><<<grid, WWG, 0, st>>>(in, p, s, nchunks); break;
+    }
+    return mor_check_launch("k_mx_quantize");
+}
+
+extern "C" int mor_mx_quantize_dual(const void* input, void* row_payload, void* row_scales, void* col_payload, void* col_scales,
+                                    int64_t rows, int64_t cols, int fmt, void* stream) {
+    if (int rc = validate_wire(input, row_payload, row_scales, rows, cols, fmt, 32)) return rc;
+    if (int rc = validate_wire(input, col_payload, col_scales, rows, cols, fmt, 32)) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t tiles = ((rows + TILE - 1) / TILE) * ((cols + TILE - 1) / TILE);
+    if (tiles > 0x7FFFFFFFll) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many tiles");
+    const uint4* in = static_cast<const uint4*>(input);
+    uint8_t *rp = static_cast<uint8_t*>(row_payload), *rs = static_cast<uint8_t*>(row_scales);
+    uint8_t *cp = static_cast<uint8_t*>(col_payload), *cs = static_cast<uint8_t*>(col_scales);
+    switch (fmt) {
+        case MOR_FMT_E4M3: k_mx_dual<FMT_E4M3><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        case MOR_FMT_E5M2: k_mx_dual<FMT_E5M2><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        case MOR_FMT_E3M2: k_mx_dual<FMT_E3M2><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        default: k_mx_dual<FMT_E2M3><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+    }
+    return mor_check_launch("k_mx_dual");
+}
+
+extern "C" int mor_mx_dequantize(const void* payload, const void* scales, void* output, int64_t rows, int64_t cols, int fmt, void* stream) {
+    if (int rc = validate_wire(output, payload, scales, rows, cols, fmt, 1)) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t nchunks = rows * cols / 8;
+    const unsigned grid = (unsigned)std::min<int64_t>((nchunks + WWG - 1) / WWG, 256 * 16);
+    const uint8_t* p = static_cast<const uint8_t*>(payload);
+    const uint8_t* s = static_cast<const uint8_t*>(scales);
+    uint4* out = static_cast<uint4*>(output);
+    switch (fmt) {
+        case MOR_FMT_E4M3: k_mx_dequantize<FMT_E4M3><<<grid, WWG, 0, st>>>(p, s, out, nchunks); break;
+        case MOR_FMT_E5M2: k_mx_dequantize<FMT_E5M2><<<grid, WWG, 0, st>>>(p, s, out, nchunks); break;
+        case MOR_FMT_E3M2: k_mx_dequantize<FMT_E3M2><<<grid, WWG, 0, st>>>(p, s, out, nchunks); break;
+        default: k_mx_dequantize<FMT_E2M3><<<grid, WWG, 0, st>>>(p, s, out, nchunks); break;
+    }
+    return mor_check_launch("k_mx_dequantize");
+}

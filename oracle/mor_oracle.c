@@ -792,3 +792,102 @@ void mor_oracle_e4m3_with_e8_scale(const float* in, float* out, size_t n, int rn
         out[i] = sqdd_e8(v, sf, rne, MOR_O_E4M3, 0, MOR_O_KERNEL);
     }
 }
+
+/* ------------------------------------------------------------------ */
+/* MX wire format: element codes + one E8M0 scale byte per block of 32 elements along a row.
+ *
+ * The reference only returns the dequantized bf16 tensor; these two functions state what its MX
+ * block quantization (quantize_kernel block modes with SF_E8, FQ:801-823, and the E2M3 branch
+ * FQ:758-770) stores before dequantizing: per block, e8 = exponent field of fl32(fmax / amax) - 127
+ * (FQ:251-252), code = cast(x * 2^e8) with the block format's cast (nearest even; the scaled value
+ * never exceeds fmax), scale byte = 127 - e8, i.e. the E8M0 encoding of the multiplier 2^-e8 that
+ * decodes the block.  Scaling is arithmetic (what the reference's torch emulation does,
+ * test_fake_quantize.py:41-46), so a zero code decodes to zero; the sign of the input is kept on
+ * every code.  A zero block has scale byte 127.  e8 is limited to [-127, 127] so that the byte
+ * stays a finite E8M0 value.  FP6 codes are packed little-endian, 4 codes in 3 bytes.
+ * Pinned by: decode(code) * 2^-e8 == mor_oracle_fake_quantize / mor_oracle_block_format in the
+ * torch-emulation flavour (itself pinned by torch), with the decode tables of
+ * tests/golden/scalar_vectors.npz; scale bytes == 254 - mor_oracle_block_stats exponents. */
+static uint32_t encode_mag(float r, int fmt) {          /* r >= 0 on the grid of fmt */
+    const fmt_t* f = &FMT[fmt];
+    if (r == 0.0f) return 0;
+    uint32_t b = f2u(r);
+    int e = (int)(b >> 23) - 127;
+    int emin = 1 - (int)f->bias;
+    if (e < emin) return (uint32_t)ldexpf(r, (int)f->mbits - emin);       /* subnormal: r / 2^(emin - mbits) */
+    return ((uint32_t)(e + (int)f->bias) << f->mbits) | ((b & 0x7FFFFFu) >> (23 - f->mbits));
+}
+
+static float decode_mag(uint32_t code, int fmt) {
+    const fmt_t* f = &FMT[fmt];
+    uint32_t e = code >> f->mbits, m = code & ((1u << f->mbits) - 1u);
+    if (e == 0) return ldexpf((float)m, 1 - (int)f->bias - (int)f->mbits);
+    return ldexpf(1.0f + (float)m / (float)(1u << f->mbits), (int)e - (int)f->bias);
+}
+
+static int mx_block_e8(const uint16_t* x, int n, int fmt, float* amax_o) {
+    float amax = 0.0f;
+    for (int i = 0; i < n; ++i) amax = max_nn(amax, fabsf(mor_oracle_bf16_to_fp32(x[i])));
+    *amax_o = amax;
+    if (!(amax > 0)) return 0;
+    int e8 = (int)((f2u(FMAX_OF[fmt] / amax) >> 23) & 0xFF) - 127;
+    return e8 > 127 ? 127 : e8 < -127 ? -127 : e8;
+}
+
+static size_t mx_row_bytes(int64_t cols, int fmt) { return (fmt <= MOR_O_E5M2) ? (size_t)cols : (size_t)cols / 4 * 3; }
+
+int mor_oracle_mx_quantize(const uint16_t* in, uint8_t* payload, uint8_t* scales, int64_t rows, int64_t cols, int fmt) {
+    if (rows <= 0 || cols <= 0 || cols % 32 || fmt < 0 || fmt > 3) return -1;
+    const int nbits = (fmt <= MOR_O_E5M2) ? 8 : 6;
+    const size_t rb = mx_row_bytes(cols, fmt);
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t b = 0; b < cols / 32; ++b) {
+            const uint16_t* x = in + r * cols + b * 32;
+            float amax;
+            int e8 = mx_block_e8(x, 32, fmt, &amax);
+            scales[r * (cols / 32) + b] = (uint8_t)(127 - e8);
+            uint8_t* dst = payload + r * rb + b * (32 * nbits / 8);
+            uint32_t codes[32];
+            for (int i = 0; i < 32; ++i) {
+                float v = mor_oracle_bf16_to_fp32(x[i]);
+                float scaled = (float)ldexp((double)fabsf(v), e8);      /* exact or below every grid's half step */
+                int over;
+                float q = rne_to_grid(scaled, (int)FMT[fmt].mbits, 1 - (int)FMT[fmt].bias, FMAX_OF[fmt], &over);
+                if (over) q = FMAX_OF[fmt];
+                codes[i] = encode_mag(q, fmt) | ((uint32_t)(x[i] >> 15) << (nbits - 1));
+            }
+            if (nbits == 8) for (int i = 0; i < 32; ++i) dst[i] = (uint8_t)codes[i];
+            else
+                for (int g = 0; g < 8; ++g) {                            /* 4 codes -> 24 bits, little-endian */
+                    uint32_t w = codes[4 * g] | (codes[4 * g + 1] << 6) | (codes[4 * g + 2] << 12) | (codes[4 * g + 3] << 18);
+                    dst[3 * g] = (uint8_t)w; dst[3 * g + 1] = (uint8_t)(w >> 8); dst[3 * g + 2] = (uint8_t)(w >> 16);
+                }
+        }
+    return 0;
+}
+
+int mor_oracle_mx_dequantize(const uint8_t* payload, const uint8_t* scales, uint16_t* out, int64_t rows, int64_t cols, int fmt) {
+    if (rows <= 0 || cols <= 0 || cols % 32 || fmt < 0 || fmt > 3) return -1;
+    const int nbits = (fmt <= MOR_O_E5M2) ? 8 : 6;
+    const size_t rb = mx_row_bytes(cols, fmt);
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t b = 0; b < cols / 32; ++b) {
+            const uint8_t* src = payload + r * rb + b * (32 * nbits / 8);
+            int de = (int)scales[r * (cols / 32) + b] - 127;
+            for (int i = 0; i < 32; ++i) {
+                uint32_t code;
+                if (nbits == 8) code = src[i];
+                else {
+                    const uint8_t* p = src + 3 * (i / 4);
+                    uint32_t w = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
+                    code = (w >> (6 * (i % 4))) & 0x3Fu;
+                }
+                uint32_t sign = code >> (nbits - 1), mag = code & ((1u << (nbits - 1)) - 1u);
+                float v = (float)ldexp((double)decode_mag(mag, fmt), de);
+                out[r * cols + b * 32 + i] = (uint16_t)(mor_oracle_fp32_to_bf16_rne(v) | (sign << 15));
+            }
+        }
+    return 0;
+}

@@ -90,6 +90,14 @@ void mor_oracle_e4m3_with_e8_scale(const float* in, float* out, size_t n, int rn
 int mor_oracle_block_stats(const uint16_t* in, int64_t rows, int64_t cols, int64_t brows,
                            int64_t bcols, float fmax, float* amax, float* scale, int32_t* e8m0);
 
+/* MX wire format (no counterpart in the reference, which returns only the dequantized tensor):
+ * blocks of 32 elements along a row, payload = element codes (FP8: one byte each, FP6: 4 codes in
+ * 3 bytes, little-endian), scales = one E8M0 byte per block (127 - e8, the decode multiplier). */
+int mor_oracle_mx_quantize(const uint16_t* in, uint8_t* payload, uint8_t* scales,
+                           int64_t rows, int64_t cols, int fmt);
+int mor_oracle_mx_dequantize(const uint8_t* payload, const uint8_t* scales, uint16_t* out,
+                             int64_t rows, int64_t cols, int fmt);
+
 int mor_oracle_num_threads(void);
 
 #ifdef __cplusplus

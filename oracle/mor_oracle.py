@@ -52,6 +52,8 @@ def lib():
             "mor_oracle_quant_dequant": (None, [vp, vp, sz, C.c_int]),
             "mor_oracle_e4m3_with_e8_scale": (None, [vp, vp, sz, C.c_int]),
             "mor_oracle_block_stats": (C.c_int, [vp, i64, i64, i64, i64, f32, vp, vp, vp]),
+            "mor_oracle_mx_quantize": (C.c_int, [vp, vp, vp, i64, i64, C.c_int]),
+            "mor_oracle_mx_dequantize": (C.c_int, [vp, vp, vp, i64, i64, C.c_int]),
             "mor_oracle_num_threads": (C.c_int, []),
         }
         for name, (res, args) in sig.items():
@@ -172,3 +174,28 @@ def block_stats(a, block_x, block_y, fmax):
     if rc:
         raise RuntimeError(f"mor_oracle_block_stats failed: {rc}")
     return amax, scale, e8
+
+
+def mx_row_bytes(cols, fmt):
+    return cols if fmt in (E4M3, E5M2) else cols // 4 * 3
+
+
+def mx_quantize(a, fmt):
+    """bf16 bits [rows, cols] -> (payload uint8 [rows, row_bytes], scales uint8 [rows, cols // 32])"""
+    a = _u16(a)
+    rows, cols = a.shape
+    payload = np.empty((rows, mx_row_bytes(cols, fmt)), np.uint8)
+    scales = np.empty((rows, cols // 32), np.uint8)
+    if lib().mor_oracle_mx_quantize(_p(a), _p(payload), _p(scales), rows, cols, fmt):
+        raise RuntimeError("mor_oracle_mx_quantize: invalid argument")
+    return payload, scales
+
+
+def mx_dequantize(payload, scales, fmt):
+    payload = np.ascontiguousarray(payload, np.uint8)
+    scales = np.ascontiguousarray(scales, np.uint8)
+    rows, cols = scales.shape[0], scales.shape[1] * 32
+    out = np.empty((rows, cols), np.uint16)
+    if lib().mor_oracle_mx_dequantize(_p(payload), _p(scales), _p(out), rows, cols, fmt):
+        raise RuntimeError("mor_oracle_mx_dequantize: invalid argument")
+    return out

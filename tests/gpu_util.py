@@ -122,3 +122,45 @@ def e4m3_with_e8_scale(x_f32, rne):
     _cabi.check(L.mor_e4m3_with_e8_scale(x.data_ptr(), out.data_ptr(), x.numel(), int(rne), stream_ptr()))
     torch.cuda.synchronize()
     return out.cpu().numpy()
+
+
+def mx_row_bytes(cols, fmt):
+    return cols if fmt in (_cabi.FMT_E4M3, _cabi.FMT_E5M2) else cols // 4 * 3
+
+
+def mx_quantize(a_u16, fmt, x_dev=None):
+    """-> (payload uint8 [rows, row_bytes], scales uint8 [rows, cols // 32]) through mor_mx_quantize"""
+    L = _cabi.lib()
+    rows, cols = a_u16.shape
+    x = to_dev_u16(a_u16) if x_dev is None else x_dev
+    payload = torch.full((rows, mx_row_bytes(cols, fmt)), 0xA5, dtype=torch.uint8, device=dev())
+    scales = torch.full((rows, cols // 32), 0xA5, dtype=torch.uint8, device=dev())
+    _cabi.check(L.mor_mx_quantize(x.data_ptr(), payload.data_ptr(), scales.data_ptr(), rows, cols, fmt, stream_ptr()))
+    torch.cuda.synchronize()
+    return payload.cpu().numpy(), scales.cpu().numpy()
+
+
+def mx_quantize_dual(a_u16, fmt):
+    """-> (row payload, row scales, column payload [cols, ...], column scales [cols, rows // 32])"""
+    L = _cabi.lib()
+    rows, cols = a_u16.shape
+    x = to_dev_u16(a_u16)
+    rp = torch.full((rows, mx_row_bytes(cols, fmt)), 0xA5, dtype=torch.uint8, device=dev())
+    rs = torch.full((rows, cols // 32), 0xA5, dtype=torch.uint8, device=dev())
+    cp = torch.full((cols, mx_row_bytes(rows, fmt)), 0xA5, dtype=torch.uint8, device=dev())
+    cs = torch.full((cols, rows // 32), 0xA5, dtype=torch.uint8, device=dev())
+    _cabi.check(L.mor_mx_quantize_dual(x.data_ptr(), rp.data_ptr(), rs.data_ptr(), cp.data_ptr(), cs.data_ptr(),
+                                       rows, cols, fmt, stream_ptr()))
+    torch.cuda.synchronize()
+    return rp.cpu().numpy(), rs.cpu().numpy(), cp.cpu().numpy(), cs.cpu().numpy()
+
+
+def mx_dequantize(payload, scales, fmt):
+    L = _cabi.lib()
+    rows, cols = scales.shape[0], scales.shape[1] * 32
+    p = torch.from_numpy(np.ascontiguousarray(payload)).to(dev())
+    s = torch.from_numpy(np.ascontiguousarray(scales)).to(dev())
+    out = torch.empty((rows, cols), dtype=torch.bfloat16, device=dev())
+    _cabi.check(L.mor_mx_dequantize(p.data_ptr(), s.data_ptr(), out.data_ptr(), rows, cols, fmt, stream_ptr()))
+    torch.cuda.synchronize()
+    return to_host_u16(out)
