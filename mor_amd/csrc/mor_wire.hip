@@ -57,14 +57,26 @@ template <int F> __device__ __forceinline__ float fp6_value(uint32_t mag) {
     return e == 0 ? sub : normal;
 }
 
-// codes of the two elements of a packed word, in bits 0..bits-1 and bits..2*bits-1
+// codes of the two elements of a packed word, in bits 0..bits-1 and bits..2*bits-1.
+// FP6 through the FP8 converts: E2M3 / E3M2 have the mantissa width of E4M3 / E5M2, so for a scaled magnitude a in
+// the normal range of the 6-bit format the 8-bit code differs from the 6-bit one by the bias difference only; below
+// that range the 6-bit grid is uniform (step = its subnormal step), which is the 8-bit grid of the binade
+// [norm_min, 2 norm_min): convert a + norm_min instead (the sum is exact whenever the rounding can depend on it).
 template <int F> __device__ __forceinline__ uint32_t code_pair(uint32_t w, int e8) {
     if constexpr (Fmt<F>::hw) {
         return hw_pack2<F>(ldexpf(bf16_lo(w), e8), ldexpf(bf16_hi(w), e8)) & 0xFFFFu;
     } else {
-        const uint32_t a = fp6_code<F>(round_mag_sat<F>(ldexpf(fabsf(bf16_lo(w)), e8))) | ((w >> 10) & 0x20u);
-        const uint32_t b = fp6_code<F>(round_mag_sat<F>(ldexpf(fabsf(bf16_hi(w)), e8))) | ((w >> 26) & 0x20u);
-        return a | (b << 6);
+        constexpr int F8 = (F == FMT_E2M3) ? FMT_E4M3 : FMT_E5M2;
+        constexpr int mb = Fmt<F>::mbits;
+        constexpr float norm_min = (F == FMT_E2M3) ? 1.0f : 0.25f;
+        constexpr uint32_t off_normal = (uint32_t)(Wire<F8>::bias - Wire<F>::bias) << mb;
+        constexpr uint32_t off_sub = (uint32_t)(1 - Wire<F>::bias + Wire<F8>::bias) << mb;
+        const float a = ldexpf(fabsf(bf16_lo(w)), e8), b = ldexpf(fabsf(bf16_hi(w)), e8);
+        const bool na = a >= norm_min, nb = b >= norm_min;
+        const uint32_t p = hw_pack2<F8>(na ? a : a + norm_min, nb ? b : b + norm_min);
+        const uint32_t ca = (p & 0xFFu) - (na ? off_normal : off_sub);
+        const uint32_t cb = ((p >> 8) & 0xFFu) - (nb ? off_normal : off_sub);
+        return ca | ((w >> 10) & 0x20u) | ((cb | ((w >> 26) & 0x20u)) << 6);
     }
 }
 
@@ -129,12 +141,19 @@ __global__ __launch_bounds__(WWG) void k_mx_quantize(const uint4* in, uint8_t* p
 // ------------------------------------------------------------------------------------------------
 // both orientations from one read.  Tile 128 x 128; rows % 32 == 0 and cols % 32 == 0.
 constexpr int TILE = 128;
-constexpr int LDS_PITCH = TILE + 8;              // in bf16 elements; keeps 16-byte alignment of the row starts
 
 template <int F>
 __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_payload, uint8_t* row_scales,
                                                  uint8_t* col_payload, uint8_t* col_scales, int64_t rows, int64_t cols) {
-    __shared__ __attribute__((aligned(16))) uint16_t tile[TILE * LDS_PITCH];
+    constexpr int PITCH = TILE + 8;               // bf16 elements per LDS row; keeps the row starts 16-byte aligned
+    constexpr int blk_bytes = 32 * Wire<F>::bits / 8;
+    constexpr int CODE_PITCH = 4 * blk_bytes + 16;    // bytes per column of the code tile
+    constexpr int SEG = Fmt<F>::hw ? 16 : 8;      // bytes per lane of the column stores (both divide blk_bytes)
+    constexpr int SEGS = 4 * blk_bytes / SEG;     // per column
+    // one buffer, two uses: the bf16 tile (34816 bytes), then the codes of the column blocks (<= 128 * 144 bytes)
+    __shared__ __attribute__((aligned(16))) uint16_t tile[TILE * PITCH];
+    __shared__ uint32_t s_cscale[TILE];
+    uint8_t* codes = reinterpret_cast<uint8_t*>(tile);
     const int tid = threadIdx.x;
     const int64_t tiles_x = (cols + TILE - 1) / TILE;
     const int64_t ty = blockIdx.x / tiles_x, tx = blockIdx.x - ty * tiles_x;
@@ -142,7 +161,6 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
     const int rows_valid = (int)min((int64_t)TILE, rows - R0), cols_valid = (int)min((int64_t)TILE, cols - C0);
     const int64_t row_chunks = cols >> 3;
 
-    // phase A: blocks along rows, from registers
     uint4 v[8];
     bool ok[8];
 #pragma unroll
@@ -155,56 +173,91 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
-        *reinterpret_cast<uint4*>(&tile[r * LDS_PITCH + cc * 8]) = v[k];
-        const float amax = group_max_t<4>(chunk_amax(v[k]), 4);
-        const int e8 = wire_e8<F>(amax);
-        const int64_t c = (R0 + r) * row_chunks + (C0 >> 3) + cc;          // chunk index in the row-major payload
-        store_codes<F>(row_payload, c, code_chunk<F>(v[k], e8), ok[k]);
-        if (ok[k] && (cc & 3) == 0) row_scales[c >> 2] = (uint8_t)(127 - e8);
+        *reinterpret_cast<uint4*>(&tile[r * PITCH + cc * 8]) = v[k];
     }
     __syncthreads();
-
-    // phase B: blocks along columns from the LDS copy; a thread owns one column and two row blocks of 32
+    // blocks along columns: a thread owns one column and two row blocks of 32, read from the LDS copy
     const int c = tid & (TILE - 1);
-    if (c < cols_valid) {
-        constexpr int blk_bytes = 32 * Wire<F>::bits / 8;
-        const int64_t col_row_bytes = rows / 32 * blk_bytes;             // bytes per column in the transposed payload
-#pragma unroll 1
-        for (int h = 0; h < 2; ++h) {
-            const int rb = (tid >> 7) * 2 + h;
-            if (rb * 32 >= rows_valid) break;
-            uint32_t w[16];
-            float amax = 0.0f;
+    uint32_t w[2][16];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                w[i] = (uint32_t)tile[(rb * 32 + 2 * i) * LDS_PITCH + c] | ((uint32_t)tile[(rb * 32 + 2 * i + 1) * LDS_PITCH + c] << 16);
-                acc_amax(amax, w[i]);
-            }
-            const int e8 = wire_e8<F>(amax);
-            uint8_t* dst = col_payload + (C0 + c) * col_row_bytes + (R0 / 32 + rb) * blk_bytes;
-            if constexpr (Fmt<F>::hw) {
-                uint32_t q[8];
+    for (int h = 0; h < 2; ++h) {
+        const int rb = (tid >> 7) * 2 + h;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) q[i] = code_pair<F>(w[2 * i], e8) | (code_pair<F>(w[2 * i + 1], e8) << 16);
-                *reinterpret_cast<uint4*>(dst) = make_uint4(q[0], q[1], q[2], q[3]);
-                *reinterpret_cast<uint4*>(dst + 16) = make_uint4(q[4], q[5], q[6], q[7]);
-            } else {
+        for (int i = 0; i < 16; ++i)
+            w[h][i] = (uint32_t)tile[(rb * 32 + 2 * i) * PITCH + c] | ((uint32_t)tile[(rb * 32 + 2 * i + 1) * PITCH + c] << 16);
+    }
+    // blocks along rows, from registers (the global stores overlap the LDS latency above)
+    const bool dword_row_scales = (cols & 127) == 0;
 #pragma unroll
-                for (int g = 0; g < 3; ++g) {                                // 3 x 64 bits = 32 codes
-                    uint64_t acc = 0;
+    for (int k = 0; k < 8; ++k) {
+        const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+        const float amax = group_max_t<4>(chunk_amax(v[k]), 4);
+        const int e8 = wire_e8<F>(amax);
+        const int64_t cidx = (R0 + r) * row_chunks + (C0 >> 3) + cc;       // chunk index in the row-major payload
+        store_codes<F>(row_payload, cidx, code_chunk<F>(v[k], e8), ok[k]);
+        const uint32_t sb = (uint32_t)(127 - e8);
+        const uint32_t s4 = sb | (__shfl_down(sb, 4, 16) << 8) | (__shfl_down(sb, 8, 16) << 16) | (__shfl_down(sb, 12, 16) << 24);
+        if (dword_row_scales && cols_valid == TILE) {
+            if (ok[k] && cc == 0) *reinterpret_cast<uint32_t*>(row_scales + (cidx >> 2)) = s4;
+        } else if (ok[k] && (cc & 3) == 0) row_scales[cidx >> 2] = (uint8_t)sb;
+    }
+    __syncthreads();                              // every thread has its column blocks in registers: reuse the buffer
+
+    uint32_t my_scales = 0;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int lo_bit = 12 * i - 64 * g;                      // position of pair i in this 64-bit word
-                        if (lo_bit > -12 && lo_bit < 64) {
-                            const uint64_t p = code_pair<F>(w[i], e8);
-                            acc |= lo_bit >= 0 ? (p << lo_bit) : (p >> (-lo_bit));
-                        }
-                    }
-                    *reinterpret_cast<uint2*>(dst + 8 * g) = make_uint2((uint32_t)acc, (uint32_t)(acc >> 32));
+    for (int h = 0; h < 2; ++h) {
+        const int rb = (tid >> 7) * 2 + h;
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc_amax(amax, w[h][i]);
+        const int e8 = wire_e8<F>(amax);
+        my_scales |= (uint32_t)(127 - e8) << (8 * h);
+        uint8_t* dst = codes + c * CODE_PITCH + rb * blk_bytes;
+        if constexpr (Fmt<F>::hw) {
+            uint32_t q[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) q[i] = code_pair<F>(w[h][2 * i], e8) | (code_pair<F>(w[h][2 * i + 1], e8) << 16);
+            *reinterpret_cast<uint4*>(dst) = make_uint4(q[0], q[1], q[2], q[3]);
+            *reinterpret_cast<uint4*>(dst + 16) = make_uint4(q[4], q[5], q[6], q[7]);
+        } else {
+            uint32_t p[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) p[i] = code_pair<F>(w[h][i], e8);
+#pragma unroll
+            for (int g = 0; g < 3; ++g) {                                    // 3 x 64 bits = 32 codes
+                uint64_t acc = 0;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int lo_bit = 12 * i - 64 * g;                      // position of pair i in this 64-bit word
+                    if (lo_bit > -12 && lo_bit < 64) acc |= lo_bit >= 0 ? ((uint64_t)p[i] << lo_bit) : ((uint64_t)p[i] >> (-lo_bit));
                 }
+                *reinterpret_cast<uint2*>(dst + 8 * g) = make_uint2((uint32_t)acc, (uint32_t)(acc >> 32));
             }
-            col_scales[(C0 + c) * (rows / 32) + R0 / 32 + rb] = (uint8_t)(127 - e8);
         }
+    }
+    if (tid >= TILE) s_cscale[c] = my_scales;
+    __syncthreads();
+
+    // the transposed payload: a column of the tile is 4 * blk_bytes contiguous bytes, SEGS lanes store one column
+    const int64_t col_row_bytes = rows / 32 * blk_bytes;                 // bytes per column in the transposed payload
+    const int valid_bytes = rows_valid / 32 * blk_bytes;
+#pragma unroll
+    for (int i = 0; i < TILE * SEGS / WWG; ++i) {
+        const int idx = i * WWG + tid, col = idx / SEGS, seg = idx % SEGS;
+        if (col < cols_valid && seg * SEG < valid_bytes) {
+            uint8_t* dst = col_payload + (C0 + col) * col_row_bytes + (R0 / 32) * blk_bytes + seg * SEG;
+            const uint8_t* src = codes + col * CODE_PITCH + seg * SEG;
+            if constexpr (SEG == 16) *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
+            else *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(src);
+        }
+    }
+    // scale bytes of the column blocks: 4 per column and tile
+    if (tid < TILE && c < cols_valid) {
+        const uint32_t s4 = my_scales | (s_cscale[c] << 16);
+        uint8_t* dst = col_scales + (C0 + c) * (rows / 32) + R0 / 32;
+        if ((rows & 127) == 0) *reinterpret_cast<uint32_t*>(dst) = s4;
+        else
+            for (int b = 0; b < rows_valid / 32; ++b) dst[b] = (uint8_t)(s4 >> (8 * b));
     }
 }
 
