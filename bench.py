@@ -257,6 +257,7 @@ def other_configs(torch, run, cabi, K, W):
     res["c4_mor_128x128_16384x14336_mixture"]["meta_histogram"] = {str(i): h for i, h in enumerate(hist) if h}
     del x4, o4
     res["c5_llama3_8b_layer"] = c5_sweep(torch, run, max(3, K // 4), 2)
+    res["mx_wire_format_8192x8192"] = wire_format(torch, run, K, W)
     # launch overhead: a 1x32 tensor
     xs = torch.randn(1, 32, device="cuda").to(torch.bfloat16)
     os_ = torch.empty_like(xs)
@@ -264,6 +265,30 @@ def other_configs(torch, run, cabi, K, W):
     ms, wall = time_launches(torch, lambda: run.fake_quantize(xs, os_, ms_, 1, 32, 0.0, 2, 2), 200, 20)
     res["tiny_1x32"] = {"us_per_call_events": round(ms * 1e3, 2), "us_per_call_wall": round(wall * 1e3, 2)}
     return res
+
+
+def wire_format(torch, run, K, W):
+    """The MX wire format on the benchmark tensor: codes + E8M0 scale bytes (2 B read + 1 or 0.75 B written per element
+    + 1 scale byte per block), both orientations from one read, and the decode."""
+    L = run.L
+    rows = cols = 8192
+    x = gen_c2_gpu(torch, rows, cols)
+    n = rows * cols
+    out = {}
+    for fmt, name, bits in ((run.cabi.FMT_E4M3, "e4m3", 8), (run.cabi.FMT_E5M2, "e5m2", 8), (run.cabi.FMT_E2M3, "e2m3", 6)):
+        pb = n * bits // 8
+        p = torch.empty(pb, dtype=torch.uint8, device="cuda")
+        s = torch.empty(n // 32, dtype=torch.uint8, device="cuda")
+        cp, cs, o = torch.empty_like(p), torch.empty_like(s), torch.empty_like(x)
+        for key, fn, nbytes in (
+            ("quantize", lambda: run.cabi.check(L.mor_mx_quantize(x.data_ptr(), p.data_ptr(), s.data_ptr(), rows, cols, fmt, run.stream())), 2 * n + pb + n // 32),
+            ("quantize_dual", lambda: run.cabi.check(L.mor_mx_quantize_dual(x.data_ptr(), p.data_ptr(), s.data_ptr(), cp.data_ptr(), cs.data_ptr(), rows, cols, fmt, run.stream())), 2 * n + 2 * (pb + n // 32)),
+            ("dequantize", lambda: run.cabi.check(L.mor_mx_dequantize(p.data_ptr(), s.data_ptr(), o.data_ptr(), rows, cols, fmt, run.stream())), 2 * n + pb + n // 32),
+        ):
+            ms = time_launches(torch, fn, K, W)[0]
+            out[f"{key}_{name}"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                    "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    return out
 
 
 def c5_sweep(torch, run, K, W):

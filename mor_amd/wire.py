@@ -1,0 +1,75 @@
+"""MX wire format on MI355X: the quantized tensor (element codes + E8M0 scale bytes) instead of its dequantized image.
+
+The reference's ops only return bf16 (mor/ops.py); these functions are the step next to them in a training loop: the
+payload a scaled-MFMA GEMM consumes.  The quantization is the reference's MX block rule (block modes with sf_type 2,
+mor/csrc/cuda/fake_quantize.cu:801-823, :251-252): blocks of 32 elements, scale 2^floor(log2(fmax / amax)), so
+`dequantize_mx(*quantize_mx(x, fmt), fmt)` equals `mor.ops.fake_quantize(x, ..., 1, 32, 0.0, mode, 2)[0]` (mode 2 for
+E4M3, 3 for E5M2) wherever the latter's values are not the exponent-clamp artefacts of that kernel.
+"""
+from typing import Tuple
+
+import torch
+from torch import Tensor
+
+from . import _cabi
+
+E4M3, E5M2, E3M2, E2M3 = _cabi.FMT_E4M3, _cabi.FMT_E5M2, _cabi.FMT_E3M2, _cabi.FMT_E2M3
+
+_L = _cabi.lib()
+
+
+def payload_row_bytes(cols: int, fmt: int) -> int:
+    return cols if fmt in (E4M3, E5M2) else cols // 4 * 3
+
+
+def _check(x: Tensor, row_multiple: int) -> Tuple[int, int]:
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_cuda:
+        raise RuntimeError("mor: expected a 2-D bfloat16 GPU tensor")
+    rows, cols = x.shape
+    if cols % 32 or rows % row_multiple:
+        raise RuntimeError(f"mor: MX blocks need cols % 32 == 0 and rows % {row_multiple} == 0, got {tuple(x.shape)}")
+    return rows, cols
+
+
+def _stream(x: Tensor) -> int:
+    return torch.cuda.current_stream(x.device).cuda_stream
+
+
+def quantize_mx(x: Tensor, fmt: int = E4M3) -> Tuple[Tensor, Tensor]:
+    """-> (payload uint8 [rows, cols * bits / 8], scales uint8 [rows, cols / 32]); blocks of 32 along rows."""
+    rows, cols = _check(x, 1)
+    x = x.contiguous()
+    with torch.cuda.device(x.device):
+        payload = torch.empty((rows, payload_row_bytes(cols, fmt)), dtype=torch.uint8, device=x.device)
+        scales = torch.empty((rows, cols // 32), dtype=torch.uint8, device=x.device)
+        _cabi.check(_L.mor_mx_quantize(x.data_ptr(), payload.data_ptr(), scales.data_ptr(), rows, cols, fmt, _stream(x)))
+    return payload, scales
+
+
+def quantize_mx_dual(x: Tensor, fmt: int = E4M3) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """One read of x, both orientations: (payload, scales) of x as quantize_mx gives them and (payload, scales) of
+    x.t() -- the operands of the dgrad and wgrad GEMMs of a linear layer."""
+    rows, cols = _check(x, 32)
+    x = x.contiguous()
+    with torch.cuda.device(x.device):
+        rp = torch.empty((rows, payload_row_bytes(cols, fmt)), dtype=torch.uint8, device=x.device)
+        rs = torch.empty((rows, cols // 32), dtype=torch.uint8, device=x.device)
+        cp = torch.empty((cols, payload_row_bytes(rows, fmt)), dtype=torch.uint8, device=x.device)
+        cs = torch.empty((cols, rows // 32), dtype=torch.uint8, device=x.device)
+        _cabi.check(_L.mor_mx_quantize_dual(x.data_ptr(), rp.data_ptr(), rs.data_ptr(), cp.data_ptr(), cs.data_ptr(),
+                                            rows, cols, fmt, _stream(x)))
+    return rp, rs, cp, cs
+
+
+def dequantize_mx(payload: Tensor, scales: Tensor, fmt: int = E4M3) -> Tensor:
+    """payload + scales -> bf16 [rows, 32 * scales.shape[1]]"""
+    if payload.dtype != torch.uint8 or scales.dtype != torch.uint8 or not payload.is_cuda or scales.dim() != 2:
+        raise RuntimeError("mor: expected uint8 GPU tensors")
+    rows, cols = scales.shape[0], scales.shape[1] * 32
+    if payload.numel() != rows * payload_row_bytes(cols, fmt):
+        raise RuntimeError("mor: payload size does not match the scales")
+    payload, scales = payload.contiguous(), scales.contiguous()
+    with torch.cuda.device(payload.device):
+        out = torch.empty((rows, cols), dtype=torch.bfloat16, device=payload.device)
+        _cabi.check(_L.mor_mx_dequantize(payload.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, cols, fmt, _stream(payload)))
+    return out

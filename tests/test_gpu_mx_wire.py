@@ -124,3 +124,24 @@ def test_full_size_properties(G, fmt):
     torch.cuda.synchronize()
     assert torch.equal(rp, p) and torch.equal(rs, s)
     assert torch.equal(cp, tp) and torch.equal(cs, ts)
+
+
+def test_python_api_round_trip():
+    from mor_amd import wire
+    import mor
+    x = data_gen.c2_student_t(256, 512, seed=31, as_tensor=True).cuda()
+    for fmt, mode in ((wire.E4M3, 2), (wire.E5M2, 3)):
+        p, s = wire.quantize_mx(x, fmt)
+        mor.ops.set_flavour("torch_emulation")
+        try:
+            want = mor.ops.fake_quantize(x, 256, 512, 1, 32, 0.0, mode, 2)[0]
+        finally:
+            mor.ops.set_flavour("kernel")
+        assert torch.equal(wire.dequantize_mx(p, s, fmt).view(torch.int16), want.view(torch.int16))
+        rp, rs, cp, cs = wire.quantize_mx_dual(x, fmt)
+        tp, ts = wire.quantize_mx(x.t().contiguous(), fmt)
+        assert torch.equal(rp, p) and torch.equal(rs, s) and torch.equal(cp, tp) and torch.equal(cs, ts)
+    with pytest.raises(RuntimeError):
+        wire.quantize_mx(x[:, :48], wire.E4M3)
+    p6, s6 = wire.quantize_mx(x, wire.E2M3)
+    assert p6.shape == (256, 384) and wire.dequantize_mx(p6, s6, wire.E2M3).shape == (256, 512)
