@@ -308,60 +308,68 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
 
 // ------------------------------------------------------------------------------------------------
 // Per-block look-up tables in LDS for fp32 scales (E4M3 / E5M2, block in the fast range).
-// The descaled value of an element depends only on its 7-bit magnitude code, so q(code) = decode(code) / s is
-// computed once per block with the IEEE division and the per-element divisions of FQ:314 disappear.
-// Entries 0..127: E4M3 with s4 = 448 / amax; entries 128..255: E5M2 with s5 = 57344 / amax.
-__device__ __forceinline__ void build_luts(float* lut, int tid, float s4, float s5) {
-    if (tid < 128) lut[tid] = hw_unpack<FMT_E4M3, 0>((uint32_t)tid) / s4;
-    else lut[tid] = hw_unpack<FMT_E5M2, 0>((uint32_t)(tid - 128)) / s5;
+// Division by the block scale without a divide per element: with r = RN(1 / s) (one IEEE division per block),
+// t = c * r; q = fma(fma(-t, s, c), r, t) is the correctly rounded quotient c / s (Markstein) as long as nothing
+// over- or underflows (the fast range) and the significand of s is not all ones (never the case for fmax / amax
+// with a bf16 amax; the callers check it anyway).
+__device__ __forceinline__ float div_by_scale(float c, float s, float r) {
+    const float t = c * r;
+    return fmaf(fmaf(-t, s, c), r, t);
 }
+__device__ __forceinline__ bool scale_divides(float s) { return (f2u(s) & 0x7FFFFFu) != 0x7FFFFFu; }
 
-// quantize one packed word through the table: |x| * s, hardware convert, table, round-half-up store, sign
-template <int F> __device__ __forceinline__ uint32_t fq_pair_lut(uint32_t w, float s, const float* lut) {
-    uint32_t p = hw_pack2<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s);
-    float q0 = lut[p & 0xFFu];
-    float q1 = lut[(p >> 8) & 0xFFu];
+// quantize one packed word with an fp32 scale: |x| * s, hardware convert, divide by s, round-half-up store, sign
+template <int F> __device__ __forceinline__ uint32_t fq_pair_div(uint32_t w, float s, float r) {
+    const uint32_t p = hw_pack2<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s);
+    const float q0 = div_by_scale(hw_unpack<F, 0>(p), s, r);
+    const float q1 = div_by_scale(hw_unpack<F, 1>(p), s, r);
     return store_pair<false>(q0, q1) | (w & 0x80008000u);
 }
-template <int F> __device__ __forceinline__ uint4 fq_vec_lut(uint4 v, float s, const float* lut) {
-    uint4 r;
-    r.x = fq_pair_lut<F>(v.x, s, lut);
-    r.y = fq_pair_lut<F>(v.y, s, lut);
-    r.z = fq_pair_lut<F>(v.z, s, lut);
-    r.w = fq_pair_lut<F>(v.w, s, lut);
-    return r;
+template <int F> __device__ __forceinline__ uint4 fq_vec_div(uint4 v, float s, float r) {
+    uint4 o;
+    o.x = fq_pair_div<F>(v.x, s, r);
+    o.y = fq_pair_div<F>(v.y, s, r);
+    o.z = fq_pair_div<F>(v.z, s, r);
+    o.w = fq_pair_div<F>(v.w, s, r);
+    return o;
 }
 
 // The two error terms of one packed word (FQ:504-542) on magnitudes; s5 = 128 * s4 exactly.
-// The reference computes |q / x - 1|; here |q - x| * (1 / x): q - x is exact in fp32 (q is within a factor 2 of
-// x, or 0), so each term carries one reciprocal's relative error (1e-7) instead of the absolute 6e-8 rounding of
-// a quotient near 1.  Both agree with the exact term far inside the 1e-6 tolerance on the sums; decisions that
-// would depend on less than 1e-5 are recomputed with the reference's divisions by the caller.
+// The reference computes |q / x - 1| with q = c / s.  E8 scale: |q - x| * (1 / x), q - x exact.  FP32 scale:
+// with y = x * s the same quantity is |c - y| / y (c - y is exact: c is within a factor 2 of y, or 0), which needs
+// neither q nor a division; for E5M2 c5 / 128 - y is one exact fma.  Each term differs from the reference's by
+// rounding errors of 1e-7 relative, of either sign, far inside the 1e-6 tolerance on the sums; decisions that would
+// depend on less than 1e-5 are recomputed with the reference's divisions by the caller.  The sums are only wanted
+// for blocks with amax / min non-zero |x| <= 939524096 (FQ:637), so a non-zero element scales to at least
+// 448 / 939524096 and no reciprocal overflows.
 template <bool E8>
-__device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, const float* lut, float& e4, float& e5) {
+__device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float& e4, float& e5) {
     float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
-    float qa4, qb4, qa5, qb5;
     if constexpr (E8) {
         const int e84 = s4.e8, e85 = s4.e8 + 7;
         uint32_t p4 = hw_pack2<FMT_E4M3>(ldexpf(a, e84), ldexpf(b, e84));
         uint32_t p5 = hw_pack2<FMT_E5M2>(ldexpf(a, e85), ldexpf(b, e85));
-        qa4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p4)) - (e84 << 23), 0));
-        qb4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p4)) - (e84 << 23), 0));
-        qa5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 0>(p5)) - (e85 << 23), 0));
-        qb5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 1>(p5)) - (e85 << 23), 0));
+        float qa4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p4)) - (e84 << 23), 0));
+        float qb4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p4)) - (e84 << 23), 0));
+        float qa5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 0>(p5)) - (e85 << 23), 0));
+        float qb5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 1>(p5)) - (e85 << 23), 0));
+        float ya = (a != 0.0f) ? __builtin_amdgcn_rcpf(a) : 0.0f;
+        float yb = (b != 0.0f) ? __builtin_amdgcn_rcpf(b) : 0.0f;
+        e4 = fmaf(fabsf(qa4 - a), ya, e4);
+        e5 = fmaf(fabsf(qa5 - a), ya, e5);
+        e4 = fmaf(fabsf(qb4 - b), yb, e4);
+        e5 = fmaf(fabsf(qb5 - b), yb, e5);
     } else {
-        float va = a * s4.s, vb = b * s4.s;
-        uint32_t p4 = hw_pack2<FMT_E4M3>(va, vb);
-        uint32_t p5 = hw_pack2<FMT_E5M2>(va * 128.0f, vb * 128.0f);
-        qa4 = lut[p4 & 0xFFu]; qb4 = lut[(p4 >> 8) & 0xFFu];
-        qa5 = lut[128u + (p5 & 0xFFu)]; qb5 = lut[128u + ((p5 >> 8) & 0xFFu)];
+        const float va = a * s4.s, vb = b * s4.s;
+        const uint32_t p4 = hw_pack2<FMT_E4M3>(va, vb);
+        const uint32_t p5 = hw_pack2<FMT_E5M2>(va * 128.0f, vb * 128.0f);
+        const float ya = (a != 0.0f) ? __builtin_amdgcn_rcpf(va) : 0.0f;
+        const float yb = (b != 0.0f) ? __builtin_amdgcn_rcpf(vb) : 0.0f;
+        e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 0>(p4) - va), ya, e4);
+        e5 = fmaf(fabsf(fmaf(hw_unpack<FMT_E5M2, 0>(p5), 0.0078125f, -va)), ya, e5);
+        e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 1>(p4) - vb), yb, e4);
+        e5 = fmaf(fabsf(fmaf(hw_unpack<FMT_E5M2, 1>(p5), 0.0078125f, -vb)), yb, e5);
     }
-    float ya = (a != 0.0f) ? __builtin_amdgcn_rcpf(a) : 0.0f;
-    float yb = (b != 0.0f) ? __builtin_amdgcn_rcpf(b) : 0.0f;
-    e4 = fmaf(fabsf(qa4 - a), ya, e4);
-    e5 = fmaf(fabsf(qa5 - a), ya, e5);
-    e4 = fmaf(fabsf(qb4 - b), yb, e4);
-    e5 = fmaf(fabsf(qb5 - b), yb, e5);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -373,10 +381,8 @@ __device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, const
 template <bool MOR, bool E8, int NV, bool FULL, bool NT>
 __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
-    constexpr bool LUT = !E8;
     __shared__ float s_f[2][WAVES];
     __shared__ uint32_t s_u[WAVES];
-    __shared__ float s_lut[LUT ? 256 : 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t bid = blockIdx.x;
     const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
@@ -420,7 +426,7 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
 
     // scales of the two fp8 formats; the fp6 scales differ from s4 by 2^4 / 2^6, inside the margin of `fast`
     const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
-    if (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90)) {           // uniform over the workgroup
+    if (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && scale_divides(s4.s))) {           // uniform over the workgroup
         generic_block<false>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
                              sh, qa, E8, bid, s_f, s_u);
         return;
@@ -429,20 +435,18 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
     int fmt = qa.fmt;
     int meta_val = qa.meta_val;
     float e4 = 0.0f, e5 = 0.0f;
-    bool lut_built = false;
     if constexpr (MOR) {
         int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
         if (qt == Q_UNKNOWN) {
             // pass 2 (registers): the two error sums, FQ:487-584.  amax > 0 here.
-            if constexpr (LUT) { build_luts(s_lut, tid, s4.s, s5.s); lut_built = true; }
-            __syncthreads();                     // tables written, s_f[0] read by every wave
+            __syncthreads();                     // s_f[0] has been read by every wave
 #pragma unroll
             for (int k = 0; k < NV; ++k)
                 if (ok[k]) {
-                    err_pair_fast<E8>(v[k].x, s4, s_lut, e4, e5);
-                    err_pair_fast<E8>(v[k].y, s4, s_lut, e4, e5);
-                    err_pair_fast<E8>(v[k].z, s4, s_lut, e4, e5);
-                    err_pair_fast<E8>(v[k].w, s4, s_lut, e4, e5);
+                    err_pair_fast<E8>(v[k].x, s4, e4, e5);
+                    err_pair_fast<E8>(v[k].y, s4, e4, e5);
+                    err_pair_fast<E8>(v[k].z, s4, e4, e5);
+                    err_pair_fast<E8>(v[k].w, s4, e4, e5);
                 }
             e4 = wave_sum(e4);
             e5 = wave_sum(e5);
@@ -488,15 +492,15 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
         }
         return;
     }
-    if constexpr (LUT) {
+    if constexpr (!E8) {
         if (fmt == FMT_E4M3 || fmt == FMT_E5M2) {
-            if (!lut_built) { build_luts(s_lut, tid, s4.s, s5.s); __syncthreads(); }
+            const float r4 = 1.0f / s4.s;            // 1 / s5 = r4 / 128 exactly
             if (fmt == FMT_E4M3) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_lut<FMT_E4M3>(v[k], s4.s, s_lut));
+                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_div<FMT_E4M3>(v[k], s4.s, r4));
             } else {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_lut<FMT_E5M2>(v[k], s5.s, s_lut + 128));
+                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f));
             }
             return;
         }
