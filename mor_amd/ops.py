@@ -78,7 +78,24 @@ def _check_result(t: Tensor, rows: int, cols: int) -> None:
 
 
 def _stream(t: Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return torch._C._cuda_getCurrentRawStream(t.device.index)
+
+
+class _on_device:
+    """`with torch.cuda.device(d)` only when d is not already the current device (the usual case costs nothing)."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, device):
+        self.ctx = None if device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
 
 
 def _cdiv(a: int, b: int) -> int:
@@ -94,7 +111,7 @@ def _fake_quantize_impl(input, dim_x, dim_y, block_x, block_y, clamp_threshold, 
     _check_input(input, torch.bfloat16, dim_x, dim_y)
     _check_blocks(block_x, block_y)
     x = input.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         out = torch.empty_like(x)
         meta = torch.empty((_cdiv(dim_x, block_x), _cdiv(dim_y, block_y)), dtype=torch.int32, device=x.device)
         _cabi.check(_L.mor_fake_quantize(x.data_ptr(), out.data_ptr(), meta.data_ptr(), dim_x, dim_y, block_x, block_y,
@@ -107,7 +124,7 @@ def _fake_quantize_no_alloc_impl(input, dim_x, dim_y, block_x, block_y, clamp_th
     _check_result(result, dim_x, dim_y)
     _check_blocks(block_x, block_y)
     x = input.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         meta = torch.empty((_cdiv(dim_x, block_x), _cdiv(dim_y, block_y)), dtype=torch.int32, device=x.device)
         _cabi.check(_L.mor_fake_quantize(x.data_ptr(), result.data_ptr(), meta.data_ptr(), dim_x, dim_y, block_x, block_y,
                                          clamp_threshold, mode, sf_type, _flags, _stream(x)))
@@ -120,7 +137,7 @@ def _scaling_impl(input, dim_x, dim_y, block_x, block_y, e4m3_threshold, ss_mode
     if dim_x % block_x or dim_y % block_y:
         raise RuntimeError(f"mor: block ({block_x}, {block_y}) does not divide the tensor ({dim_x}, {dim_y})")
     x = input.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         dev = x.device
         out = x if inplace else torch.empty_like(x)
         meta = torch.empty(1, dtype=torch.int32, device=dev)
@@ -144,7 +161,7 @@ def _e8mx_impl(input, dim_x, dim_y, block_x, block_y, quantize_type, scaling_str
     if result is not None:
         _check_result(result, dim_x, dim_y)
     x = input.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         out = torch.empty_like(x) if result is None else result
         nbytes = _L.mor_workspace_bytes(_cabi.OP_E8MX, dim_x, dim_y, block_x, block_y)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
@@ -156,7 +173,7 @@ def _e8mx_impl(input, dim_x, dim_y, block_x, block_y, quantize_type, scaling_str
 def _quant_dequant_impl(input, dim_x, dim_y, fmt):
     _check_input(input, torch.float32, dim_x, dim_y)
     x = input.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         out = torch.empty_like(x)
         _cabi.check(_L.mor_quant_dequant(x.data_ptr(), out.data_ptr(), x.numel(), fmt, _stream(x)))
     return out
@@ -165,7 +182,7 @@ def _quant_dequant_impl(input, dim_x, dim_y, fmt):
 def _e8_scale_impl(input, dim_x, dim_y, rne):
     _check_input(input, torch.float32, dim_x, dim_y)
     x = input.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         out = torch.empty_like(x)
         _cabi.check(_L.mor_e4m3_with_e8_scale(x.data_ptr(), out.data_ptr(), x.numel(), rne, _stream(x)))
     return out
