@@ -139,49 +139,54 @@ __global__ __launch_bounds__(WWG) void k_mx_quantize(const uint4* in, uint8_t* p
 }
 
 // ------------------------------------------------------------------------------------------------
-// both orientations from one read.  Tile 128 x 128; rows % 32 == 0 and cols % 32 == 0.
-constexpr int TILE = 128;
+// both orientations from one read.  Tile TR rows x 128 columns (TR = 64 or 128); rows % 32 == 0, cols % 32 == 0.
+constexpr int TILE_C = 128;
+constexpr int TILE_ROWS = 128;
 
-template <int F>
+template <int F, int TR>
 __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_payload, uint8_t* row_scales,
                                                  uint8_t* col_payload, uint8_t* col_scales, int64_t rows, int64_t cols) {
-    constexpr int PITCH = TILE + 8;               // bf16 elements per LDS row; keeps the row starts 16-byte aligned
+    constexpr int PITCH = TILE_C + 8;             // bf16 elements per LDS row; keeps the row starts 16-byte aligned
+    constexpr int NV = TR * (TILE_C / 8) / WWG;   // 16-byte chunks per thread
+    constexpr int RB = TR / 32;                   // row blocks per tile column
+    constexpr int BPT = TILE_C * RB / WWG;        // column blocks per thread
     constexpr int blk_bytes = 32 * Wire<F>::bits / 8;
-    constexpr int CODE_PITCH = 4 * blk_bytes + 16;    // bytes per column of the code tile
     constexpr int SEG = Fmt<F>::hw ? 16 : 8;      // bytes per lane of the column stores (both divide blk_bytes)
-    constexpr int SEGS = 4 * blk_bytes / SEG;     // per column
-    // one buffer, two uses: the bf16 tile (34816 bytes), then the codes of the column blocks (<= 128 * 144 bytes)
-    __shared__ __attribute__((aligned(16))) uint16_t tile[TILE * PITCH];
-    __shared__ uint32_t s_cscale[TILE];
+    constexpr int CODE_PITCH = RB * blk_bytes + SEG;  // bytes per column of the code tile (the pad spreads the banks)
+    constexpr int SEGS = RB * blk_bytes / SEG;    // per column
+    // one buffer, two uses: the bf16 tile, then the codes of the column blocks (smaller)
+    __shared__ __attribute__((aligned(16))) uint16_t tile[TR * PITCH];
+    __shared__ uint32_t s_cscale[TILE_C];
     uint8_t* codes = reinterpret_cast<uint8_t*>(tile);
+    static_assert(TILE_C * CODE_PITCH <= TR * PITCH * 2, "the code tile must fit the bf16 tile");
     const int tid = threadIdx.x;
-    const int64_t tiles_x = (cols + TILE - 1) / TILE;
+    const int64_t tiles_x = (cols + TILE_C - 1) / TILE_C;
     const int64_t ty = blockIdx.x / tiles_x, tx = blockIdx.x - ty * tiles_x;
-    const int64_t R0 = ty * TILE, C0 = tx * TILE;
-    const int rows_valid = (int)min((int64_t)TILE, rows - R0), cols_valid = (int)min((int64_t)TILE, cols - C0);
+    const int64_t R0 = ty * TR, C0 = tx * TILE_C;
+    const int rows_valid = (int)min((int64_t)TR, rows - R0), cols_valid = (int)min((int64_t)TILE_C, cols - C0);
     const int64_t row_chunks = cols >> 3;
 
-    uint4 v[8];
-    bool ok[8];
+    uint4 v[NV];
+    bool ok[NV];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    for (int k = 0; k < NV; ++k) {
         const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
         ok[k] = (r < rows_valid) && (cc * 8 < cols_valid);
         v[k] = make_uint4(0, 0, 0, 0);
         if (ok[k]) v[k] = in[(R0 + r) * row_chunks + (C0 >> 3) + cc];
     }
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    for (int k = 0; k < NV; ++k) {
         const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
         *reinterpret_cast<uint4*>(&tile[r * PITCH + cc * 8]) = v[k];
     }
     __syncthreads();
-    // blocks along columns: a thread owns one column and two row blocks of 32, read from the LDS copy
-    const int c = tid & (TILE - 1);
-    uint32_t w[2][16];
+    // blocks along columns: a thread owns one column and BPT row blocks of 32, read from the LDS copy
+    const int c = tid & (TILE_C - 1);
+    uint32_t w[BPT][16];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int rb = (tid >> 7) * 2 + h;
+    for (int h = 0; h < BPT; ++h) {
+        const int rb = (tid >> 7) * BPT + h;
 #pragma unroll
         for (int i = 0; i < 16; ++i)
             w[h][i] = (uint32_t)tile[(rb * 32 + 2 * i) * PITCH + c] | ((uint32_t)tile[(rb * 32 + 2 * i + 1) * PITCH + c] << 16);
@@ -189,7 +194,7 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
     // blocks along rows, from registers (the global stores overlap the LDS latency above)
     const bool dword_row_scales = (cols & 127) == 0;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    for (int k = 0; k < NV; ++k) {
         const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
         const float amax = group_max_t<4>(chunk_amax(v[k]), 4);
         const int e8 = wire_e8<F>(amax);
@@ -197,7 +202,7 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
         store_codes<F>(row_payload, cidx, code_chunk<F>(v[k], e8), ok[k]);
         const uint32_t sb = (uint32_t)(127 - e8);
         const uint32_t s4 = sb | (__shfl_down(sb, 4, 16) << 8) | (__shfl_down(sb, 8, 16) << 16) | (__shfl_down(sb, 12, 16) << 24);
-        if (dword_row_scales && cols_valid == TILE) {
+        if (dword_row_scales && cols_valid == TILE_C) {
             if (ok[k] && cc == 0) *reinterpret_cast<uint32_t*>(row_scales + (cidx >> 2)) = s4;
         } else if (ok[k] && (cc & 3) == 0) row_scales[cidx >> 2] = (uint8_t)sb;
     }
@@ -205,8 +210,8 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
 
     uint32_t my_scales = 0;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int rb = (tid >> 7) * 2 + h;
+    for (int h = 0; h < BPT; ++h) {
+        const int rb = (tid >> 7) * BPT + h;
         float amax = 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc_amax(amax, w[h][i]);
@@ -223,26 +228,29 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
             uint32_t p[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) p[i] = code_pair<F>(w[h][i], e8);
+            uint32_t d[6];                                                   // 6 x 32 bits = 32 codes
 #pragma unroll
-            for (int g = 0; g < 3; ++g) {                                    // 3 x 64 bits = 32 codes
-                uint64_t acc = 0;
+            for (int g = 0; g < 6; ++g) {
+                d[g] = 0;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const int lo_bit = 12 * i - 64 * g;                      // position of pair i in this 64-bit word
-                    if (lo_bit > -12 && lo_bit < 64) acc |= lo_bit >= 0 ? ((uint64_t)p[i] << lo_bit) : ((uint64_t)p[i] >> (-lo_bit));
+                    const int lo_bit = 12 * i - 32 * g;                      // position of pair i in this word
+                    if (lo_bit > -12 && lo_bit < 32) d[g] |= lo_bit >= 0 ? (p[i] << lo_bit) : (p[i] >> (-lo_bit));
                 }
-                *reinterpret_cast<uint2*>(dst + 8 * g) = make_uint2((uint32_t)acc, (uint32_t)(acc >> 32));
             }
+            *reinterpret_cast<uint2*>(dst) = make_uint2(d[0], d[1]);
+            *reinterpret_cast<uint2*>(dst + 8) = make_uint2(d[2], d[3]);
+            *reinterpret_cast<uint2*>(dst + 16) = make_uint2(d[4], d[5]);
         }
     }
-    if (tid >= TILE) s_cscale[c] = my_scales;
+    if (tid >= TILE_C) s_cscale[c] = my_scales;
     __syncthreads();
 
-    // the transposed payload: a column of the tile is 4 * blk_bytes contiguous bytes, SEGS lanes store one column
+    // the transposed payload: a column of the tile is RB * blk_bytes contiguous bytes, SEGS lanes store one column
     const int64_t col_row_bytes = rows / 32 * blk_bytes;                 // bytes per column in the transposed payload
     const int valid_bytes = rows_valid / 32 * blk_bytes;
 #pragma unroll
-    for (int i = 0; i < TILE * SEGS / WWG; ++i) {
+    for (int i = 0; i < TILE_C * SEGS / WWG; ++i) {
         const int idx = i * WWG + tid, col = idx / SEGS, seg = idx % SEGS;
         if (col < cols_valid && seg * SEG < valid_bytes) {
             uint8_t* dst = col_payload + (C0 + col) * col_row_bytes + (R0 / 32) * blk_bytes + seg * SEG;
@@ -251,13 +259,14 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
             else *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(src);
         }
     }
-    // scale bytes of the column blocks: 4 per column and tile
-    if (tid < TILE && c < cols_valid) {
-        const uint32_t s4 = my_scales | (s_cscale[c] << 16);
+    // scale bytes of the column blocks: RB per column and tile
+    if (tid < TILE_C && c < cols_valid) {
+        const uint32_t sall = my_scales | (s_cscale[c] << (8 * BPT));
         uint8_t* dst = col_scales + (C0 + c) * (rows / 32) + R0 / 32;
-        if ((rows & 127) == 0) *reinterpret_cast<uint32_t*>(dst) = s4;
+        if (RB == 4 && (rows & 127) == 0) *reinterpret_cast<uint32_t*>(dst) = sall;
+        else if (RB == 2 && (rows & 63) == 0) *reinterpret_cast<uint16_t*>(dst) = (uint16_t)sall;
         else
-            for (int b = 0; b < rows_valid / 32; ++b) dst[b] = (uint8_t)(s4 >> (8 * b));
+            for (int b = 0; b < rows_valid / 32; ++b) dst[b] = (uint8_t)(sall >> (8 * b));
     }
 }
 
@@ -332,16 +341,16 @@ extern "C" int mor_mx_quantize_dual(const void* input, void* row_payload, void* 
     if (int rc = validate_wire(input, row_payload, row_scales, rows, cols, fmt, 32)) return rc;
     if (int rc = validate_wire(input, col_payload, col_scales, rows, cols, fmt, 32)) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int64_t tiles = ((rows + TILE - 1) / TILE) * ((cols + TILE - 1) / TILE);
+    const int64_t tiles = ((rows + TILE_ROWS - 1) / TILE_ROWS) * ((cols + TILE_C - 1) / TILE_C);
     if (tiles > 0x7FFFFFFFll) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many tiles");
     const uint4* in = static_cast<const uint4*>(input);
     uint8_t *rp = static_cast<uint8_t*>(row_payload), *rs = static_cast<uint8_t*>(row_scales);
     uint8_t *cp = static_cast<uint8_t*>(col_payload), *cs = static_cast<uint8_t*>(col_scales);
     switch (fmt) {
-        case MOR_FMT_E4M3: k_mx_dual<FMT_E4M3><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
-        case MOR_FMT_E5M2: k_mx_dual<FMT_E5M2><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
-        case MOR_FMT_E3M2: k_mx_dual<FMT_E3M2><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
-        default: k_mx_dual<FMT_E2M3><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        case MOR_FMT_E4M3: k_mx_dual<FMT_E4M3, TILE_ROWS><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        case MOR_FMT_E5M2: k_mx_dual<FMT_E5M2, TILE_ROWS><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        case MOR_FMT_E3M2: k_mx_dual<FMT_E3M2, TILE_ROWS><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        default: k_mx_dual<FMT_E2M3, TILE_ROWS><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
     }
     return mor_check_launch("k_mx_dual");
 }
