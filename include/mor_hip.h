@@ -18,6 +18,9 @@
 #include <stddef.h>
 #include <stdint.h>
 
+/* the library is built with hidden visibility: only these entry points are exported */
+#define MOR_API __attribute__((visibility("default")))
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -49,13 +52,13 @@ extern "C" {
 #define MOR_OP_CHANNEL_SCALING 2
 #define MOR_OP_E8MX 3
 
-const char* mor_last_error(void);
+MOR_API const char* mor_last_error(void);
 
 /* Library version and the offload architecture it was built for. */
-const char* mor_version(void);
+MOR_API const char* mor_version(void);
 
 /* Bytes of device workspace an op needs for this shape (0 for ops that need none). */
-size_t mor_workspace_bytes(int op, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols);
+MOR_API size_t mor_workspace_bytes(int op, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols);
 
 /*
  * fake_quantize / fake_quantize_no_alloc: FQ:1839-1907 (launch decoding FQ:1763-1835,
@@ -66,7 +69,7 @@ size_t mor_workspace_bytes(int op, int64_t rows, int64_t cols, int64_t block_row
  * int32 entries.  output may alias input.  Any shape is accepted (the reference
  * requires even cols and launchable block shapes).
  */
-int mor_fake_quantize(const void* input, void* output, int32_t* meta,
+MOR_API int mor_fake_quantize(const void* input, void* output, int32_t* meta,
                       int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
                       double clamp_threshold, int64_t mode, int64_t sf_type,
                       uint32_t flags, void* stream);
@@ -77,7 +80,7 @@ int mor_fake_quantize(const void* input, void* output, int32_t* meta,
  * (software saturating cast).  The reference has no public op for a forced E2M3; this
  * entry exists for the MX E2M3 benchmark configuration and for tests.
  */
-int mor_block_format(const void* input, void* output,
+MOR_API int mor_block_format(const void* input, void* output,
                      int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
                      int fmt, int64_t sf_type, uint32_t flags, void* stream);
 
@@ -90,7 +93,7 @@ int mor_block_format(const void* input, void* output,
  * global_non_zero / global_error are device pointers to one element each.  output may
  * alias input (the in-place ops).  rows % block_rows == 0 and cols % block_cols == 0.
  */
-int mor_block_scaling(const void* input, void* output, int32_t* meta,
+MOR_API int mor_block_scaling(const void* input, void* output, int32_t* meta,
                       float* global_amax, int32_t* global_non_zero, float* global_error,
                       int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
                       double e4m3_threshold, int64_t ss_mode, int channel,
@@ -98,27 +101,27 @@ int mor_block_scaling(const void* input, void* output, int32_t* meta,
 
 /* fake_quantize_e8mx(_inplace): FQ:2232-2397.  quantize_type 1/2/3 = E8M1/2/3;
  * scaling_strategy 1 = scale by the tensor amax, else no scale.  output may alias input. */
-int mor_e8mx(const void* input, void* output, int64_t rows, int64_t cols,
+MOR_API int mor_e8mx(const void* input, void* output, int64_t rows, int64_t cols,
              int64_t block_rows, int64_t block_cols, int64_t quantize_type, int64_t scaling_strategy,
              void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
 
 /* quant_dequant_e4m3/e5m2/e3m2/e2m3: FQ:1909-1964 (fp32 in, fp32 out, n elements). */
-int mor_quant_dequant(const float* input, float* output, int64_t n, int fmt, void* stream);
+MOR_API int mor_quant_dequant(const float* input, float* output, int64_t n, int fmt, void* stream);
 
 /* e4m3_with_e8_scale_rne / _rz: FQ:1966-2011 (fp32 in, fp32 out, n elements). */
-int mor_e4m3_with_e8_scale(const float* input, float* output, int64_t n, int rne, void* stream);
+MOR_API int mor_e4m3_with_e8_scale(const float* input, float* output, int64_t n, int rne, void* stream);
 
 /*
  * Debug view that the public ops never return: per block amax, the fp32 scale fmax/amax
  * and its biased exponent field (the E8M0 shared exponent of the power-of-two scale,
  * FQ:251-252).  Arrays have ceil(rows/block_rows) x ceil(cols/block_cols) entries.
  */
-int mor_block_stats(const void* input, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
+MOR_API int mor_block_stats(const void* input, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
                     float fmax, float* amax, float* scale, int32_t* e8m0, void* stream);
 
 /* Per block {amax, min non-zero |x|, E4M3 error sum, E5M2 error sum} of the MoR decision
  * (FQ:407-584); error sums are 0 for blocks that did not need them.  4 floats per block. */
-int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
+MOR_API int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
                   double clamp_threshold, int64_t mode, int64_t sf_type, float* stats, void* stream);
 
 /*
@@ -126,7 +129,7 @@ int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t block_r
  * cast over all 2^32 fp32 inputs whose magnitude does not exceed the format maximum.
  * mismatches[0] = E4M3 count, mismatches[1] = E5M2 count (device pointer, 2 x uint64).
  */
-int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
+MOR_API int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
 
 /*
  * MX wire format: the quantized tensor itself instead of its dequantized bf16 image.
@@ -143,21 +146,21 @@ int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
  * E3M2): 32 codes packed little-endian into 24 bytes, element i in bits [6i, 6i + 6) of its block.
  * cols must be a multiple of 32; tensors and payloads 16-byte aligned, scales 4-byte aligned.
  */
-size_t mor_mx_payload_bytes(int64_t rows, int64_t cols, int fmt);
+MOR_API size_t mor_mx_payload_bytes(int64_t rows, int64_t cols, int fmt);
 
 /* Blocks of 32 along rows.  payload: [rows, cols * bits / 8] bytes, scales: [rows, cols / 32]. */
-int mor_mx_quantize(const void* input, void* payload, void* scales, int64_t rows, int64_t cols,
+MOR_API int mor_mx_quantize(const void* input, void* payload, void* scales, int64_t rows, int64_t cols,
                     int fmt, void* stream);
 
 /* Both orientations from one read of the tensor (rows and cols multiples of 32): the row-wise
  * result as above and the column-wise one (blocks of 32 along columns) stored transposed, i.e. what
  * mor_mx_quantize returns for the transposed tensor: col_payload [cols, rows * bits / 8],
  * col_scales [cols, rows / 32].  This is the pair a linear layer needs for dgrad and wgrad. */
-int mor_mx_quantize_dual(const void* input, void* row_payload, void* row_scales, void* col_payload,
+MOR_API int mor_mx_quantize_dual(const void* input, void* row_payload, void* row_scales, void* col_payload,
                          void* col_scales, int64_t rows, int64_t cols, int fmt, void* stream);
 
 /* payload + scales -> bf16 [rows, cols] (blocks of 32 along rows). */
-int mor_mx_dequantize(const void* payload, const void* scales, void* output, int64_t rows,
+MOR_API int mor_mx_dequantize(const void* payload, const void* scales, void* output, int64_t rows,
                       int64_t cols, int fmt, void* stream);
 
 #ifdef __cplusplus

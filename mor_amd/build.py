@@ -7,7 +7,7 @@ SOURCES = [os.path.join(_HERE, "csrc", "mor_kernels.hip"), os.path.join(_HERE, "
 OUT = os.path.join(_HERE, "lib", "libmor_hip.so")
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
     # keep packed fp32 instructions out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
