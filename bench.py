@@ -288,6 +288,14 @@ def wire_format(torch, run, K, W):
             ms = time_launches(torch, fn, K, W)[0]
             out[f"{key}_{name}"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                     "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    # fake quantization of the tensor and of its transpose from one read (2 B read + 4 B written per element + meta)
+    o, ot = torch.empty_like(x), torch.empty_like(x)
+    m, mt = (torch.empty(n // 32, dtype=torch.int32, device="cuda") for _ in range(2))
+    ms = time_launches(torch, lambda: run.cabi.check(L.mor_fake_quantize_dual(x.data_ptr(), o.data_ptr(), m.data_ptr(), ot.data_ptr(),
+                                                                              mt.data_ptr(), rows, cols, 2, 2, run.stream())), K, W)[0]
+    nbytes = 6 * n + 2 * (n // 32) * 4
+    out["fake_quantize_dual_e4m3"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                      "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     return out
 
 

@@ -163,6 +163,19 @@ MOR_API int mor_mx_quantize_dual(const void* input, void* row_payload, void* row
 MOR_API int mor_mx_dequantize(const void* payload, const void* scales, void* output, int64_t rows,
                       int64_t cols, int fmt, void* stream);
 
+/*
+ * Fake quantization of a tensor and of its transpose from one read (no counterpart in the
+ * reference, whose callers run fake_quantize on x and on x.t().contiguous(), FQ:1839-1871 twice):
+ *   output_rows [rows, cols], meta_rows [rows, cols / 32]  == mor_fake_quantize(x,   rows, cols, 1, 32, 0, mode, sf_type)
+ *   output_cols [cols, rows], meta_cols [cols, rows / 32]  == mor_fake_quantize(x^T, cols, rows, 1, 32, 0, mode, sf_type)
+ * bit for bit, for mode 2 (E4M3) or 3 (E5M2), sf_type 1 (fp32 scale) or 2 (power-of-two scale), default
+ * flavour.  rows and cols multiples of 32, 16-byte aligned tensors, outputs distinct from the
+ * input; either meta pointer may be NULL.
+ */
+MOR_API int mor_fake_quantize_dual(const void* input, void* output_rows, int32_t* meta_rows,
+                                   void* output_cols, int32_t* meta_cols, int64_t rows, int64_t cols,
+                                   int64_t mode, int64_t sf_type, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -271,6 +271,133 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
 }
 
 // ------------------------------------------------------------------------------------------------
+// Fake quantization of both orientations from one read: what mor_fake_quantize returns for the tensor with 1 x 32
+// blocks and for its transpose with 1 x 32 blocks (FQ:801-823 per block), the second written transposed.  Same tile
+// scheme as k_mx_dual with bf16 outputs: 2 bytes read and 4 written per element instead of 8 + a transpose.
+// Blocks outside the fast exponent range take the exact path in a non-unrolled loop.
+template <int F, bool E8> __device__ __forceinline__ Scale block_scale(float amax) {
+    if constexpr (E8) return make_scale_e8<F>(amax);
+    else return make_scale(Fmt<F>::fmax / amax);
+}
+
+template <int F, bool E8>
+__global__ __launch_bounds__(WWG) void k_fq_dual(const uint4* in, uint4* out_rows, int32_t* meta_rows, uint16_t* out_cols,
+                                                 int32_t* meta_cols, int64_t rows, int64_t cols, int meta_val) {
+    constexpr int TR = 128;
+    constexpr int PITCH = TILE_C + 8;             // bf16 elements per LDS row (both uses of the buffer)
+    constexpr int NV = TR * (TILE_C / 8) / WWG;   // 8
+    constexpr int BPT = 2;                        // column blocks per thread
+    __shared__ __attribute__((aligned(16))) uint16_t tile[TR * PITCH];
+    const int tid = threadIdx.x;
+    const int64_t tiles_x = (cols + TILE_C - 1) / TILE_C;
+    const int64_t ty = blockIdx.x / tiles_x, tx = blockIdx.x - ty * tiles_x;
+    const int64_t R0 = ty * TR, C0 = tx * TILE_C;
+    const int rows_valid = (int)min((int64_t)TR, rows - R0), cols_valid = (int)min((int64_t)TILE_C, cols - C0);
+    const int64_t row_chunks = cols >> 3;
+
+    uint4 v[NV];
+    bool ok[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+        ok[k] = (r < rows_valid) && (cc * 8 < cols_valid);
+        v[k] = make_uint4(0, 0, 0, 0);
+        if (ok[k]) v[k] = in[(R0 + r) * row_chunks + (C0 >> 3) + cc];
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+        *reinterpret_cast<uint4*>(&tile[r * PITCH + cc * 8]) = v[k];
+    }
+    __syncthreads();
+    const int c = tid & (TILE_C - 1);
+    uint32_t w[BPT][16];
+#pragma unroll
+    for (int h = 0; h < BPT; ++h) {
+        const int rb = (tid >> 7) * BPT + h;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            w[h][i] = (uint32_t)tile[(rb * 32 + 2 * i) * PITCH + c] | ((uint32_t)tile[(rb * 32 + 2 * i + 1) * PITCH + c] << 16);
+    }
+    // blocks along rows, from registers
+    uint32_t slow = 0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+        const float amax = group_max_t<4>(chunk_amax(v[k]), 4);
+        const Scale sc = block_scale<F, E8>(amax);
+        const bool quant = (amax > 0.0f) && sc.fast;
+        const uint4 q = fq_vec_fast<F, E8>(v[k], sc);
+        uint4 o;
+        o.x = quant ? q.x : v[k].x; o.y = quant ? q.y : v[k].y; o.z = quant ? q.z : v[k].z; o.w = quant ? q.w : v[k].w;
+        if ((amax > 0.0f) && !sc.fast) slow |= 1u << k;
+        const int64_t cidx = (R0 + r) * row_chunks + (C0 >> 3) + cc;
+        if (ok[k]) {
+            out_rows[cidx] = o;
+            if (meta_rows && (cc & 3) == 0) meta_rows[cidx >> 2] = meta_val;
+        }
+    }
+    if (slow) {
+#pragma unroll 1
+        for (int k = 0; k < NV; ++k) {
+            if (!((slow >> k) & 1u)) continue;                       // uniform over the 4 lanes of a block
+            const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+            const uint4 x = *reinterpret_cast<const uint4*>(&tile[r * PITCH + cc * 8]);
+            const float amax = group_max_t<4>(chunk_amax(x), 4);
+            const Scale sc = make_scale(Fmt<F>::fmax / amax);
+            uint4 o;
+            o.x = fq_pair_exact<F, E8, false>(x.x, sc); o.y = fq_pair_exact<F, E8, false>(x.y, sc);
+            o.z = fq_pair_exact<F, E8, false>(x.z, sc); o.w = fq_pair_exact<F, E8, false>(x.w, sc);
+            if (ok[k]) out_rows[(R0 + r) * row_chunks + (C0 >> 3) + cc] = o;
+        }
+    }
+    __syncthreads();                              // every thread has its column blocks in registers: reuse the buffer
+
+    // blocks along columns; results go to LDS transposed (PITCH elements per column, 128 of them used)
+    int32_t col_meta_ok = 0;
+#pragma unroll
+    for (int h = 0; h < BPT; ++h) {
+        const int rb = (tid >> 7) * BPT + h;
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc_amax(amax, w[h][i]);
+        const Scale sc = block_scale<F, E8>(amax);
+        uint32_t q[16];
+        if ((amax > 0.0f) && !sc.fast) {
+            const Scale se = make_scale(Fmt<F>::fmax / amax);
+#pragma unroll 1
+            for (int i = 0; i < 16; ++i) q[i] = fq_pair_exact<F, E8, false>(w[h][i], se);
+        } else {
+            const bool quant = amax > 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t f = fq_pair_fast<F, E8>(w[h][i], sc);
+                q[i] = quant ? f : w[h][i];
+            }
+        }
+        uint4* dst = reinterpret_cast<uint4*>(&tile[c * PITCH + rb * 32]);
+        dst[0] = make_uint4(q[0], q[1], q[2], q[3]);
+        dst[1] = make_uint4(q[4], q[5], q[6], q[7]);
+        dst[2] = make_uint4(q[8], q[9], q[10], q[11]);
+        dst[3] = make_uint4(q[12], q[13], q[14], q[15]);
+        col_meta_ok |= (c < cols_valid && rb * 32 < rows_valid) ? (1 << h) : 0;
+    }
+    __syncthreads();
+    // transposed output: a column of the tile is 256 contiguous bytes, 16 lanes store one column
+#pragma unroll
+    for (int i = 0; i < TILE_C * 16 / WWG; ++i) {
+        const int idx = i * WWG + tid, col = idx >> 4, seg = idx & 15;
+        if (col < cols_valid && seg * 8 < rows_valid)
+            *reinterpret_cast<uint4*>(out_cols + (C0 + col) * rows + R0 + seg * 8) = *reinterpret_cast<const uint4*>(&tile[col * PITCH + seg * 8]);
+    }
+    if (meta_cols) {
+#pragma unroll
+        for (int h = 0; h < BPT; ++h)
+            if ((col_meta_ok >> h) & 1) meta_cols[(C0 + c) * (rows / 32) + R0 / 32 + (tid >> 7) * BPT + h] = meta_val;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 template <int F>
 __global__ __launch_bounds__(WWG) void k_mx_dequantize(const uint8_t* payload, const uint8_t* scales, uint4* out, int64_t nchunks) {
     for (int64_t c = (int64_t)blockIdx.x * WWG + threadIdx.x; c < nchunks; c += (int64_t)gridDim.x * WWG) {
@@ -370,4 +497,34 @@ extern "C" int mor_mx_dequantize(const void* payload, const void* scales, void* 
         default: k_mx_dequantize<FMT_E2M3><<<grid, WWG, 0, st>>>(p, s, out, nchunks); break;
     }
     return mor_check_launch("k_mx_dequantize");
+}
+
+extern "C" int mor_fake_quantize_dual(const void* input, void* output_rows, int32_t* meta_rows, void* output_cols,
+                                      int32_t* meta_cols, int64_t rows, int64_t cols, int64_t mode, int64_t sf_type,
+                                      void* stream) {
+    if (!input || !output_rows || !output_cols) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "NULL tensor pointer");
+    if (rows <= 0 || cols <= 0 || rows % 32 || cols % 32)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "rows and cols must be positive multiples of 32 (got %lld x %lld)", (long long)rows, (long long)cols);
+    if ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(output_rows) | reinterpret_cast<uintptr_t>(output_cols)) & 15u)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensors must be 16-byte aligned");
+    if (input == output_rows || input == output_cols)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "the outputs must not alias the input (tiles are read while others are written)");
+    const int qmode = (int)(mode % 10);
+    if (qmode != 2 && qmode != 3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mode must be 2 (E4M3) or 3 (E5M2), got %lld", (long long)mode);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t tiles = ((rows + 127) / 128) * ((cols + TILE_C - 1) / TILE_C);
+    if (tiles > 0x7FFFFFFFll) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many tiles");
+    const uint4* in = static_cast<const uint4*>(input);
+    uint4* orow = static_cast<uint4*>(output_rows);
+    uint16_t* ocol = static_cast<uint16_t*>(output_cols);
+    const bool e8 = (sf_type == 2);
+    const unsigned grid = (unsigned)tiles;
+    if (qmode == 2) {
+        if (e8) k_fq_dual<FMT_E4M3, true><<<grid, WWG, 0, st>>>(in, orow, meta_rows, ocol, meta_cols, rows, cols, 1);
+        else k_fq_dual<FMT_E4M3, false><<<grid, WWG, 0, st>>>(in, orow, meta_rows, ocol, meta_cols, rows, cols, 1);
+    } else {
+        if (e8) k_fq_dual<FMT_E5M2, true><<<grid, WWG, 0, st>>>(in, orow, meta_rows, ocol, meta_cols, rows, cols, 2);
+        else k_fq_dual<FMT_E5M2, false><<<grid, WWG, 0, st>>>(in, orow, meta_rows, ocol, meta_cols, rows, cols, 2);
+    }
+    return mor_check_launch("k_fq_dual");
 }

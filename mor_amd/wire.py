@@ -1,4 +1,4 @@
-"""MX wire format on MI355X: the quantized tensor (element codes + E8M0 scale bytes) instead of its dequantized image.
+"""MX wire format and dual-orientation quantization on MI355X: the quantized tensor (element codes + E8M0 scale bytes) instead of its dequantized image.
 
 The reference's ops only return bf16 (mor/ops.py); these functions are the step next to them in a training loop: the
 payload a scaled-MFMA GEMM consumes.  The quantization is the reference's MX block rule (block modes with sf_type 2,
@@ -73,3 +73,19 @@ def dequantize_mx(payload: Tensor, scales: Tensor, fmt: int = E4M3) -> Tensor:
         out = torch.empty((rows, cols), dtype=torch.bfloat16, device=payload.device)
         _cabi.check(_L.mor_mx_dequantize(payload.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, cols, fmt, _stream(payload)))
     return out
+
+
+def fake_quantize_mx_dual(x: Tensor, mode: int = 2, sf_type: int = 2) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """One read of x: (out, meta) = mor.ops.fake_quantize(x, rows, cols, 1, 32, 0.0, mode, sf_type) and
+    (out_t, meta_t) = the same op on x.t().contiguous(), bit for bit, without materialising the transpose.
+    mode 2 = E4M3, 3 = E5M2; sf_type 1 = fp32 scale, 2 = power-of-two scale."""
+    rows, cols = _check(x, 32)
+    x = x.contiguous()
+    with torch.cuda.device(x.device):
+        out = torch.empty_like(x)
+        out_t = torch.empty((cols, rows), dtype=torch.bfloat16, device=x.device)
+        meta = torch.empty((rows, cols // 32), dtype=torch.int32, device=x.device)
+        meta_t = torch.empty((cols, rows // 32), dtype=torch.int32, device=x.device)
+        _cabi.check(_L.mor_fake_quantize_dual(x.data_ptr(), out.data_ptr(), meta.data_ptr(), out_t.data_ptr(), meta_t.data_ptr(),
+                                              rows, cols, mode, sf_type, _stream(x)))
+    return out, meta, out_t, meta_t

@@ -164,3 +164,18 @@ def mx_dequantize(payload, scales, fmt):
     _cabi.check(L.mor_mx_dequantize(p.data_ptr(), s.data_ptr(), out.data_ptr(), rows, cols, fmt, stream_ptr()))
     torch.cuda.synchronize()
     return to_host_u16(out)
+
+
+def fake_quantize_dual(a_u16, mode, sf_type, want_meta=True):
+    """-> (out [rows, cols], meta [rows, cols/32], out_t [cols, rows], meta_t [cols, rows/32]) through mor_fake_quantize_dual"""
+    L = _cabi.lib()
+    rows, cols = a_u16.shape
+    x = to_dev_u16(a_u16)
+    o = torch.full((rows, cols), 7.0, dtype=torch.bfloat16, device=dev())
+    ot = torch.full((cols, rows), 7.0, dtype=torch.bfloat16, device=dev())
+    m = torch.full((rows, cols // 32), -7, dtype=torch.int32, device=dev())
+    mt = torch.full((cols, rows // 32), -7, dtype=torch.int32, device=dev())
+    _cabi.check(L.mor_fake_quantize_dual(x.data_ptr(), o.data_ptr(), m.data_ptr() if want_meta else None, ot.data_ptr(),
+                                         mt.data_ptr() if want_meta else None, rows, cols, mode, sf_type, stream_ptr()))
+    torch.cuda.synchronize()
+    return to_host_u16(o), m.cpu().numpy(), to_host_u16(ot), mt.cpu().numpy()
