@@ -223,6 +223,17 @@ def other_configs(torch, run, cabi, K, W):
     add("mor_128x128_8192x8192_normal", lambda: run.fake_quantize(x, out, meta, 128, 128, 1e-15, 1, 1), n * 4 + meta.numel() * 4, n)
     add("copy_mode7_8192x8192", lambda: run.fake_quantize(x, out, meta, 128, 128, 0.0, 7, 1), n * 4 + meta.numel() * 4, n)
     add("block_e4m3_128x128_8192x8192_fp32scale", lambda: run.fake_quantize(x, out, meta, 128, 128, 0.0, 2, 1), n * 4 + meta.numel() * 4, n)
+    # the benchmark kernel with nothing left in the 256 MB last-level cache: 6 input / output pairs (1.6 GB) in rotation
+    xs6 = [x] + [x.clone() for _ in range(5)]
+    os6 = [torch.empty_like(x) for _ in range(6)]
+    mx_meta = torch.empty((8192, 256), dtype=torch.int32, device="cuda")
+    turn = [0]
+
+    def rotating():
+        i = turn[0] = (turn[0] + 1) % 6
+        run.fake_quantize(xs6[i], os6[i], mx_meta, 1, 32, 0.0, 2, 2)
+    add("mx_e4m3_8192x8192_rotating_buffers_cold_cache", rotating, n * 4 + (n // 32) * 4, n)
+    del xs6, os6, mx_meta
     # C1: per-tensor E4M3, 4096x4096, scale from the tensor amax (the quantize pass only: 4 B/element)
     x1 = x[:4096, :4096].contiguous()
     o1 = torch.empty_like(x1)
