@@ -251,7 +251,7 @@ __global__ __launch_bounds__(WG) void k_copy(const uint16_t* in, uint16_t* out, 
 // replaced by the input for all-zero groups (FQ:802, 814) and for groups whose scale is outside the fast range; the
 // latter are redone by a second, non-unrolled exact loop.  GT > 0 fixes the group size at compile time; FULL means
 // nchunks is a multiple of NV * 256.
-template <int F, bool E8, int NV, int GT, bool FULL>
+template <int F, bool E8, int NV, int GT, bool FULL, bool SNT = false>
 __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                  int64_t nchunks, int G, int logG, int meta_val) {
     if constexpr (GT > 0) { G = GT; }
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
         r.w = quant ? q.w : v[k].w;
         if ((amax > 0.0f) && !sc.fast) slow |= 1u << k;
         if (FULL || c < nchunks) {
-            out[c] = r;
+            store16<SNT>(out + c, r);
             if (meta_val >= 0 && (c & (G - 1)) == 0) meta[c >> logG] = meta_val;
         }
     }
@@ -307,7 +307,6 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
 }
 
 // ------------------------------------------------------------------------------------------------
-// Per-block look-up tables in LDS for fp32 scales (E4M3 / E5M2, block in the fast range).
 // Division by the block scale without a divide per element: with r = RN(1 / s) (one IEEE division per block),
 // t = c * r; q = fma(fma(-t, s, c), r, t) is the correctly rounded quotient c / s (Markstein) as long as nothing
 // over- or underflows (the fast range) and the significand of s is not all ones (never the case for fmax / amax
@@ -378,7 +377,7 @@ __device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float
 // MOR: per-block format selection (FQ:610-682), else one forced format.  FULL: every block is complete and has
 // exactly NV * 256 chunks, so no predicates.  NT: streaming loads and stores.  Blocks outside the fast range go
 // through generic_block.
-template <bool MOR, bool E8, int NV, bool FULL, bool NT>
+template <bool MOR, bool E8, int NV, bool FULL, int NT>
 __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
     __shared__ float s_f[2][WAVES];
@@ -404,7 +403,7 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
         int cc = ch - r * cpr;
         ok[k] = FULL || ((ch < nch) && (r < rows_valid) && (cc < cols_valid));
         off[k] = (uint32_t)r * row_stride + (uint32_t)cc;
-        if (ok[k]) v[k] = load16<NT>(bin + off[k]);
+        if (ok[k]) v[k] = load16<(NT == 1)>(bin + off[k]);
     }
 
     // pass 1 (registers): amax and min over non-zero magnitudes, FQ:407-485
@@ -488,7 +487,7 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
     if ((fmt < 0) || !(amax > 0.0f)) {
         if (out != in) {
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], v[k]);
+            for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], v[k]);
         }
         return;
     }
@@ -497,10 +496,10 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
             const float r4 = 1.0f / s4.s;            // 1 / s5 = r4 / 128 exactly
             if (fmt == FMT_E4M3) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_div<FMT_E4M3>(v[k], s4.s, r4));
+                for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_div<FMT_E4M3>(v[k], s4.s, r4));
             } else {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f));
+                for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f));
             }
             return;
         }
@@ -509,21 +508,21 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
     switch (fmt) {
         case FMT_E4M3:
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_fast<FMT_E4M3, E8>(v[k], sc));
+            for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_fast<FMT_E4M3, E8>(v[k], sc));
             break;
         case FMT_E5M2:
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_fast<FMT_E5M2, E8>(v[k], sc));
+            for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_fast<FMT_E5M2, E8>(v[k], sc));
             break;
         case FMT_E3M2:
             if constexpr (!MOR) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_fast<FMT_E3M2, E8>(v[k], sc));
+                for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_fast<FMT_E3M2, E8>(v[k], sc));
             }
             break;
         default:
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) store16<NT>(bout + off[k], fq_vec_fast<FMT_E2M3, E8>(v[k], sc));
+            for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_fast<FMT_E2M3, E8>(v[k], sc));
             break;
     }
 }
@@ -667,19 +666,22 @@ static int validate_shape(const void* input, int64_t rows, int64_t cols, int64_t
 
 template <int F, bool E8>
 static void launch_rowgroup_f(const uint4* i4, uint4* o4, int32_t* meta, int64_t nchunks, int G, int meta_val, hipStream_t st) {
-    // small tensors take fewer chunks per workgroup so that every CU still gets several workgroups
+    // small tensors take fewer chunks per workgroup so that every CU still gets several workgroups; outputs of 4 MiB
+    // and more are written with streaming stores, which keeps the input and whatever the caller has in
+    // the last-level cache from being evicted by data nobody reads back soon (measured: 45.6 -> 41.9 us at 8192^2)
     const int lg = ilog2(G);
     if (nchunks >= 8ll * WG * 2048) {
         constexpr int NV = 8;
         const int grid = (int)cdiv(nchunks, (int64_t)NV * WG);
         const bool full = nchunks % ((int64_t)NV * WG) == 0;
-        if (G == 4 && full) k_rowgroup<F, E8, NV, 4, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
-        else if (G == 16 && full) k_rowgroup<F, E8, NV, 16, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
-        else k_rowgroup<F, E8, NV, 0, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+        if (G == 4 && full) k_rowgroup<F, E8, NV, 4, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+        else if (G == 16 && full) k_rowgroup<F, E8, NV, 16, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+        else k_rowgroup<F, E8, NV, 0, false, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
     } else {
         constexpr int NV = 2;
         const int grid = (int)cdiv(nchunks, (int64_t)NV * WG);
-        k_rowgroup<F, E8, NV, 0, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+        if (nchunks * 16 >= ((int64_t)4 << 20)) k_rowgroup<F, E8, NV, 0, false, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+        else k_rowgroup<F, E8, NV, 0, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
     }
 }
 
@@ -698,11 +700,15 @@ static void launch_rowgroup(int fmt, const void* in, void* out, int32_t* meta, i
 template <bool MOR, bool E8, int NV>
 static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, int32_t* meta, float* stats,
                               const Shape& sh, const QuantArgs& qa, int cpr, int shift, hipStream_t st) {
-    // tensors that cannot stay in the 256 MB last-level cache between the read and later uses are streamed
-    const bool nt = full && (sh.rows * sh.cols * 4 > (int64_t)512 << 20);
-    if (nt) k_wgblock<MOR, E8, NV, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
-    else if (full) k_wgblock<MOR, E8, NV, true, false><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
-    else k_wgblock<MOR, E8, NV, false, false><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    // Streaming stores for outputs that do not fit an L2 anyway (>= 4 MiB): the quantized tensor then does not evict
+    // the input or the caller's data from the caches (measured at 8192^2: 42.7 -> 40.4 us, at 4096^2: 13.3 -> 10.3 us).
+    // Tensors whose traffic exceeds twice the 256 MB last-level cache stream their loads as well.
+    const int64_t out_bytes = sh.rows * sh.cols * 2;
+    const int ntm = !full ? 0 : (2 * out_bytes > ((int64_t)512 << 20)) ? 1 : (out_bytes >= ((int64_t)4 << 20)) ? 2 : 0;
+    if (ntm == 1) k_wgblock<MOR, E8, NV, true, 1><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    else if (ntm == 2) k_wgblock<MOR, E8, NV, true, 2><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    else if (full) k_wgblock<MOR, E8, NV, true, 0><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    else k_wgblock<MOR, E8, NV, false, 0><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
 }
 
 template <bool MOR, bool E8>
