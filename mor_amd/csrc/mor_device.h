@@ -48,6 +48,14 @@ template <bool NT> __device__ __forceinline__ void store16(uint4* p, uint4 v) {
     }
 }
 
+// Run-time choice (uniform over the grid).  Outputs of 4 MiB and more do not fit an L2 and are not read back by
+// the kernel that writes them: streaming stores keep them from evicting the input and the caller's data.
+__device__ __forceinline__ bool streams_out(int64_t bf16_elements) { return bf16_elements >= ((int64_t)2 << 20); }
+__device__ __forceinline__ void store16_rt(uint4* p, uint4 v, bool nt) {
+    if (nt) store16<true>(p, v);
+    else store16<false>(p, v);
+}
+
 // ---------------------------------------------------------------- bf16 <-> fp32
 // FQ:38-44: a bf16 is the upper half of an fp32.
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }

@@ -202,12 +202,13 @@ __global__ __launch_bounds__(WG) void k_elementwise_fast(const uint16_t* in, uin
     uint4 v[EW_NV];
 #pragma unroll
     for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = in4[c]; }
+    const bool nt = streams_out(n);
     if (fmt == FMT_E4M3) {
 #pragma unroll
-        for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) out4[c] = fq_vec_fast<FMT_E4M3, E8, true>(v[k], sc); }
+        for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) store16_rt(out4 + c, fq_vec_fast<FMT_E4M3, E8, true>(v[k], sc), nt); }
     } else {
 #pragma unroll
-        for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) out4[c] = fq_vec_fast<FMT_E5M2, E8, true>(v[k], sc); }
+        for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) store16_rt(out4 + c, fq_vec_fast<FMT_E5M2, E8, true>(v[k], sc), nt); }
     }
 #pragma unroll 1
     for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = fq_one_exact<false>(in[i], fmt, E8, sc);
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(WG) void k_copy(const uint16_t* in, uint16_t* out, 
 #pragma unroll
     for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = in4[c]; }
 #pragma unroll
-    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) out4[c] = v[k]; }
+    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) store16_rt(out4 + c, v[k], streams_out(n)); }
     for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = in[i];
 }
 
@@ -1230,7 +1231,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
                     }
                 }
             }
-            if constexpr (WRITE) out4[c] = make_uint4(w[0], w[1], w[2], w[3]);
+            if constexpr (WRITE) store16_rt(out4 + c, make_uint4(w[0], w[1], w[2], w[3]), streams_out(sh.rows * sh.cols));
         }
     } else {
         const int64_t n = sh.rows * sh.cols;
@@ -1267,6 +1268,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
     const uint4* in4 = reinterpret_cast<const uint4*>(in);
     uint4* out4 = reinterpret_cast<uint4*>(out);
     float err = 0.0f;
+    const bool nt = streams_out(sh.rows * sh.cols);
     if (col0 < sh.cols) {
         for (int64_t seg = blockIdx.y; seg < sh.gy * segs_per_block; seg += gridDim.y) {
             const int64_t by = seg / segs_per_block;
@@ -1308,7 +1310,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
                         }
                         err += row_err;
                         if constexpr (WRITE) {
-                            if (r + k < r_end) out4[(r + k) * row_stride + (col0 >> 3)] = make_uint4(w[0], w[1], w[2], w[3]);
+                            if (r + k < r_end) store16_rt(out4 + (r + k) * row_stride + (col0 >> 3), make_uint4(w[0], w[1], w[2], w[3]), nt);
                         }
                     }
                 }
@@ -1452,7 +1454,7 @@ __global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, 
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 w[j] = store_pair<EMU>(e8mx_element<MB, UNIT>(bf16_lo(w[j]), sf, rs, mk), e8mx_element<MB, UNIT>(bf16_hi(w[j]), sf, rs, mk));
-            if (c0 + k * stride < nvec) out4[c0 + k * stride] = make_uint4(w[0], w[1], w[2], w[3]);
+            if (c0 + k * stride < nvec) store16_rt(out4 + c0 + k * stride, make_uint4(w[0], w[1], w[2], w[3]), streams_out(n));
         }
     }
     for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = store_bf16<EMU>(e8mx_element<MB, UNIT>(bf16_one(in[i]), sf, rs, mk));

@@ -320,6 +320,7 @@ __global__ __launch_bounds__(WWG) void k_fq_dual(const uint4* in, uint4* out_row
             w[h][i] = (uint32_t)tile[(rb * 32 + 2 * i) * PITCH + c] | ((uint32_t)tile[(rb * 32 + 2 * i + 1) * PITCH + c] << 16);
     }
     // blocks along rows, from registers
+    const bool nt = streams_out(rows * cols);
     uint32_t slow = 0;
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
@@ -333,7 +334,7 @@ __global__ __launch_bounds__(WWG) void k_fq_dual(const uint4* in, uint4* out_row
         if ((amax > 0.0f) && !sc.fast) slow |= 1u << k;
         const int64_t cidx = (R0 + r) * row_chunks + (C0 >> 3) + cc;
         if (ok[k]) {
-            out_rows[cidx] = o;
+            store16_rt(out_rows + cidx, o, nt);
             if (meta_rows && (cc & 3) == 0) meta_rows[cidx >> 2] = meta_val;
         }
     }
@@ -388,7 +389,7 @@ __global__ __launch_bounds__(WWG) void k_fq_dual(const uint4* in, uint4* out_row
     for (int i = 0; i < TILE_C * 16 / WWG; ++i) {
         const int idx = i * WWG + tid, col = idx >> 4, seg = idx & 15;
         if (col < cols_valid && seg * 8 < rows_valid)
-            *reinterpret_cast<uint4*>(out_cols + (C0 + col) * rows + R0 + seg * 8) = *reinterpret_cast<const uint4*>(&tile[col * PITCH + seg * 8]);
+            store16_rt(reinterpret_cast<uint4*>(out_cols + (C0 + col) * rows + R0 + seg * 8), *reinterpret_cast<const uint4*>(&tile[col * PITCH + seg * 8]), nt);
     }
     if (meta_cols) {
 #pragma unroll
@@ -421,7 +422,7 @@ __global__ __launch_bounds__(WWG) void k_mx_dequantize(const uint8_t* payload, c
         r.y = store_pair<true>(ldexpf(x[2], de), ldexpf(x[3], de));
         r.z = store_pair<true>(ldexpf(x[4], de), ldexpf(x[5], de));
         r.w = store_pair<true>(ldexpf(x[6], de), ldexpf(x[7], de));
-        out[c] = r;
+        store16_rt(out + c, r, streams_out(nchunks * 8));
     }
 }
 
