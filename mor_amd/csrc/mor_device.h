@@ -172,6 +172,7 @@ template <int F, bool EMU> __device__ __forceinline__ float sqdd_fp32_exact(floa
 // Per-block scale state shared by the fast and exact paths.
 struct Scale {
     float s;      // fp32 scale (fmax / amax, or the caller's)
+    float r;      // RN(1 / s) for div_by_scale (fp32-scale paths only)
     int e8;       // exponent field of s minus 127
     bool fast;    // the fast path reproduces the exact one for every finite bf16 element
 };
@@ -181,8 +182,10 @@ __device__ __forceinline__ Scale make_scale(float s) {
     sc.s = s;
     sc.e8 = (int)((f2u(s) >> 23) & 0xFF) - 127;
     // |e8| <= 100 keeps every scaled / descaled exponent inside the normal range, so exponent-field
-    // arithmetic, ldexp and IEEE multiply/divide agree (see the fast paths below).
-    sc.fast = (sc.e8 >= -100) && (sc.e8 <= 100);
+    // arithmetic, ldexp and IEEE multiply/divide agree (see the fast paths below); a significand of all ones is
+    // the one case in which div_by_scale may differ from the IEEE quotient.
+    sc.r = 1.0f / s;
+    sc.fast = (sc.e8 >= -100) && (sc.e8 <= 100) && ((f2u(s) & 0x7FFFFFu) != 0x7FFFFFu);
     return sc;
 }
 
@@ -197,6 +200,7 @@ template <int F> __device__ __forceinline__ Scale make_scale_e8(float amax) {
     const int ea = (int)(b >> 23);
     Scale sc;
     sc.s = 0.0f;
+    sc.r = 0.0f;
     sc.e8 = (127 + eb) - ea - (((b >> 16) & 0x7Fu) > mth ? 1 : 0);
     sc.fast = (ea != 0) && (sc.e8 >= -100) && (sc.e8 <= 100);
     return sc;
@@ -230,24 +234,32 @@ template <int F, bool CLAMP> __device__ __forceinline__ uint32_t e8_pair_fast(ui
     }
 }
 
-// Fast fp32-scale path on a pair: multiply, convert, IEEE divide, round-half-up store.
-template <int F, bool CLAMP> __device__ __forceinline__ uint32_t fp32_pair_fast(uint32_t w, float s) {
-    float x0 = bf16_lo(w), x1 = bf16_hi(w);
-    float d0, d1;
+// Division by the block scale without a divide per element: with r = RN(1 / s) (one IEEE division per block),
+// t = c * r; q = fma(fma(-t, s, c), r, t) is the correctly rounded quotient c / s (Markstein) as long as nothing
+// over- or underflows (the fast range) and the significand of s is not all ones (make_scale clears `fast` then).
+__device__ __forceinline__ float div_by_scale(float c, float s, float r) {
+    const float t = c * r;
+    return fmaf(fmaf(-t, s, c), r, t);
+}
+
+// Fast fp32-scale path on a pair: multiply, convert, divide by the scale, round-half-up store.  Works on
+// magnitudes; the hardware cast keeps the sign (also of a zero result), the software cast returns +0.
+template <int F, bool CLAMP> __device__ __forceinline__ uint32_t fp32_pair_fast(uint32_t w, float s, float r) {
+    const float a = fabsf(bf16_lo(w)) * s, b = fabsf(bf16_hi(w)) * s;
     if constexpr (Fmt<F>::hw) {
-        float v0 = x0 * s, v1 = x1 * s;
+        float v0 = a, v1 = b;
         if constexpr (CLAMP) {   // the reference's hardware cast saturates (user-supplied scales only)
-            v0 = __builtin_amdgcn_fmed3f(v0, -Fmt<F>::fmax, Fmt<F>::fmax);
-            v1 = __builtin_amdgcn_fmed3f(v1, -Fmt<F>::fmax, Fmt<F>::fmax);
+            v0 = fminf(v0, Fmt<F>::fmax);
+            v1 = fminf(v1, Fmt<F>::fmax);
         }
-        uint32_t p = hw_pack2<F>(v0, v1);
-        d0 = hw_unpack<F, 0>(p);
-        d1 = hw_unpack<F, 1>(p);
+        const uint32_t p = hw_pack2<F>(v0, v1);
+        const float q0 = div_by_scale(hw_unpack<F, 0>(p), s, r), q1 = div_by_scale(hw_unpack<F, 1>(p), s, r);
+        return store_pair<false>(q0, q1) | (w & 0x80008000u);
     } else {
-        d0 = cast_sw_exact<F>(x0 * s);
-        d1 = cast_sw_exact<F>(x1 * s);
+        const float d0 = cast_sw_exact<F>(a), d1 = cast_sw_exact<F>(b);
+        const uint32_t sign = ((d0 != 0.0f) ? (w & 0x8000u) : 0u) | ((d1 != 0.0f) ? (w & 0x80000000u) : 0u);
+        return store_pair<false>(div_by_scale(d0, s, r), div_by_scale(d1, s, r)) | sign;
     }
-    return store_pair<false>(d0 / s, d1 / s);
 }
 
 // One element, exact path, any flavour -> fp32 result before the bf16 store.
@@ -260,7 +272,7 @@ template <int F, bool E8, bool EMU> __device__ __forceinline__ float sqdd_exact(
 template <int F, bool E8, bool CLAMP = false>
 __device__ __forceinline__ uint32_t fq_pair_fast(uint32_t w, const Scale& sc) {
     if constexpr (E8) return e8_pair_fast<F, CLAMP>(w, sc.e8);
-    else return fp32_pair_fast<F, CLAMP>(w, sc.s);
+    else return fp32_pair_fast<F, CLAMP>(w, sc.s, sc.r);
 }
 template <int F, bool E8, bool CLAMP = false>
 __device__ __forceinline__ uint4 fq_vec_fast(uint4 v, const Scale& sc) {

@@ -308,16 +308,6 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
 }
 
 // ------------------------------------------------------------------------------------------------
-// Division by the block scale without a divide per element: with r = RN(1 / s) (one IEEE division per block),
-// t = c * r; q = fma(fma(-t, s, c), r, t) is the correctly rounded quotient c / s (Markstein) as long as nothing
-// over- or underflows (the fast range) and the significand of s is not all ones (never the case for fmax / amax
-// with a bf16 amax; the callers check it anyway).
-__device__ __forceinline__ float div_by_scale(float c, float s, float r) {
-    const float t = c * r;
-    return fmaf(fmaf(-t, s, c), r, t);
-}
-__device__ __forceinline__ bool scale_divides(float s) { return (f2u(s) & 0x7FFFFFu) != 0x7FFFFFu; }
-
 // quantize one packed word with an fp32 scale: |x| * s, hardware convert, divide by s, round-half-up store, sign
 template <int F> __device__ __forceinline__ uint32_t fq_pair_div(uint32_t w, float s, float r) {
     const uint32_t p = hw_pack2<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s);
@@ -426,7 +416,7 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
 
     // scales of the two fp8 formats; the fp6 scales differ from s4 by 2^4 / 2^6, inside the margin of `fast`
     const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
-    if (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && scale_divides(s4.s))) {           // uniform over the workgroup
+    if (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast)) {           // uniform over the workgroup
         generic_block<false>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
                              sh, qa, E8, bid, s_f, s_u);
         return;
