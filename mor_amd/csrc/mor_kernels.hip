@@ -1,7 +1,7 @@
 // HIP kernels and C ABI of the MoR fake-quantization path for MI355X (gfx950, wave64).
 //
 // One pass over HBM wherever a quantization block fits in registers:
-//   k_rowgroup   blocks 1 x 8G elements (G = 1..64 lanes, 16-byte loads; the MX 1x32 case is G = 4):
+//   k_rowgroup   blocks 1 x 8G elements (G = 1..256 lanes, 16-byte loads; the MX 1x32 case is G = 4):
 //                amax by DPP inside the lane group, quantize from registers, 16-byte stores.
 //   k_wgblock    one 256-thread workgroup per block of up to 16384 elements (128x128 tiles, 1x4096 rows):
 //                the block lives in registers as 16-byte vectors; amax / min-nonzero / MoR error sums by
@@ -250,8 +250,8 @@ __global__ __launch_bounds__(WG) void k_copy(const uint16_t* in, uint16_t* out, 
 // consecutive chunks held by G consecutive lanes.  A workgroup owns NV * 256 consecutive chunks and issues all of
 // its loads before it computes.  The main path is branch-free: the fast result is computed for every chunk and
 // replaced by the input for all-zero groups (FQ:802, 814) and for groups whose scale is outside the fast range; the
-// latter are redone by a second, non-unrolled exact loop.  GT > 0 fixes the group size at compile time; FULL means
-// nchunks is a multiple of NV * 256.
+// latter are redone by a second, non-unrolled exact loop.  GT > 0 fixes the group size at compile time (GT = 128 / 256:
+// a block spans 2 / 4 waves, whose maxima meet in LDS); FULL means nchunks is a multiple of NV * 256.
 template <int F, bool E8, int NV, int GT, bool FULL, bool SNT = false>
 __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                  int64_t nchunks, int G, int logG, int meta_val) {
@@ -264,13 +264,35 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
         v[k] = make_uint4(0, 0, 0, 0);
         if (FULL || c < nchunks) v[k] = in[c];
     }
+    // groups wider than a wave (GT = 128 / 256 lanes): the waves' maxima meet in LDS, once for all NV chunks
+    float wide_amax[NV];
+    if constexpr (GT > 64) {
+        __shared__ float s_am[NV][WAVES];
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            float a = 0.0f;
+            acc_amax(a, v[k].x); acc_amax(a, v[k].y); acc_amax(a, v[k].z); acc_amax(a, v[k].w);
+            a = group_max_t<64>(a, 64);
+            if (lane == 0) s_am[k][wave] = a;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < NV; ++k)
+            wide_amax[k] = (GT == 256) ? fmaxf(fmaxf(s_am[k][0], s_am[k][1]), fmaxf(s_am[k][2], s_am[k][3]))
+                                       : fmaxf(s_am[k][wave & 2], s_am[k][(wave & 2) + 1]);
+    }
+    const bool snt = SNT || (GT > 64 && streams_out(nchunks * 8));
     uint32_t slow = 0;
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         int64_t c = base + k * WG;
         float amax = 0.0f;
-        acc_amax(amax, v[k].x); acc_amax(amax, v[k].y); acc_amax(amax, v[k].z); acc_amax(amax, v[k].w);
-        amax = group_max_t<GT>(amax, G);
+        if constexpr (GT > 64) amax = wide_amax[k];
+        else {
+            acc_amax(amax, v[k].x); acc_amax(amax, v[k].y); acc_amax(amax, v[k].z); acc_amax(amax, v[k].w);
+            amax = group_max_t<GT>(amax, G);
+        }
         Scale sc;
         if constexpr (E8) sc = make_scale_e8<F>(amax);
         else sc = make_scale(Fmt<F>::fmax / amax);
@@ -283,26 +305,42 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
         r.w = quant ? q.w : v[k].w;
         if ((amax > 0.0f) && !sc.fast) slow |= 1u << k;
         if (FULL || c < nchunks) {
-            store16<SNT>(out + c, r);
+            if constexpr (GT > 64) store16_rt(out + c, r, snt);
+            else store16<SNT>(out + c, r);
             if (meta_val >= 0 && (c & (G - 1)) == 0) meta[c >> logG] = meta_val;
         }
     }
     if (slow) {
+        if constexpr (GT > 64) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                int64_t c = base + k * WG;
+                if (!((slow >> k) & 1u) || !(FULL || c < nchunks)) continue;
+                const Scale sc = make_scale(Fmt<F>::fmax / wide_amax[k]);
+                uint4 r;
+                r.x = fq_pair_exact<F, E8, false>(v[k].x, sc);
+                r.y = fq_pair_exact<F, E8, false>(v[k].y, sc);
+                r.z = fq_pair_exact<F, E8, false>(v[k].z, sc);
+                r.w = fq_pair_exact<F, E8, false>(v[k].w, sc);
+                out[c] = r;
+            }
+        } else {
 #pragma unroll 1
-        for (int k = 0; k < NV; ++k) {
-            if (!((slow >> k) & 1u)) continue;
-            int64_t c = base + k * WG;
-            uint4 x = in[c];                    // when out == in this is the input again: it was stored back above
-            float amax = 0.0f;
-            acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
-            amax = group_max_t<GT>(amax, G);
-            const Scale sc = make_scale(Fmt<F>::fmax / amax);
-            uint4 r;
-            r.x = fq_pair_exact<F, E8, false>(x.x, sc);
-            r.y = fq_pair_exact<F, E8, false>(x.y, sc);
-            r.z = fq_pair_exact<F, E8, false>(x.z, sc);
-            r.w = fq_pair_exact<F, E8, false>(x.w, sc);
-            out[c] = r;
+            for (int k = 0; k < NV; ++k) {
+                if (!((slow >> k) & 1u)) continue;
+                int64_t c = base + k * WG;
+                uint4 x = in[c];                    // when out == in this is the input again: it was stored back above
+                float amax = 0.0f;
+                acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
+                amax = group_max_t<GT>(amax, G);
+                const Scale sc = make_scale(Fmt<F>::fmax / amax);
+                uint4 r;
+                r.x = fq_pair_exact<F, E8, false>(x.x, sc);
+                r.y = fq_pair_exact<F, E8, false>(x.y, sc);
+                r.z = fq_pair_exact<F, E8, false>(x.z, sc);
+                r.w = fq_pair_exact<F, E8, false>(x.w, sc);
+                out[c] = r;
+            }
         }
     }
 }
@@ -661,6 +699,13 @@ static void launch_rowgroup_f(const uint4* i4, uint4* o4, int32_t* meta, int64_t
     // and more are written with streaming stores, which keeps the input and whatever the caller has in
     // the last-level cache from being evicted by data nobody reads back soon (measured: 45.6 -> 41.9 us at 8192^2)
     const int lg = ilog2(G);
+    if (G > 64) {                         // 128 or 256 lanes per block: rows of 1024 / 2048 elements
+        constexpr int NV = 2;
+        const int grid = (int)cdiv(nchunks, (int64_t)NV * WG);
+        if (G == 128) k_rowgroup<F, E8, NV, 128, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+        else k_rowgroup<F, E8, NV, 256, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+        return;
+    }
     if (nchunks >= 8ll * WG * 2048) {
         constexpr int NV = 8;
         const int grid = (int)cdiv(nchunks, (int64_t)NV * WG);
@@ -695,11 +740,14 @@ static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, i
     // the input or the caller's data from the caches (measured at 8192^2: 42.7 -> 40.4 us, at 4096^2: 13.3 -> 10.3 us).
     // Tensors whose traffic exceeds twice the 256 MB last-level cache stream their loads as well.
     const int64_t out_bytes = sh.rows * sh.cols * 2;
-    const int ntm = !full ? 0 : (2 * out_bytes > ((int64_t)512 << 20)) ? 1 : (out_bytes >= ((int64_t)4 << 20)) ? 2 : 0;
-    if (ntm == 1) k_wgblock<MOR, E8, NV, true, 1><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
-    else if (ntm == 2) k_wgblock<MOR, E8, NV, true, 2><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
-    else if (full) k_wgblock<MOR, E8, NV, true, 0><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
-    else k_wgblock<MOR, E8, NV, false, 0><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift);
+    const int ntm = (2 * out_bytes > ((int64_t)512 << 20)) ? 1 : (out_bytes >= ((int64_t)4 << 20)) ? 2 : 0;
+#define MOR_WGBLOCK(FULL, NT) k_wgblock<MOR, E8, NV, FULL, NT><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift)
+    if (full) {
+        if (ntm == 1) MOR_WGBLOCK(true, 1); else if (ntm == 2) MOR_WGBLOCK(true, 2); else MOR_WGBLOCK(true, 0);
+    } else {
+        if (ntm == 1) MOR_WGBLOCK(false, 1); else if (ntm == 2) MOR_WGBLOCK(false, 2); else MOR_WGBLOCK(false, 0);
+    }
+#undef MOR_WGBLOCK
 }
 
 template <bool MOR, bool E8>
@@ -758,7 +806,7 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
     const bool vec_ok = fast_ok && aligned16(input) && (!output || aligned16(output)) && cols % 8 == 0 && bcols % 8 == 0
                         && brows * (cols / 8) < 0x7FFFFFFFll;
     const int64_t G = bcols / 8;
-    if (qa.qmode == 2 && !stats && output && vec_ok && brows == 1 && cols % bcols == 0 && is_pow2(G) && G <= 64) {
+    if (qa.qmode == 2 && !stats && output && vec_ok && brows == 1 && cols % bcols == 0 && is_pow2(G) && G <= 256) {
         if (e8) launch_rowgroup<true>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
         else launch_rowgroup<false>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
         return mor_check_launch("k_rowgroup");

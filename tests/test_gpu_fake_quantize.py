@@ -87,6 +87,9 @@ SHAPES = [
     (64, 256, 1, 32),                 # row groups of 4 lanes (MX)
     (16, 1024, 1, 8),                 # 1 lane per block
     (8, 2048, 1, 512),                # 64 lanes per block
+    (7, 2048, 1, 1024),               # 128 lanes per block: two waves meet in LDS; 7 rows leave a partial workgroup
+    (5, 2048, 1, 2048),               # 256 lanes per block: the whole workgroup
+    (8200, 1024, 1, 1024),            # 128 lanes, 16 MiB output (streaming stores)
     (32, 4096, 1, 4096),              # workgroup per row
     (256, 384, 128, 128),             # workgroup per tile
     (200, 256, 128, 128),             # partial tile rows
@@ -188,6 +191,16 @@ def test_extreme_exponents(G):
     a[5] = rng.integers(0x0080, 0x1000, 256)
     a[6] = rng.integers(0x7000, 0x7F80, 256)
     a[7, ::2] = rng.integers(0x0001, 0x7F80, 128)
+    wide = np.zeros((8, 2048), np.uint16)                # rows of 1024 / 2048 elements: blocks spanning 2 / 4 waves
+    for r in range(8):
+        wide[r] = np.tile(a[r], 8)
+    for (br, bc) in ((1, 1024), (1, 2048)):
+        for mode, sf in ((2, 1), (2, 2), (3, 1), (3, 2)):
+            print("extreme wide", br, bc, mode, sf, flush=True)
+            out, meta = G.fake_quantize(wide, br, bc, 1e-15, mode, sf)
+            want, wmeta = O.fake_quantize(wide, br, bc, 1e-15, mode, sf)
+            assert np.array_equal(meta, wmeta), (br, bc, mode, sf)
+            assert_same(out, want, f"extreme wide {br}x{bc} mode {mode} sf {sf}")
     for (br, bc) in ((1, 32), (1, 256), (8, 256)):
         for mode, sf in ((2, 1), (2, 2), (3, 1), (3, 2), (1, 1), (1, 2), (101, 2)):
             print("extreme", br, bc, mode, sf, flush=True)
