@@ -1378,26 +1378,126 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
     }
 }
 
-// pass 3 (FQ:1178-1241): total error (fixed summation order), the bf16 decision, the scalar outputs
-__global__ __launch_bounds__(WG) void k_bs_finalize(const uint32_t* ws, int npartials, float threshold, int32_t* meta,
-                                                    float* gamax_o, int32_t* gnnz_o, float* gerr_o) {
+// pass 3 (FQ:1178-1241): total error (fixed summation order), the bf16 decision, the scalar outputs.
+// npart_stats > 0: the tensor amax and the non-zero count are still per-workgroup partials (single-pass kernel)
+// and are reduced here; otherwise they are in the header words.
+__global__ __launch_bounds__(WG) void k_bs_finalize(const uint32_t* ws, int npartials, int npart_stats, float threshold,
+                                                    int32_t* meta, float* gamax_o, int32_t* gnnz_o, float* gerr_o) {
     __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
     const float* part = reinterpret_cast<const float*>(ws) + WS_ERR;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float gamax = u2f(ws[0]);
+    int gnnz = (int)ws[1];
+    if (npart_stats > 0) {
+        gamax = reduce_partial_amax(ws, npart_stats, s_f);
+        const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
+        int n = 0;
+#pragma unroll 8
+        for (int i = threadIdx.x; i < npart_stats; i += WG) n += pn[i];
+        n = wave_sum_i(n);
+        if (lane == 0) s_i[wave] = n;
+        __syncthreads();
+        gnnz = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    }
     float acc = 0.0f;
 #pragma unroll 8
     for (int i = threadIdx.x; i < npartials; i += WG) acc += part[i];
     acc = wave_sum(acc);
+    __syncthreads();
     if (lane == 0) s_f[wave] = acc;
     __syncthreads();
     if (threadIdx.x == 0) {
         const float gerr = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
-        const int gnnz = (int)ws[1];
         const float avg = gerr / (float)gnnz;        // 0 / 0 = NaN on an all-zero tensor: not above the threshold
         meta[0] = (avg > threshold) ? 3 : 1;
-        gamax_o[0] = u2f(ws[0]);
+        gamax_o[0] = gamax;
         gnnz_o[0] = gnnz;
         gerr_o[0] = gerr;
+    }
+}
+
+// Single pass for the strategies whose scale depends on the block alone (ss_mode 2 and 3, FQ:1079-1088), out of
+// place: one workgroup per block of up to 16384 elements holds it in registers (as k_wgblock does), finds amax and
+// the non-zero count, quantizes, accumulates the relative error and stores -- one read and one write of the tensor
+// instead of two reads.  Workgroups walk the blocks grid-stride and publish one partial each of the tensor amax, the
+// non-zero count and the error sum.  A block whose scale is outside the fast range is redone from memory with the
+// exact arithmetic.
+template <bool E8, int NV, bool FULL>
+__global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, uint32_t* ws, Shape sh, int ss_mode,
+                                                 int cpr, int cpr_shift, int64_t nblocks) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3);
+    const int nch = (int)sh.brows * cpr;
+    const bool nt = streams_out(sh.rows * sh.cols);
+    float gmax = 0.0f, err = 0.0f;
+    int nnz_total = 0;
+    for (int64_t bid = blockIdx.x; bid < nblocks; bid += gridDim.x) {
+        const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+        const int64_t base = by * sh.brows * row_stride + ((bx * sh.bcols) >> 3);
+        uint4 v[NV];
+        uint32_t off[NV];
+        bool ok[NV];
+        float amax = 0.0f;
+        int nnz = 0;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int ch = k * WG + tid;
+            const int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
+            ok[k] = FULL || (ch < nch);
+            off[k] = (uint32_t)r * row_stride + (uint32_t)(ch - r * cpr);
+            v[k] = make_uint4(0, 0, 0, 0);
+            if (ok[k]) v[k] = in[base + off[k]];
+        }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) acc_amax_nnz(amax, nnz, v[k]);
+        amax = group_max(amax, 64);
+        __syncthreads();                          // the previous block's readers of s_f are done
+        if (lane == 0) s_f[wave] = amax;
+        __syncthreads();
+        amax = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        gmax = fmaxf(gmax, amax);
+        nnz_total += nnz;
+        const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
+        if (sc.fast) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                uint4 q;
+                q.x = bs_pair_fast<E8>(v[k].x, sc, sc.r, err);
+                q.y = bs_pair_fast<E8>(v[k].y, sc, sc.r, err);
+                q.z = bs_pair_fast<E8>(v[k].z, sc, sc.r, err);
+                q.w = bs_pair_fast<E8>(v[k].w, sc, sc.r, err);
+                if (ok[k]) store16_rt(out + base + off[k], q, nt);
+            }
+        } else {
+            const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in);
+            uint16_t* out16 = reinterpret_cast<uint16_t*>(out);
+            const int64_t e0 = by * sh.brows * sh.cols + bx * sh.bcols;
+#pragma unroll 1
+            for (int64_t i = tid; i < sh.brows * sh.bcols; i += WG) {
+                const int64_t r = i / sh.bcols, c = i - r * sh.bcols;
+                const float q = bs_element<E8, false>(bf16_one(in16[e0 + r * sh.cols + c]), sc, err);
+                out16[e0 + r * sh.cols + c] = store_bf16<false>(q);
+            }
+        }
+    }
+    err = wave_sum(err);
+    nnz_total = wave_sum_i(nnz_total);
+    gmax = group_max(gmax, 64);
+    __syncthreads();
+    if (lane == 0) { s_f[wave] = err; s_i[wave] = nnz_total; }
+    __syncthreads();
+    const float e = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+    const int n = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    __syncthreads();
+    if (lane == 0) s_f[wave] = gmax;
+    __syncthreads();
+    if (tid == 0) {
+        reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = e;
+        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
+        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
     }
 }
 
@@ -1563,6 +1663,30 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
     const int vec = (aligned16(input) && aligned16(output) && cols % 8 == 0) ? 1 : 0;
     const bool col = (bcols == 1 && brows > 1);
 
+    // block-local scales, out of place: one pass
+    const int64_t blk_chunks = (bcols % 8 == 0) ? brows * (bcols / 8) : 0;
+    if (!inplace && !emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG / 2 && blk_chunks <= 8 * WG
+        && brows * (cols / 8) < 0x7FFFFFFFll) {
+        const int cpr = (int)(bcols / 8);
+        const int shift = is_pow2(cpr) ? ilog2(cpr) : -1;
+        const int nv = (int)cdiv(blk_chunks, WG);
+        const int NVc = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
+        const bool full = blk_chunks == (int64_t)NVc * WG;
+        const int grid = (int)std::min<int64_t>(nb, MAX_PARTIALS);
+        const uint4* i4 = static_cast<const uint4*>(input);
+        uint4* o4 = static_cast<uint4*>(output);
+#define MOR_BS_FUSED(E8, NV) do { \
+        if (full) k_bs_fused<E8, NV, true><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb); \
+        else k_bs_fused<E8, NV, false><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb); } while (0)
+        if (ss_mode == 2) { switch (NVc) { case 1: MOR_BS_FUSED(true, 1); break; case 2: MOR_BS_FUSED(true, 2); break; case 4: MOR_BS_FUSED(true, 4); break; default: MOR_BS_FUSED(true, 8); break; } }
+        else { switch (NVc) { case 1: MOR_BS_FUSED(false, 1); break; case 2: MOR_BS_FUSED(false, 2); break; case 4: MOR_BS_FUSED(false, 4); break; default: MOR_BS_FUSED(false, 8); break; } }
+#undef MOR_BS_FUSED
+        k_bs_finalize<<<1, WG, 0, st>>>(ws, grid, grid, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        const int64_t n_all = rows * cols;
+        k_copy_if<<<grid_for(n_all / 8, 16), WG, 0, st>>>(in16, out16, meta, 3, n_all, n_all / 8);
+        return mor_check_launch("mor_block_scaling (single pass)");
+    }
+
     // pass 1: per-block amax, per-workgroup partials of the tensor amax and the non-zero count
     const int64_t G = bcols / 8;
     int npart;
@@ -1599,7 +1723,7 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
         const dim3 grid(gx, (unsigned)std::min<int64_t>(segs, std::max<int64_t>(MAX_PARTIALS / gx, 1)));
         if (inplace) k_bs_quant_col<false, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 0, sh, rows_per_wg);
         else k_bs_quant_col<true, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 0, sh, rows_per_wg);
-        k_bs_finalize<<<1, WG, 0, st>>>(ws, (int)(grid.x * grid.y), (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        k_bs_finalize<<<1, WG, 0, st>>>(ws, (int)(grid.x * grid.y), 0, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
         if (inplace) k_bs_quant_col<true, false><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 1, sh, rows_per_wg);
     } else {
         const bool vec2 = vec && (col || bcols % 8 == 0) && n / 8 < 0xFFFFFFFFll;
@@ -1608,7 +1732,7 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
         DivU32 d0 = make_div((uint32_t)std::max<int64_t>(cols / 8, 1)), d1 = make_div((uint32_t)brows),
                d2 = make_div((uint32_t)std::max<int64_t>(bcols / 8, 1)), d3 = make_div((uint32_t)bcols);
         dispatch_bs_quant(e8, emu, col, !inplace, true, grid2, st, in16, out16, ws, blocks, meta, 0, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
-        k_bs_finalize<<<1, WG, 0, st>>>(ws, grid2, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        k_bs_finalize<<<1, WG, 0, st>>>(ws, grid2, 0, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
         if (inplace) dispatch_bs_quant(e8, emu, col, true, false, grid2, st, in16, out16, ws, blocks, meta, 1, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
     }
     if (!inplace) {

@@ -40,7 +40,11 @@ def check_scaling(G, a, br, bc, thr, ss, channel, flags=0, inplace=False):
 @pytest.mark.parametrize("ss", [1, 2, 3, 4])
 @pytest.mark.parametrize("shape", [(256, 256, 128, 128, False), (256, 256, 1, 256, True), (256, 256, 256, 1, True),
                                    (64, 512, 1, 32, True), (96, 80, 32, 16, False), (60, 36, 20, 12, False),
-                                   (512, 40, 128, 1, True)])
+                                   (512, 40, 128, 1, True),
+                                   # single-pass kernel (ss_mode 2 / 3): whole rows, 128 lanes, odd chunks per row,
+                                   # more blocks than partial slots
+                                   (64, 4096, 1, 4096, True), (32, 2048, 1, 1024, True), (64, 240, 16, 120, False),
+                                   (9000, 1024, 1, 1024, True)])
 def test_scaling_fixture_and_random(G, ss, shape):
     rows, cols, br, bc, channel = shape
     if rows == 256 and cols == 256:
