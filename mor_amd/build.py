@@ -30,5 +30,28 @@ def build_hip(verbose=False):
     return OUT
 
 
+TORCH_BINDING_SRC = os.path.join(_HERE, "csrc", "torch_binding.cpp")
+TORCH_BINDING_OUT = os.path.join(_HERE, "lib", "libmor_torch.so")
+
+
+def build_torch_binding(verbose=False):
+    """The C++ operator registrations (no kernels): plain g++ against torch's headers and libmor_hip.so."""
+    import torch
+    from torch.utils import cpp_extension as ce
+    tlib = ce.library_paths()[0]
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}"]
+    cmd += [f"-I{p}" for p in ce.include_paths()] + ["-I/opt/rocm/include", TORCH_BINDING_SRC, "-o", TORCH_BINDING_OUT,
+            f"-L{tlib}", "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_hip", "-lc10_hip",
+            f"-L{os.path.dirname(OUT)}", "-lmor_hip", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"g++ failed:\n{res.stdout}")
+    return TORCH_BINDING_OUT
+
+
 if __name__ == "__main__":
     print(build_hip(verbose=True))
+    print(build_torch_binding(verbose=True))

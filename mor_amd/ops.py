@@ -39,6 +39,8 @@ def set_flavour(name: str) -> None:
     global _flags
     _flags = {"kernel": _cabi.FLAG_DEFAULT, "torch_emulation": _cabi.FLAG_TORCH_EMULATION,
               "software_cast": _cabi.FLAG_SOFTWARE_CAST}[name]
+    if _native is not None:
+        _native.mor_torch_set_flags(_flags)
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -188,27 +190,55 @@ def _e8_scale_impl(input, dim_x, dim_y, rne):
     return out
 
 
-# registrations for the CUDA key: FQ:2663-2678
-_lib.impl("fake_quantize", _fake_quantize_impl, "CUDA")
-_lib.impl("fake_quantize_no_alloc", _fake_quantize_no_alloc_impl, "CUDA")
-_lib.impl("quant_dequant_e4m3", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E4M3), "CUDA")
-_lib.impl("quant_dequant_e5m2", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E5M2), "CUDA")
-_lib.impl("quant_dequant_e3m2", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E3M2), "CUDA")
-_lib.impl("quant_dequant_e2m3", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E2M3), "CUDA")
-_lib.impl("e4m3_with_e8_scale_rne", lambda i, x, y, bx, by: _e8_scale_impl(i, x, y, 1), "CUDA")
-_lib.impl("e4m3_with_e8_scale_rz", lambda i, x, y, bx, by: _e8_scale_impl(i, x, y, 0), "CUDA")
-_lib.impl("fake_quantize_block_scaling", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, False, False), "CUDA")
-_lib.impl("fake_quantize_block_scaling_inplace", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, False, True), "CUDA")
-_lib.impl("fake_quantize_channel_scaling", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, True, False), "CUDA")
-_lib.impl("fake_quantize_channel_scaling_inplace", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, True, True), "CUDA")
-_lib.impl("fake_quantize_e8mx", lambda i, x, y, bx, by, q, s: _e8mx_impl(i, x, y, bx, by, q, s), "CUDA")
+# registrations for the CUDA key: FQ:2663-2678.  The C++ registrations of csrc/torch_binding.cpp (libmor_torch.so)
+# are used when that library has been built: the same checks, allocations and C ABI calls without the interpreter
+# (about 6 instead of 14 microseconds per call).  The Python implementations below are the same path otherwise.
+def _load_native():
+    import ctypes
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libmor_torch.so")
+    if os.environ.get("MOR_PYTHON_OPS") == "1" or not os.path.exists(path):
+        return None
+    torch.ops.load_library(path)
+    lib = ctypes.CDLL(path)
+    lib.mor_torch_set_flags.argtypes = [ctypes.c_uint32]
+    lib.mor_torch_set_flags.restype = None
+    return lib
+
+
+_native = _load_native()
+
+
+class _PythonImpls:
+    """Registers an implementation only when the C++ ones are not loaded."""
+
+    @staticmethod
+    def impl(name, fn, key):
+        if _native is None:
+            _lib.impl(name, fn, key)
+
+
+_reg = _PythonImpls
+_reg.impl("fake_quantize", _fake_quantize_impl, "CUDA")
+_reg.impl("fake_quantize_no_alloc", _fake_quantize_no_alloc_impl, "CUDA")
+_reg.impl("quant_dequant_e4m3", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E4M3), "CUDA")
+_reg.impl("quant_dequant_e5m2", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E5M2), "CUDA")
+_reg.impl("quant_dequant_e3m2", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E3M2), "CUDA")
+_reg.impl("quant_dequant_e2m3", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E2M3), "CUDA")
+_reg.impl("e4m3_with_e8_scale_rne", lambda i, x, y, bx, by: _e8_scale_impl(i, x, y, 1), "CUDA")
+_reg.impl("e4m3_with_e8_scale_rz", lambda i, x, y, bx, by: _e8_scale_impl(i, x, y, 0), "CUDA")
+_reg.impl("fake_quantize_block_scaling", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, False, False), "CUDA")
+_reg.impl("fake_quantize_block_scaling_inplace", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, False, True), "CUDA")
+_reg.impl("fake_quantize_channel_scaling", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, True, False), "CUDA")
+_reg.impl("fake_quantize_channel_scaling_inplace", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, True, True), "CUDA")
+_reg.impl("fake_quantize_e8mx", lambda i, x, y, bx, by, q, s: _e8mx_impl(i, x, y, bx, by, q, s), "CUDA")
 
 
 def _e8mx_inplace_impl(input, dim_x, dim_y, block_x, block_y, quantize_type, scaling_strategy, result):
     _e8mx_impl(input, dim_x, dim_y, block_x, block_y, quantize_type, scaling_strategy, result)
 
 
-_lib.impl("fake_quantize_e8mx_inplace", _e8mx_inplace_impl, "CUDA")
+_reg.impl("fake_quantize_e8mx_inplace", _e8mx_inplace_impl, "CUDA")
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -327,11 +357,14 @@ def e4m3_with_e8_scale_rz(a: Tensor, dim_x: int, dim_y: int, block_x: int, block
 
 
 # (op, number of non-tensor arguments that get a None gradient); fake_quantize_e8mx_inplace has no autograd
-# registration in the reference either (mor/ops.py:104-106)
+# registration in the reference either (mor/ops.py:104-106).  The four differentiable forward ops have their
+# straight-through autograd in C++ when libmor_torch.so is loaded.
+_NATIVE_AUTOGRAD = ("fake_quantize", "fake_quantize_block_scaling", "fake_quantize_channel_scaling", "fake_quantize_e8mx")
 for _name, _n in (("fake_quantize", 7), ("fake_quantize_no_alloc", 8),
                   ("fake_quantize_block_scaling", 6), ("fake_quantize_block_scaling_inplace", 6),
                   ("fake_quantize_channel_scaling", 6), ("fake_quantize_channel_scaling_inplace", 6),
                   ("fake_quantize_e8mx", 6),
                   ("quant_dequant_e4m3", 4), ("quant_dequant_e5m2", 4), ("quant_dequant_e2m3", 4), ("quant_dequant_e3m2", 4),
                   ("e4m3_with_e8_scale_rne", 4), ("e4m3_with_e8_scale_rz", 4)):
-    torch.library.register_autograd(f"mor::{_name}", _ste(_n), setup_context=_noop_setup_context)
+    if _native is None or _name not in _NATIVE_AUTOGRAD:
+        torch.library.register_autograd(f"mor::{_name}", _ste(_n), setup_context=_noop_setup_context)
