@@ -275,6 +275,12 @@ def other_configs(torch, run, cabi, K, W):
     ms_ = torch.empty((1, 1), dtype=torch.int32, device="cuda")
     ms, wall = time_launches(torch, lambda: run.fake_quantize(xs, os_, ms_, 1, 32, 0.0, 2, 2), 200, 20)
     res["tiny_1x32"] = {"us_per_call_events": round(ms * 1e3, 2), "us_per_call_wall": round(wall * 1e3, 2)}
+    # the same call through the operator layer a user of the reference calls (allocations of out and meta included)
+    import mor
+    xg = xs.clone().requires_grad_(True)
+    for key, t in (("mor_ops_us_per_call", xs), ("mor_ops_requires_grad_us_per_call", xg)):
+        ms, wall = time_launches(torch, lambda: mor.ops.fake_quantize(t, 1, 32, 1, 32, 0.0, 2, 2), 500, 50)
+        res["tiny_1x32"][key] = round(wall * 1e3, 2)
     return res
 
 
