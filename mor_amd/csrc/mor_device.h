@@ -19,10 +19,10 @@ __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 
 template <int F> struct Fmt;
-template <> struct Fmt<FMT_E4M3> { static constexpr float fmax = 448.0f;   static constexpr int mbits = 3; static constexpr int emin = -6;  static constexpr bool hw = true;  static constexpr float ovf = 464.0f; };
-template <> struct Fmt<FMT_E5M2> { static constexpr float fmax = 57344.0f; static constexpr int mbits = 2; static constexpr int emin = -14; static constexpr bool hw = true;  static constexpr float ovf = 61440.0f; };
-template <> struct Fmt<FMT_E3M2> { static constexpr float fmax = 28.0f;    static constexpr int mbits = 2; static constexpr int emin = -2;  static constexpr bool hw = false; static constexpr float ovf = 0.0f; };
-template <> struct Fmt<FMT_E2M3> { static constexpr float fmax = 7.5f;     static constexpr int mbits = 3; static constexpr int emin = 0;   static constexpr bool hw = false; static constexpr float ovf = 0.0f; };
+template <> struct Fmt<FMT_E4M3> { static constexpr float fmax = 448.0f;   static constexpr int mbits = 3; static constexpr int emin = -6;  static constexpr bool hw = true; };
+template <> struct Fmt<FMT_E5M2> { static constexpr float fmax = 57344.0f; static constexpr int mbits = 2; static constexpr int emin = -14; static constexpr bool hw = true; };
+template <> struct Fmt<FMT_E3M2> { static constexpr float fmax = 28.0f;    static constexpr int mbits = 2; static constexpr int emin = -2;  static constexpr bool hw = false; };
+template <> struct Fmt<FMT_E2M3> { static constexpr float fmax = 7.5f;     static constexpr int mbits = 3; static constexpr int emin = 0;   static constexpr bool hw = false; };
 
 __host__ __device__ __forceinline__ float fmax_of(int fmt) {
     return fmt == FMT_E4M3 ? 448.0f : fmt == FMT_E5M2 ? 57344.0f : fmt == FMT_E3M2 ? 28.0f : 7.5f;

@@ -9,8 +9,9 @@
 //                    along columns through an LDS copy of the tile, written transposed ([cols, rows] payload) so that
 //                    the reduction dimension of a weight-gradient GEMM is contiguous
 //   k_mx_dequantize  payload + scales -> bf16
-// FP8 codes come from the gfx950 converts; FP6 codes (E2M3 / E3M2) are computed in integer arithmetic and packed
-// little-endian, 32 codes in 24 bytes.
+// All codes come from the gfx950 FP8 converts (E2M3 / E3M2 share the mantissa width of E4M3 / E5M2, see code_pair);
+// FP6 codes are packed little-endian, 32 codes in 24 bytes.  The file also holds k_fq_dual, the fake-quantized
+// tensor and the fake-quantized transpose from one read.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -39,16 +40,7 @@ template <int F> __device__ __forceinline__ int wire_e8(float amax) {
     return min(max(e8, -127), 127);
 }
 
-// 6-bit code (without sign) of a non-negative value on the grid of F
-template <int F> __device__ __forceinline__ uint32_t fp6_code(float r) {
-    constexpr int mb = Fmt<F>::mbits, bias = Wire<F>::bias;
-    const uint32_t b = f2u(r);
-    const int e = (int)(b >> 23) - 127;
-    const uint32_t normal = ((uint32_t)(e + bias) << mb) | ((b >> (23 - mb)) & ((1u << mb) - 1u));
-    const uint32_t sub = (uint32_t)(r * (float)(1 << (mb + bias - 1)));
-    return (e < 1 - bias) ? sub : normal;
-}
-
+// value of a 5-bit magnitude code of F
 template <int F> __device__ __forceinline__ float fp6_value(uint32_t mag) {
     constexpr int mb = Fmt<F>::mbits, bias = Wire<F>::bias;
     const uint32_t e = mag >> mb, m = mag & ((1u << mb) - 1u);
