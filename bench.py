@@ -256,7 +256,7 @@ def other_configs(torch, run, cabi, K, W):
     add("c3_per_row_e4m3_16384x4096", lambda: run.fake_quantize(w, ow, mw, 1, 4096, 0.0, 2, 1), w.numel() * 4 + 16384 * 4, w.numel())
     add("c3_per_row_e5m2_16384x4096", lambda: run.fake_quantize(w, ow, mw, 1, 4096, 0.0, 3, 1), w.numel() * 4 + 16384 * 4, w.numel())
     st3 = run.scaling_state(16384, 4096, 1, 4096, True)
-    add("c3_per_row_e4m3_16384x4096_channel_op_ss3", lambda: run.block_scaling(w, ow, st3, 1, 4096, 0.045, 3), w.numel() * 6, w.numel())
+    add("c3_per_row_e4m3_16384x4096_channel_op_ss3", lambda: run.block_scaling(w, ow, st3, 1, 4096, 0.045, 3), w.numel() * 4, w.numel())   # block-local scale: one pass
     del w, ow
     # C4: MoR 128x128 on the 16384x14336 mixture
     x4 = gen_c4_gpu(torch, 16384, 14336)

@@ -1501,6 +1501,82 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
     }
 }
 
+// The same single pass for row blocks of 1 x 8G elements, G <= 64 lanes (MX 1 x 32 through the channel op is G = 4):
+// the flat chunk array in tiles of 4 * 256 chunks, a block is G consecutive lanes (amax by DPP), as in k_rowgroup.
+// Groups whose scale is outside the fast range are redone from memory by a second, non-unrolled loop.
+template <bool E8>
+__global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* out, uint32_t* ws, int64_t nchunks, int G, int ss_mode) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    constexpr int NV = 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool nt = streams_out(nchunks * 8);
+    float gmax = 0.0f, err = 0.0f;
+    int nnz = 0;
+    const int64_t ntiles = (nchunks + NV * WG - 1) / (NV * WG);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t base = tile * (NV * WG) + tid;
+        uint4 v[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            v[k] = make_uint4(0, 0, 0, 0);
+            if (base + k * WG < nchunks) v[k] = in[base + k * WG];
+        }
+        uint32_t slow = 0;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int64_t c = base + k * WG;
+            float amax = 0.0f;
+            acc_amax_nnz(amax, nnz, v[k]);
+            amax = group_max(amax, G);
+            gmax = fmaxf(gmax, amax);
+            const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
+            float e = 0.0f;
+            uint4 q;
+            q.x = bs_pair_fast<E8>(v[k].x, sc, sc.r, e);
+            q.y = bs_pair_fast<E8>(v[k].y, sc, sc.r, e);
+            q.z = bs_pair_fast<E8>(v[k].z, sc, sc.r, e);
+            q.w = bs_pair_fast<E8>(v[k].w, sc, sc.r, e);
+            if (sc.fast) {
+                err += e;
+                if (c < nchunks) store16_rt(out + c, q, nt);
+            } else if (c < nchunks) slow |= 1u << k;
+        }
+        if (slow) {
+#pragma unroll 1
+            for (int k = 0; k < NV; ++k) {
+                if (!((slow >> k) & 1u)) continue;              // uniform over the lanes of a group
+                const int64_t c = base + k * WG;
+                const uint4 x = in[c];
+                float amax = 0.0f;
+                acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
+                amax = group_max(amax, G);
+                const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
+                uint32_t w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    w[j] = store_pair<false>(bs_element<E8, false>(bf16_lo(w[j]), sc, err), bs_element<E8, false>(bf16_hi(w[j]), sc, err));
+                out[c] = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+    }
+    err = wave_sum(err);
+    nnz = wave_sum_i(nnz);
+    gmax = group_max(gmax, 64);
+    if (lane == 0) { s_f[wave] = err; s_i[wave] = nnz; }
+    __syncthreads();
+    const float e = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+    const int n = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    __syncthreads();
+    if (lane == 0) s_f[wave] = gmax;
+    __syncthreads();
+    if (tid == 0) {
+        reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = e;
+        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
+        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+    }
+}
+
 // pass 4 for the out-of-place ops (FQ:1217-1235): copy the input over the quantized output when meta[0] == 3
 __global__ __launch_bounds__(WG) void k_copy_if(const uint16_t* in, uint16_t* out, const int32_t* meta, int gate, int64_t n, int64_t nvec) {
     if (meta[0] != gate) return;
@@ -1685,6 +1761,19 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
         const int64_t n_all = rows * cols;
         k_copy_if<<<grid_for(n_all / 8, 16), WG, 0, st>>>(in16, out16, meta, 3, n_all, n_all / 8);
         return mor_check_launch("mor_block_scaling (single pass)");
+    }
+
+    if (!inplace && !emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && brows == 1 && bcols % 8 == 0 && is_pow2(bcols / 8)
+        && bcols / 8 <= 64) {
+        const int64_t nchunks = rows * cols / 8;
+        const int grid = (int)std::min<int64_t>(cdiv(nchunks, 4 * WG), MAX_PARTIALS);
+        const uint4* i4 = static_cast<const uint4*>(input);
+        uint4* o4 = static_cast<uint4*>(output);
+        if (ss_mode == 2) k_bs_fused_rows<true><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, (int)(bcols / 8), (int)ss_mode);
+        else k_bs_fused_rows<false><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, (int)(bcols / 8), (int)ss_mode);
+        k_bs_finalize<<<1, WG, 0, st>>>(ws, grid, grid, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        k_copy_if<<<grid_for(nchunks, 16), WG, 0, st>>>(in16, out16, meta, 3, rows * cols, nchunks);
+        return mor_check_launch("mor_block_scaling (single pass, row blocks)");
     }
 
     // pass 1: per-block amax, per-workgroup partials of the tensor amax and the non-zero count
