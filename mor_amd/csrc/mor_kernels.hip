@@ -1461,7 +1461,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
         gmax = fmaxf(gmax, amax);
         nnz_total += nnz;
         const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
-        if (sc.fast) {
+        if (sc.fast || !(amax > 0.0f)) {          // an all-zero block gives +0 whatever its (clamped) scale is
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
                 uint4 q;
@@ -1537,7 +1537,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
             q.y = bs_pair_fast<E8>(v[k].y, sc, sc.r, e);
             q.z = bs_pair_fast<E8>(v[k].z, sc, sc.r, e);
             q.w = bs_pair_fast<E8>(v[k].w, sc, sc.r, e);
-            if (sc.fast) {
+            if (sc.fast || !(amax > 0.0f)) {      // an all-zero block gives +0 whatever its (clamped) scale is
                 err += e;
                 if (c < nchunks) store16_rt(out + c, q, nt);
             } else if (c < nchunks) slow |= 1u << k;
