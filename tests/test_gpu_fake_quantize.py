@@ -208,3 +208,22 @@ def test_extreme_exponents(G):
             want, wmeta = O.fake_quantize(a, br, bc, 1e-15, mode, sf)
             assert np.array_equal(meta, wmeta), (br, bc, mode, sf)
             assert_same(out, want, f"extreme {br}x{bc} mode {mode} sf {sf}")
+
+
+@pytest.mark.parametrize("br,bc", [(1, 32), (128, 128), (1, 512)])
+@pytest.mark.parametrize("mode,sf", [(1, 1), (2, 2), (3, 1)])
+def test_nan_and_inf_elements_stay_inside_their_block(G, br, bc, mode, sf):
+    """NaN / Inf inputs have no pinned reference result; what is asserted: the call completes and every block without
+    such an element is bit-equal to the oracle's."""
+    a = data_gen.c1_normal(256, 512, seed=91)
+    special = [(3, 5, 0x7FC0), (3, 6, 0xFFC0), (140, 300, 0x7F80), (200, 40, 0xFF80), (17, 490, 0x7FFF)]
+    for r, c, bits in special:
+        a[r, c] = bits
+    out, meta = G.fake_quantize(a, br, bc, 1e-15, mode, sf)
+    want, wmeta = O.fake_quantize(a, br, bc, 1e-15, mode, sf)
+    clean = np.ones((256 // br, 512 // bc), bool)
+    for r, c, _ in special:
+        clean[r // br, c // bc] = False
+    mask = np.repeat(np.repeat(clean, br, 0), bc, 1)
+    assert np.array_equal(out[mask], want[mask])
+    assert np.array_equal(meta[clean], wmeta[clean])
