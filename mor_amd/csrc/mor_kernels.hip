@@ -391,8 +391,9 @@ __device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float
         const float va = a * s4.s, vb = b * s4.s;
         const uint32_t p4 = hw_pack2<FMT_E4M3>(va, vb);
         const uint32_t p5 = hw_pack2<FMT_E5M2>(va * 128.0f, vb * 128.0f);
-        const float ya = (a != 0.0f) ? __builtin_amdgcn_rcpf(va) : 0.0f;
-        const float yb = (b != 0.0f) ? __builtin_amdgcn_rcpf(vb) : 0.0f;
+        // a zero element has c = y = 0: its term is 0 * rcp(2^-100) = 0 without a select
+        const float ya = __builtin_amdgcn_rcpf(fmaxf(va, 0x1p-100f));
+        const float yb = __builtin_amdgcn_rcpf(fmaxf(vb, 0x1p-100f));
         e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 0>(p4) - va), ya, e4);
         e5 = fmaf(fabsf(fmaf(hw_unpack<FMT_E5M2, 0>(p5), 0.0078125f, -va)), ya, e5);
         e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 1>(p4) - vb), yb, e4);
