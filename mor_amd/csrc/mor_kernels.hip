@@ -105,27 +105,119 @@ __device__ __forceinline__ void err_terms_exact(float x, bool e8, const Scale& s
 }
 
 // ------------------------------------------------------------------------------------------------
+// quantize one packed word with an fp32 scale: |x| * s, hardware convert, divide by s, round-half-up store, sign
+template <int F> __device__ __forceinline__ uint32_t fq_pair_div(uint32_t w, float s, float r) {
+    const uint32_t p = hw_pack2<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s);
+    const float q0 = div_by_scale(hw_unpack<F, 0>(p), s, r);
+    const float q1 = div_by_scale(hw_unpack<F, 1>(p), s, r);
+    return store_pair<false>(q0, q1) | (w & 0x80008000u);
+}
+template <int F> __device__ __forceinline__ uint4 fq_vec_div(uint4 v, float s, float r) {
+    uint4 o;
+    o.x = fq_pair_div<F>(v.x, s, r);
+    o.y = fq_pair_div<F>(v.y, s, r);
+    o.z = fq_pair_div<F>(v.z, s, r);
+    o.w = fq_pair_div<F>(v.w, s, r);
+    return o;
+}
+
+// The two error terms of one packed word (FQ:504-542) on magnitudes; s5 = 128 * s4 exactly.
+// The reference computes |q / x - 1| with q = c / s.  E8 scale: |q - x| * (1 / x), q - x exact.  FP32 scale:
+// with y = x * s the same quantity is |c - y| / y (c - y is exact: c is within a factor 2 of y, or 0), which needs
+// neither q nor a division; for E5M2 c5 / 128 - y is one exact fma.  Each term differs from the reference's by
+// rounding errors of 1e-7 relative, of either sign, far inside the 1e-6 tolerance on the sums; decisions that would
+// depend on less than 1e-5 are recomputed with the reference's divisions by the caller.  The sums are only wanted
+// for blocks with amax / min non-zero |x| <= 939524096 (FQ:637), so a non-zero element scales to at least
+// 448 / 939524096 and no reciprocal overflows.
+template <bool E8>
+__device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float& e4, float& e5) {
+    float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
+    if constexpr (E8) {
+        const int e84 = s4.e8, e85 = s4.e8 + 7;
+        uint32_t p4 = hw_pack2<FMT_E4M3>(ldexpf(a, e84), ldexpf(b, e84));
+        uint32_t p5 = hw_pack2<FMT_E5M2>(ldexpf(a, e85), ldexpf(b, e85));
+        float qa4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p4)) - (e84 << 23), 0));
+        float qb4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p4)) - (e84 << 23), 0));
+        float qa5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 0>(p5)) - (e85 << 23), 0));
+        float qb5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 1>(p5)) - (e85 << 23), 0));
+        float ya = (a != 0.0f) ? __builtin_amdgcn_rcpf(a) : 0.0f;
+        float yb = (b != 0.0f) ? __builtin_amdgcn_rcpf(b) : 0.0f;
+        e4 = fmaf(fabsf(qa4 - a), ya, e4);
+        e5 = fmaf(fabsf(qa5 - a), ya, e5);
+        e4 = fmaf(fabsf(qb4 - b), yb, e4);
+        e5 = fmaf(fabsf(qb5 - b), yb, e5);
+    } else {
+        const float va = a * s4.s, vb = b * s4.s;
+        const uint32_t p4 = hw_pack2<FMT_E4M3>(va, vb);
+        const uint32_t p5 = hw_pack2<FMT_E5M2>(va * 128.0f, vb * 128.0f);
+        // a zero element has c = y = 0: its term is 0 * rcp(2^-100) = 0 without a select
+        const float ya = __builtin_amdgcn_rcpf(fmaxf(va, 0x1p-100f));
+        const float yb = __builtin_amdgcn_rcpf(fmaxf(vb, 0x1p-100f));
+        e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 0>(p4) - va), ya, e4);
+        e5 = fmaf(fabsf(fmaf(hw_unpack<FMT_E5M2, 0>(p5), 0.0078125f, -va)), ya, e5);
+        e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 1>(p4) - vb), yb, e4);
+        e5 = fmaf(fabsf(fmaf(hw_unpack<FMT_E5M2, 1>(p5), 0.0078125f, -vb)), yb, e5);
+    }
+}
+
+// One element through the fast pair functions (the other half of the word is zero and contributes nothing).
+__device__ __forceinline__ uint16_t fq_one_fast(uint16_t h, int fmt, bool e8, const Scale& sc) {
+    const uint32_t w = h;
+    uint32_t r;
+    if (e8) {
+        switch (fmt) {
+            case FMT_E4M3: r = fq_pair_fast<FMT_E4M3, true>(w, sc); break;
+            case FMT_E5M2: r = fq_pair_fast<FMT_E5M2, true>(w, sc); break;
+            case FMT_E3M2: r = fq_pair_fast<FMT_E3M2, true>(w, sc); break;
+            default:       r = fq_pair_fast<FMT_E2M3, true>(w, sc); break;
+        }
+    } else {
+        switch (fmt) {
+            case FMT_E4M3: r = fq_pair_fast<FMT_E4M3, false>(w, sc); break;
+            case FMT_E5M2: r = fq_pair_fast<FMT_E5M2, false>(w, sc); break;
+            case FMT_E3M2: r = fq_pair_fast<FMT_E3M2, false>(w, sc); break;
+            default:       r = fq_pair_fast<FMT_E2M3, false>(w, sc); break;
+        }
+    }
+    return (uint16_t)r;
+}
+
+// Walks the elements tid, tid + 256, ... of a bh x bw block in row-major order and calls f(offset of the element
+// from the block's first element) without a division per element: (r, c) advance by (256 / bw, 256 % bw) with one
+// carry.
+template <class F>
+__device__ __forceinline__ void for_block_elements(int64_t bh, int64_t bw, int64_t row_pitch, int tid, F&& f) {
+    const int64_t step_r = WG / bw, step_c = WG % bw;
+    int64_t r = tid / bw, c = tid % bw;
+#pragma unroll 1
+    while (r < bh) {
+        f(r * row_pitch + c);
+        r += step_r;
+        c += step_c;
+        if (c >= bw) { c -= bw; ++r; }
+    }
+}
+
 // generic_block: one workgroup quantizes one block of any shape straight from memory with the exact arithmetic.
-// It is the body of k_generic and the fallback of k_wgblock for blocks outside the fast range.
-template <bool EMU>
+// It is the body of k_generic and the fallback of k_wgblock for blocks outside the fast range.  FAST (k_generic, default
+// flavour): blocks whose scale is in the fast range use the few-instruction arithmetic, with the same safeguard on
+// close MoR decisions as k_wgblock.
+template <bool EMU, bool FAST = false>
 __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out, int32_t* meta, float* stats,
                                               const Shape& sh, const QuantArgs& qa, bool e8, int64_t bid,
-                                              float (*s_f)[WAVES], uint32_t* s_u) {
+                                              float (*s_f)[WAVES], uint32_t* s_u, bool allow_fast = false) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
     const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
     const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
-    const int64_t nel = bh * bw;
-
     float amax = 0.0f;
     uint32_t amin_m1 = AMIN_INIT_M1;
-#pragma unroll 1
-    for (int64_t i = tid; i < nel; i += WG) {
-        int64_t r = i / bw, c = i - r * bw;
-        uint32_t a = ((uint32_t)in[(r0 + r) * sh.cols + c0 + c] << 16) & 0x7FFFFFFFu;
+    const uint16_t* bin = in + r0 * sh.cols + c0;
+    for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) {
+        uint32_t a = ((uint32_t)bin[at] << 16) & 0x7FFFFFFFu;
         amax = fmaxf(amax, u2f(a));
         amin_m1 = min(amin_m1, a - 1u);
-    }
+    });
     amax = group_max(amax, 64);
     amin_m1 = group_umin(amin_m1, 64);
     __syncthreads();
@@ -142,18 +234,32 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
         int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
         if (qt == Q_UNKNOWN) {
             const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
-#pragma unroll 1
-            for (int64_t i = tid; i < nel; i += WG) {
-                int64_t r = i / bw, c = i - r * bw;
-                err_terms_exact<EMU>(bf16_one(in[(r0 + r) * sh.cols + c0 + c]), e8, s4, s5, e4, e5);
+            bool exact = true;
+            if constexpr (FAST && !EMU) {
+                if (allow_fast && s4.fast && s4.e8 >= -90 && s4.e8 <= 90) {
+                    if (e8) for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<true>((uint32_t)bin[at], s4, e4, e5); });
+                    else for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<false>((uint32_t)bin[at], s4, e4, e5); });
+                    e4 = wave_sum(e4);
+                    e5 = wave_sum(e5);
+                    __syncthreads();
+                    if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+                    __syncthreads();
+                    e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
+                    e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+                    exact = !(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5));       // too close: repeat with the reference's divisions
+                    if (exact) { e4 = 0.0f; e5 = 0.0f; }
+                }
             }
-            e4 = wave_sum(e4);
-            e5 = wave_sum(e5);
-            __syncthreads();
-            if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
-            __syncthreads();
-            e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
-            e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+            if (exact) {
+                for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_terms_exact<EMU>(bf16_one(bin[at]), e8, s4, s5, e4, e5); });
+                e4 = wave_sum(e4);
+                e5 = wave_sum(e5);
+                __syncthreads();
+                if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+                __syncthreads();
+                e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
+                e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+            }
             qt = mor_decide_error(amax, qa.clamp, e4, e5);
         }
         meta_val = qt;
@@ -167,13 +273,17 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
     const bool copy = (fmt < 0) || !(amax > 0.0f);
     if (copy && out == in) return;
     const Scale sc = make_scale(copy ? 1.0f : fmax_of(fmt) / amax);
-#pragma unroll 1
-    for (int64_t i = tid; i < nel; i += WG) {
-        int64_t r = i / bw, c = i - r * bw;
-        int64_t at = (r0 + r) * sh.cols + c0 + c;
-        uint16_t h = in[at];
-        if (!copy) h = fq_one_exact<EMU>(h, fmt, e8, sc);
-        out[at] = h;
+    uint16_t* bout = out + r0 * sh.cols + c0;
+    bool fast = false;
+    if constexpr (FAST && !EMU) fast = allow_fast && !copy && sc.fast && sc.e8 >= -90 && sc.e8 <= 90;
+    if (fast) {
+        for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { bout[at] = fq_one_fast(bin[at], fmt, e8, sc); });
+    } else {
+        for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) {
+            uint16_t h = bin[at];
+            if (!copy) h = fq_one_exact<EMU>(h, fmt, e8, sc);
+            bout[at] = h;
+        });
     }
 }
 
@@ -182,7 +292,7 @@ __global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* ou
                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int e8) {
     __shared__ float s_f[2][WAVES];
     __shared__ uint32_t s_u[WAVES];
-    generic_block<EMU>(in, out, meta, stats, sh, qa, e8 != 0, blockIdx.x, s_f, s_u);
+    generic_block<EMU, true>(in, out, meta, stats, sh, qa, (e8 & 1) != 0, blockIdx.x, s_f, s_u, (e8 & 2) != 0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -346,61 +456,6 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
 }
 
 // ------------------------------------------------------------------------------------------------
-// quantize one packed word with an fp32 scale: |x| * s, hardware convert, divide by s, round-half-up store, sign
-template <int F> __device__ __forceinline__ uint32_t fq_pair_div(uint32_t w, float s, float r) {
-    const uint32_t p = hw_pack2<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s);
-    const float q0 = div_by_scale(hw_unpack<F, 0>(p), s, r);
-    const float q1 = div_by_scale(hw_unpack<F, 1>(p), s, r);
-    return store_pair<false>(q0, q1) | (w & 0x80008000u);
-}
-template <int F> __device__ __forceinline__ uint4 fq_vec_div(uint4 v, float s, float r) {
-    uint4 o;
-    o.x = fq_pair_div<F>(v.x, s, r);
-    o.y = fq_pair_div<F>(v.y, s, r);
-    o.z = fq_pair_div<F>(v.z, s, r);
-    o.w = fq_pair_div<F>(v.w, s, r);
-    return o;
-}
-
-// The two error terms of one packed word (FQ:504-542) on magnitudes; s5 = 128 * s4 exactly.
-// The reference computes |q / x - 1| with q = c / s.  E8 scale: |q - x| * (1 / x), q - x exact.  FP32 scale:
-// with y = x * s the same quantity is |c - y| / y (c - y is exact: c is within a factor 2 of y, or 0), which needs
-// neither q nor a division; for E5M2 c5 / 128 - y is one exact fma.  Each term differs from the reference's by
-// rounding errors of 1e-7 relative, of either sign, far inside the 1e-6 tolerance on the sums; decisions that would
-// depend on less than 1e-5 are recomputed with the reference's divisions by the caller.  The sums are only wanted
-// for blocks with amax / min non-zero |x| <= 939524096 (FQ:637), so a non-zero element scales to at least
-// 448 / 939524096 and no reciprocal overflows.
-template <bool E8>
-__device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float& e4, float& e5) {
-    float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
-    if constexpr (E8) {
-        const int e84 = s4.e8, e85 = s4.e8 + 7;
-        uint32_t p4 = hw_pack2<FMT_E4M3>(ldexpf(a, e84), ldexpf(b, e84));
-        uint32_t p5 = hw_pack2<FMT_E5M2>(ldexpf(a, e85), ldexpf(b, e85));
-        float qa4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p4)) - (e84 << 23), 0));
-        float qb4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p4)) - (e84 << 23), 0));
-        float qa5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 0>(p5)) - (e85 << 23), 0));
-        float qb5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 1>(p5)) - (e85 << 23), 0));
-        float ya = (a != 0.0f) ? __builtin_amdgcn_rcpf(a) : 0.0f;
-        float yb = (b != 0.0f) ? __builtin_amdgcn_rcpf(b) : 0.0f;
-        e4 = fmaf(fabsf(qa4 - a), ya, e4);
-        e5 = fmaf(fabsf(qa5 - a), ya, e5);
-        e4 = fmaf(fabsf(qb4 - b), yb, e4);
-        e5 = fmaf(fabsf(qb5 - b), yb, e5);
-    } else {
-        const float va = a * s4.s, vb = b * s4.s;
-        const uint32_t p4 = hw_pack2<FMT_E4M3>(va, vb);
-        const uint32_t p5 = hw_pack2<FMT_E5M2>(va * 128.0f, vb * 128.0f);
-        // a zero element has c = y = 0: its term is 0 * rcp(2^-100) = 0 without a select
-        const float ya = __builtin_amdgcn_rcpf(fmaxf(va, 0x1p-100f));
-        const float yb = __builtin_amdgcn_rcpf(fmaxf(vb, 0x1p-100f));
-        e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 0>(p4) - va), ya, e4);
-        e5 = fmaf(fabsf(fmaf(hw_unpack<FMT_E5M2, 0>(p5), 0.0078125f, -va)), ya, e5);
-        e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 1>(p4) - vb), yb, e4);
-        e5 = fmaf(fabsf(fmaf(hw_unpack<FMT_E5M2, 1>(p5), 0.0078125f, -vb)), yb, e5);
-    }
-}
-
 // ------------------------------------------------------------------------------------------------
 // k_wgblock: one workgroup per quantization block, the block held in registers (NV 16-byte vectors per lane).
 // Chunk ch = k * 256 + tid of the block sits at block row ch / cpr, chunk column ch % cpr.
@@ -822,8 +877,10 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
         }
         return mor_check_launch("k_wgblock");
     }
-    if (emu) k_generic<true><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, e8 ? 1 : 0);
-    else k_generic<false><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, e8 ? 1 : 0);
+    // bit 0: power-of-two scale; bit 1: the few-instruction arithmetic (hardware converts) is allowed
+    const int gflags = (e8 ? 1 : 0) | (fast_ok ? 2 : 0);
+    if (emu) k_generic<true><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags);
+    else k_generic<false><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags);
     return mor_check_launch("k_generic");
 }
 
