@@ -1715,18 +1715,20 @@ __global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, 
     const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
     const uint4* in4 = reinterpret_cast<const uint4*>(in);
     uint4* out4 = reinterpret_cast<uint4*>(out);
-    constexpr int NV = 4;
-    for (int64_t c0 = gtid; c0 < nvec; c0 += stride * NV) {
+    constexpr int NV = 4;                       // a workgroup takes tiles of NV * 256 consecutive 16-byte chunks
+    const int64_t ntiles = (nvec + NV * WG - 1) / (NV * WG);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t c0 = tile * (NV * WG) + threadIdx.x;
         uint4 v[NV];
 #pragma unroll
-        for (int k = 0; k < NV; ++k) { v[k] = make_uint4(0, 0, 0, 0); if (c0 + k * stride < nvec) v[k] = in4[c0 + k * stride]; }
+        for (int k = 0; k < NV; ++k) { v[k] = make_uint4(0, 0, 0, 0); if (c0 + k * WG < nvec) v[k] = in4[c0 + k * WG]; }
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 w[j] = store_pair<EMU>(e8mx_element<MB, UNIT>(bf16_lo(w[j]), sf, rs, mk), e8mx_element<MB, UNIT>(bf16_hi(w[j]), sf, rs, mk));
-            if (c0 + k * stride < nvec) store16_rt(out4 + c0 + k * stride, make_uint4(w[0], w[1], w[2], w[3]), streams_out(n));
+            if (c0 + k * WG < nvec) store16_rt(out4 + c0 + k * WG, make_uint4(w[0], w[1], w[2], w[3]), streams_out(n));
         }
     }
     for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = store_bf16<EMU>(e8mx_element<MB, UNIT>(bf16_one(in[i]), sf, rs, mk));
@@ -1904,7 +1906,7 @@ extern "C" int mor_e8mx(const void* input, void* output, int64_t rows, int64_t c
     uint16_t* out16 = static_cast<uint16_t*>(output);
     const int64_t n = rows * cols;
     const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
-    const int grid = grid_for(nvec > 0 ? nvec : n, 16);
+    const int grid = nvec > 0 ? (int)std::min<int64_t>(cdiv(nvec, 4 * WG), 1 << 20) : grid_for(n, 16);
     const int strategy = (int)scaling_strategy;
     int npart = 0;
     if (strategy == 1) {
