@@ -1,0 +1,133 @@
+"""Seeded random sweep over shapes, block shapes, modes and data kinds: every case goes through the C ABI and must
+equal the CPU oracle bit for bit (error sums to 1e-6).  The case list is fixed by the seed, so a failure names its case."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mor_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    assert torch.cuda.is_available()
+    return gpu_util
+
+
+def make_data(rng, rows, cols, kind):
+    if kind == 0:      # normal
+        x = rng.standard_normal((rows, cols)).astype(np.float32)
+    elif kind == 1:    # heavy tails with outliers
+        x = (rng.standard_t(3, (rows, cols)) * 0.02).astype(np.float32)
+        x[rng.random((rows, cols)) < 1e-2] *= 1000
+    elif kind == 2:    # log-normal magnitudes, random sign, sparse zeros
+        x = (np.exp(3 * rng.standard_normal((rows, cols))) * rng.choice([-1.0, 1.0], (rows, cols))).astype(np.float32)
+        x[rng.random((rows, cols)) < 0.05] = 0
+    else:              # tiny values with a zero stripe
+        x = (rng.standard_normal((rows, cols)) * 1e-4).astype(np.float32)
+        x[rows // 3] = 0
+    t = torch.from_numpy(x).to(torch.bfloat16)
+    return t.view(torch.int16).numpy().view(np.uint16).copy()
+
+
+def fq_cases():
+    rng = np.random.default_rng(20251)
+    blocks = [(1, 8), (1, 16), (1, 32), (1, 64), (1, 128), (1, 256), (1, 512), (1, 1024), (1, 2048), (2, 64), (4, 32),
+              (8, 8), (16, 16), (16, 56), (32, 32), (64, 64), (128, 128), (128, 64), (64, 256), (3, 40), (5, 7), (1, 24)]
+    cases = []
+    for i in range(90):
+        br, bc = blocks[rng.integers(len(blocks))]
+        exact = rng.random() < 0.6
+        ny, nx = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+        rows = br * ny if exact else br * ny - int(rng.integers(0, br))
+        cols = bc * nx if exact else bc * nx - int(rng.integers(0, min(bc, 9)))
+        rows, cols = max(rows, 1), max(cols, 1)
+        mode = int(rng.choice([1, 101, 2, 3, 4, 5, 7]))
+        sf = int(rng.choice([1, 2]))
+        cases.append((i, rows, cols, br, bc, mode, sf, int(rng.integers(4))))
+    return cases
+
+
+@pytest.mark.parametrize("case", fq_cases(), ids=lambda c: "fq%d_%dx%d_b%dx%d_m%d_s%d_k%d" % c)
+def test_fake_quantize_sweep(G, case):
+    i, rows, cols, br, bc, mode, sf, kind = case
+    rng = np.random.default_rng(1000 + i)
+    a = make_data(rng, rows, cols, kind)
+    clamp = 1e-15 if mode not in (4, 5) else float(np.float32((448.0 if mode == 4 else 57344.0) / max(np.abs((a.astype(np.uint32) << 16).view(np.float32)).max(), 1e-30)))
+    print("sweep", case, flush=True)
+    out, meta = G.fake_quantize(a, br, bc, clamp, mode, sf)
+    want, wmeta, stats = O.fake_quantize(a, br, bc, clamp, mode, sf, want_stats=True)
+    ok_blocks = np.ones(meta.shape, bool)
+    if mode in (1, 101):
+        flip = meta != wmeta                       # a decision may differ only where the two error sums tie to 1e-6
+        if flip.any():
+            e4, e5 = stats[..., 2][flip], stats[..., 3][flip]
+            assert np.all(np.abs(e4 - e5) <= 1e-6 * np.maximum(e4, e5)), (case, e4, e5)
+            ok_blocks = ~flip
+    assert np.array_equal(meta[ok_blocks], wmeta[ok_blocks]), case
+    mask = np.repeat(np.repeat(ok_blocks, br, 0), bc, 1)[:rows, :cols]
+    bad = np.argwhere((out != want) & mask)
+    assert len(bad) == 0, (case, len(bad), tuple(bad[0]), hex(int(out[tuple(bad[0])])), hex(int(want[tuple(bad[0])])))
+
+
+def scaling_cases():
+    rng = np.random.default_rng(20252)
+    blocks = [(1, 32), (1, 64), (1, 256), (1, 1024), (1, 2048), (128, 128), (64, 64), (32, 16), (16, 120), (20, 12),
+              (64, 1), (256, 1), (8, 1)]
+    cases = []
+    for i in range(60):
+        br, bc = blocks[rng.integers(len(blocks))]
+        ny, nx = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        if bc == 1:
+            nx = int(rng.choice([40, 64, 200, 520]))
+        cases.append((i, br * ny, bc * nx, br, bc, int(rng.choice([1, 2, 3, 4])), int(rng.integers(3)), bool(rng.integers(2)),
+                      float(rng.choice([0.02, 0.045, 0.2]))))
+    return cases
+
+
+@pytest.mark.parametrize("case", scaling_cases(), ids=lambda c: "bs%d_%dx%d_b%dx%d_ss%d_k%d_%s_%g" % c)
+def test_scaling_sweep(G, case):
+    i, rows, cols, br, bc, ss, kind, inplace, thr = case
+    rng = np.random.default_rng(2000 + i)
+    a = make_data(rng, rows, cols, kind)
+    channel = (br == 1 or bc == 1)
+    print("sweep", case, flush=True)
+    out, meta, gamax, gnnz, gerr = G.block_scaling(a, br, bc, thr, ss, channel=channel, inplace=inplace)
+    want, wmeta, wamax, wnnz, werr = O.block_scaling(a, br, bc, thr, ss, channel=channel)
+    assert gamax[0] == wamax[0] and gnnz[0] == wnnz[0], case
+    np.testing.assert_allclose(gerr[0], werr[0], rtol=2e-6, atol=0)
+    avg = werr[0] / max(wnnz[0], 1)
+    if abs(avg - thr) > 1e-5 * thr:
+        assert meta[0] == wmeta[0], case
+    if meta[0] == wmeta[0]:
+        bad = np.argwhere(out != want)
+        assert len(bad) == 0, (case, len(bad), tuple(bad[0]), hex(int(out[tuple(bad[0])])), hex(int(want[tuple(bad[0])])))
+
+
+def wire_cases():
+    rng = np.random.default_rng(20253)
+    return [(i, 32 * int(rng.integers(1, 9)), 32 * int(rng.integers(1, 12)), int(rng.integers(4)), int(rng.integers(4))) for i in range(32)]
+
+
+@pytest.mark.parametrize("case", wire_cases(), ids=lambda c: "mx%d_%dx%d_f%d_k%d" % c)
+def test_wire_sweep(G, case):
+    i, rows, cols, fmt, kind = case
+    rng = np.random.default_rng(3000 + i)
+    a = make_data(rng, rows, cols, kind)
+    print("sweep", case, flush=True)
+    wp, ws = O.mx_quantize(a, fmt)
+    tp, ts = O.mx_quantize(np.ascontiguousarray(a.T), fmt)
+    rp, rs, cp, cs = G.mx_quantize_dual(a, fmt)
+    gp, gs = G.mx_quantize(a, fmt)
+    assert np.array_equal(gp, wp) and np.array_equal(gs, ws), case
+    assert np.array_equal(rp, wp) and np.array_equal(rs, ws) and np.array_equal(cp, tp) and np.array_equal(cs, ts), case
+    assert np.array_equal(G.mx_dequantize(wp, ws, fmt), O.mx_dequantize(wp, ws, fmt)), case
+    if fmt in (O.E4M3, O.E5M2):
+        for sf in (1, 2):
+            mode = 2 if fmt == O.E4M3 else 3
+            o, m, ot, mt = G.fake_quantize_dual(a, mode, sf)
+            w, _ = O.fake_quantize(a, 1, 32, 0.0, mode, sf)
+            wt, _ = O.fake_quantize(np.ascontiguousarray(a.T), 1, 32, 0.0, mode, sf)
+            assert np.array_equal(o, w) and np.array_equal(ot, wt), (case, sf)
