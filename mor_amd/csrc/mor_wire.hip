@@ -63,7 +63,8 @@ template <int F> __device__ __forceinline__ uint32_t code_pair(uint32_t w, int e
         constexpr float norm_min = (F == FMT_E2M3) ? 1.0f : 0.25f;
         constexpr uint32_t off_normal = (uint32_t)(Wire<F8>::bias - Wire<F>::bias) << mb;
         constexpr uint32_t off_sub = (uint32_t)(1 - Wire<F>::bias + Wire<F8>::bias) << mb;
-        const float a = ldexpf(fabsf(bf16_lo(w)), e8), b = ldexpf(fabsf(bf16_hi(w)), e8);
+        // (in a block scaled by its own e8 nothing exceeds fmax; the clamp is the cast's saturation for any other use)
+        const float a = fminf(ldexpf(fabsf(bf16_lo(w)), e8), Fmt<F>::fmax), b = fminf(ldexpf(fabsf(bf16_hi(w)), e8), Fmt<F>::fmax);
         const bool na = a >= norm_min, nb = b >= norm_min;
         const uint32_t p = hw_pack2<F8>(na ? a : a + norm_min, nb ? b : b + norm_min);
         const uint32_t ca = (p & 0xFFu) - (na ? off_normal : off_sub);
@@ -79,25 +80,79 @@ template <int F> __device__ __forceinline__ uint64_t code_chunk(uint4 v, int e8)
            ((uint64_t)code_pair<F>(v.z, e8) << (2 * pb)) | ((uint64_t)code_pair<F>(v.w, e8) << (3 * pb));
 }
 
+// FP6 by the gfx950 block convert: v_cvt_scalef32_pk32_{fp6,bf6}_bf16 turns 32 bf16 values into 32 packed 6-bit codes
+// of RNE(x / 2^floor(log2(scale))), saturating, sign kept (E2M3 = "fp6", E3M2 = "bf6"); mor_selftest_hw_fp6 compares it
+// with the software codes over every bf16 value and every scale exponent.  Used when 2^-e8 is a normal float.
+typedef __bf16 bf16x32 __attribute__((ext_vector_type(32)));
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x6 __attribute__((ext_vector_type(6)));
+__device__ __forceinline__ bool fp6_hw_ok(int e8) { return e8 >= -126 && e8 <= 126; }
+template <int F> __device__ __forceinline__ u32x6 fp6_block_hw(const uint32_t (&words)[16], int e8) {
+    const float scale = u2f((uint32_t)(127 - e8) << 23);
+    u32x16 t;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) t[i] = words[i];
+    const bf16x32 x = __builtin_bit_cast(bf16x32, t);
+    if constexpr (F == FMT_E2M3) return __builtin_bit_cast(u32x6, __builtin_amdgcn_cvt_scalef32_pk32_fp6_bf16(x, scale));
+    else return __builtin_bit_cast(u32x6, __builtin_amdgcn_cvt_scalef32_pk32_bf6_bf16(x, scale));
+}
+// the same 6 words from the software codes of 16 packed pairs
+template <int F> __device__ __forceinline__ u32x6 fp6_block_sw(const uint32_t (&words)[16], int e8) {
+    uint32_t p[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) p[i] = code_pair<F>(words[i], e8);
+    u32x6 d;
+#pragma unroll
+    for (int g = 0; g < 6; ++g) {
+        uint32_t acc = 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int lo_bit = 12 * i - 32 * g;                      // position of pair i in this word
+            if (lo_bit > -12 && lo_bit < 32) acc |= lo_bit >= 0 ? (p[i] << lo_bit) : (p[i] >> (-lo_bit));
+        }
+        d[g] = acc;
+    }
+    return d;
+}
+
 __device__ __forceinline__ float chunk_amax(uint4 v) {
     float amax = 0.0f;
     acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
     return amax;
 }
 
-// Stores the codes of one chunk.  `c` is the chunk's index in the payload's own row-major order (4 chunks = 1 block).
-// FP8: 8 bytes per lane.  FP6: the 4 lanes of a block hold 4 x 48 bits = 24 bytes; lanes 0..2 store 8 bytes each,
-// built from their own bits and the next lane's.
-template <int F> __device__ __forceinline__ void store_codes(uint8_t* payload, int64_t c, uint64_t codes, bool ok) {
+// Quantizes and stores one chunk; `c` is the chunk's index in the payload's own row-major order (4 chunks = 1 block,
+// held by the 4 lanes of a quad; every lane of the quad must call this).
+// FP8: 8 bytes per lane.  FP6: the quad's 16 words are broadcast to its lanes (DPP), every lane converts the whole
+// block with one instruction and lanes 0..2 store 8 of the 24 bytes each; outside the range of the block convert the
+// software codes are merged across the quad instead.
+template <int J> __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) { return dpp_u<J * 0x55>(v); }
+template <int F> __device__ __forceinline__ void emit_chunk(uint8_t* payload, int64_t c, uint4 v, int e8, bool ok) {
     if constexpr (Fmt<F>::hw) {
+        const uint64_t codes = code_chunk<F>(v, e8);
         if (ok) *reinterpret_cast<uint2*>(payload + c * 8) = make_uint2((uint32_t)codes, (uint32_t)(codes >> 32));
     } else {
-        constexpr int NEXT = 0xF9;                               // quad_perm [1,2,3,3]: lane i reads lane i + 1
-        const uint32_t nlo = dpp_u<NEXT>((uint32_t)codes), nhi = dpp_u<NEXT>((uint32_t)(codes >> 32));
-        const uint64_t next = (uint64_t)nlo | ((uint64_t)nhi << 32);
         const int j = (int)(c & 3);
-        const uint64_t word = (codes >> (16 * j)) | (next << (48 - 16 * j));
-        if (ok && j < 3) *reinterpret_cast<uint2*>(payload + (c >> 2) * 24 + j * 8) = make_uint2((uint32_t)word, (uint32_t)(word >> 32));
+        uint32_t lo, hi;
+        if (fp6_hw_ok(e8)) {                                     // uniform over the quad (e8 is the block's)
+            uint32_t w[16];
+            w[0] = quad_bcast<0>(v.x); w[1] = quad_bcast<0>(v.y); w[2] = quad_bcast<0>(v.z); w[3] = quad_bcast<0>(v.w);
+            w[4] = quad_bcast<1>(v.x); w[5] = quad_bcast<1>(v.y); w[6] = quad_bcast<1>(v.z); w[7] = quad_bcast<1>(v.w);
+            w[8] = quad_bcast<2>(v.x); w[9] = quad_bcast<2>(v.y); w[10] = quad_bcast<2>(v.z); w[11] = quad_bcast<2>(v.w);
+            w[12] = quad_bcast<3>(v.x); w[13] = quad_bcast<3>(v.y); w[14] = quad_bcast<3>(v.z); w[15] = quad_bcast<3>(v.w);
+            const u32x6 d = fp6_block_hw<F>(w, e8);
+            lo = j == 0 ? d[0] : j == 1 ? d[2] : d[4];
+            hi = j == 0 ? d[1] : j == 1 ? d[3] : d[5];
+        } else {
+            const uint64_t codes = code_chunk<F>(v, e8);
+            constexpr int NEXT = 0xF9;                           // quad_perm [1,2,3,3]: lane i reads lane i + 1
+            const uint32_t nlo = dpp_u<NEXT>((uint32_t)codes), nhi = dpp_u<NEXT>((uint32_t)(codes >> 32));
+            const uint64_t next = (uint64_t)nlo | ((uint64_t)nhi << 32);
+            const uint64_t word = (codes >> (16 * j)) | (next << (48 - 16 * j));
+            lo = (uint32_t)word;
+            hi = (uint32_t)(word >> 32);
+        }
+        if (ok && j < 3) *reinterpret_cast<uint2*>(payload + (c >> 2) * 24 + j * 8) = make_uint2(lo, hi);
     }
 }
 
@@ -118,7 +173,7 @@ __global__ __launch_bounds__(WWG) void k_mx_quantize(const uint4* in, uint8_t* p
         const int64_t c = base + k * WWG;
         const float amax = group_max_t<4>(chunk_amax(v[k]), 4);
         const int e8 = wire_e8<F>(amax);
-        store_codes<F>(payload, c, code_chunk<F>(v[k], e8), c < nchunks);
+        emit_chunk<F>(payload, c, v[k], e8, c < nchunks);
         // the scale bytes of 4 consecutive blocks (16 lanes) leave as one 32-bit store
         const uint32_t sb = (uint32_t)(127 - e8);
         const uint32_t s4 = sb | (__shfl_down(sb, 4, 16) << 8) | (__shfl_down(sb, 8, 16) << 16) | (__shfl_down(sb, 12, 16) << 24);
@@ -144,7 +199,7 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
     constexpr int BPT = TILE_C * RB / WWG;        // column blocks per thread
     constexpr int blk_bytes = 32 * Wire<F>::bits / 8;
     constexpr int SEG = Fmt<F>::hw ? 16 : 8;      // bytes per lane of the column stores (both divide blk_bytes)
-    constexpr int CODE_PITCH = RB * blk_bytes + SEG;  // bytes per column of the code tile (the pad spreads the banks)
+    constexpr int CODE_PITCH = (RB * blk_bytes + 16 + 15) / 16 * 16;   // bytes per column of the code tile (padded, 16-byte aligned)
     constexpr int SEGS = RB * blk_bytes / SEG;    // per column
     // one buffer, two uses: the bf16 tile, then the codes of the column blocks (smaller)
     __shared__ __attribute__((aligned(16))) uint16_t tile[TR * PITCH];
@@ -194,7 +249,7 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
         const float amax = group_max_t<4>(chunk_amax(v[k]), 4);
         const int e8 = wire_e8<F>(amax);
         const int64_t cidx = (R0 + r) * row_chunks + (C0 >> 3) + cc;       // chunk index in the row-major payload
-        store_codes<F>(row_payload, cidx, code_chunk<F>(v[k], e8), ok[k]);
+        emit_chunk<F>(row_payload, cidx, v[k], e8, ok[k]);
         const uint32_t sb = (uint32_t)(127 - e8);
         const uint32_t s4 = sb | (__shfl_down(sb, 4, 16) << 8) | (__shfl_down(sb, 8, 16) << 16) | (__shfl_down(sb, 12, 16) << 24);
         if (dword_row_scales && cols_valid == TILE_C) {
@@ -220,19 +275,7 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
             *reinterpret_cast<uint4*>(dst) = make_uint4(q[0], q[1], q[2], q[3]);
             *reinterpret_cast<uint4*>(dst + 16) = make_uint4(q[4], q[5], q[6], q[7]);
         } else {
-            uint32_t p[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) p[i] = code_pair<F>(w[h][i], e8);
-            uint32_t d[6];                                                   // 6 x 32 bits = 32 codes
-#pragma unroll
-            for (int g = 0; g < 6; ++g) {
-                d[g] = 0;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int lo_bit = 12 * i - 32 * g;                      // position of pair i in this word
-                    if (lo_bit > -12 && lo_bit < 32) d[g] |= lo_bit >= 0 ? (p[i] << lo_bit) : (p[i] >> (-lo_bit));
-                }
-            }
+            const u32x6 d = fp6_hw_ok(e8) ? fp6_block_hw<F>(w[h], e8) : fp6_block_sw<F>(w[h], e8);
             *reinterpret_cast<uint2*>(dst) = make_uint2(d[0], d[1]);
             *reinterpret_cast<uint2*>(dst + 8) = make_uint2(d[2], d[3]);
             *reinterpret_cast<uint2*>(dst + 16) = make_uint2(d[4], d[5]);
@@ -244,14 +287,22 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
     // the transposed payload: a column of the tile is RB * blk_bytes contiguous bytes, SEGS lanes store one column
     const int64_t col_row_bytes = rows / 32 * blk_bytes;                 // bytes per column in the transposed payload
     const int valid_bytes = rows_valid / 32 * blk_bytes;
+    if (SEG == 16 || ((col_row_bytes & 15) == 0 && rows_valid == TR)) {      // 16 bytes per lane wherever they are aligned
+        constexpr int S16 = RB * blk_bytes / 16;
 #pragma unroll
-    for (int i = 0; i < TILE_C * SEGS / WWG; ++i) {
-        const int idx = i * WWG + tid, col = idx / SEGS, seg = idx % SEGS;
-        if (col < cols_valid && seg * SEG < valid_bytes) {
-            uint8_t* dst = col_payload + (C0 + col) * col_row_bytes + (R0 / 32) * blk_bytes + seg * SEG;
-            const uint8_t* src = codes + col * CODE_PITCH + seg * SEG;
-            if constexpr (SEG == 16) store16_rt(reinterpret_cast<uint4*>(dst), *reinterpret_cast<const uint4*>(src), nt);
-            else *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(src);
+        for (int i = 0; i < (TILE_C * S16 + WWG - 1) / WWG; ++i) {
+            const int idx = i * WWG + tid, col = idx / S16, seg = idx % S16;
+            if (col < cols_valid && seg * 16 < valid_bytes && idx < TILE_C * S16)
+                store16_rt(reinterpret_cast<uint4*>(col_payload + (C0 + col) * col_row_bytes + (R0 / 32) * blk_bytes + seg * 16),
+                           *reinterpret_cast<const uint4*>(codes + col * CODE_PITCH + seg * 16), nt);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < TILE_C * SEGS / WWG; ++i) {
+            const int idx = i * WWG + tid, col = idx / SEGS, seg = idx % SEGS;
+            if (col < cols_valid && seg * SEG < valid_bytes)
+                *reinterpret_cast<uint2*>(col_payload + (C0 + col) * col_row_bytes + (R0 / 32) * blk_bytes + seg * SEG) =
+                    *reinterpret_cast<const uint2*>(codes + col * CODE_PITCH + seg * SEG);
         }
     }
     // scale bytes of the column blocks: RB per column and tile
@@ -421,6 +472,34 @@ __global__ __launch_bounds__(WWG) void k_mx_dequantize(const uint8_t* payload, c
     }
 }
 
+// Every bf16 value x every scale exponent the block convert is used with: hardware codes against software codes.
+// One thread per (32 consecutive bf16 patterns, e8); counts the differing codes.
+template <int F>
+__global__ __launch_bounds__(WWG) void k_selftest_hw_fp6(unsigned long long* mismatches) {
+    const uint32_t idx = blockIdx.x * WWG + threadIdx.x;
+    if (idx >= 2048u * 253u) return;
+    const uint32_t group = idx & 2047u;
+    const int e8 = (int)(idx >> 11) - 126;
+    uint32_t words[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        uint32_t lo = group * 32u + 2u * i, hi = lo + 1u;
+        if ((lo & 0x7F80u) == 0x7F80u) lo = 0;                   // Inf / NaN patterns are outside the contract
+        if ((hi & 0x7F80u) == 0x7F80u) hi = 0;
+        words[i] = lo | (hi << 16);
+    }
+    const u32x6 a = fp6_block_hw<F>(words, e8), b = fp6_block_sw<F>(words, e8);
+    unsigned bad = 0;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+        const int bit = 6 * j, g = bit >> 5, sh = bit & 31;
+        uint32_t x = (a[g] ^ b[g]) >> sh;
+        if (sh > 26 && g < 5) x |= (a[g + 1] ^ b[g + 1]) << (32 - sh);
+        bad += (x & 0x3Fu) != 0;
+    }
+    if (bad) atomicAdd(mismatches + (F == FMT_E2M3 ? 0 : 1), (unsigned long long)bad);
+}
+
 }  // namespace mor
 
 using namespace mor;
@@ -523,4 +602,15 @@ extern "C" int mor_fake_quantize_dual(const void* input, void* output_rows, int3
         else k_fq_dual<FMT_E5M2, false><<<grid, WWG, 0, st>>>(in, orow, meta_rows, ocol, meta_cols, rows, cols, 2);
     }
     return mor_check_launch("k_fq_dual");
+}
+
+extern "C" int mor_selftest_hw_fp6(uint64_t* mismatches, void* stream) {
+    if (!mismatches) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mismatches is NULL");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = hipMemsetAsync(mismatches, 0, 2 * sizeof(uint64_t), st);
+    if (e != hipSuccess) return mor_fail(MOR_ERR_LAUNCH, "hipMemsetAsync: %s", hipGetErrorString(e));
+    const unsigned grid = (2048u * 253u + WWG - 1) / WWG;
+    k_selftest_hw_fp6<FMT_E2M3><<<grid, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
+    k_selftest_hw_fp6<FMT_E3M2><<<grid, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
+    return mor_check_launch("k_selftest_hw_fp6");
 }

@@ -145,3 +145,13 @@ def test_python_api_round_trip():
         wire.quantize_mx(x[:, :48], wire.E4M3)
     p6, s6 = wire.quantize_mx(x, wire.E2M3)
     assert p6.shape == (256, 384) and wire.dequantize_mx(p6, s6, wire.E2M3).shape == (256, 512)
+
+
+def test_hw_fp6_block_convert_selftest(G):
+    """v_cvt_scalef32_pk32_{fp6,bf6}_bf16 against the software codes: 65 280 finite bf16 values x 253 scale exponents."""
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    bad = torch.full((2,), -1, dtype=torch.int64, device="cuda")
+    _cabi.check(L.mor_selftest_hw_fp6(bad.data_ptr(), None))
+    torch.cuda.synchronize()
+    assert bad.tolist() == [0, 0]
