@@ -133,7 +133,8 @@ MOR_API int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
 
 /*
  * The same for the gfx950 block convert of 32 bf16 values to packed FP6 (used by the MX wire format):
- * every finite bf16 value with every scale exponent against the software codes.
+ * every finite bf16 value with every scale exponent against the software codes, and the inverse
+ * convert (codes to bf16) for every code and scale exponent it is used with.
  * mismatches[0] = E2M3 count, mismatches[1] = E3M2 count (device pointer, 2 x uint64).
  */
 MOR_API int mor_selftest_hw_fp6(uint64_t* mismatches, void* stream);

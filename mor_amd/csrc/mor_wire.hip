@@ -96,6 +96,14 @@ template <int F> __device__ __forceinline__ u32x6 fp6_block_hw(const uint32_t (&
     if constexpr (F == FMT_E2M3) return __builtin_bit_cast(u32x6, __builtin_amdgcn_cvt_scalef32_pk32_fp6_bf16(x, scale));
     else return __builtin_bit_cast(u32x6, __builtin_amdgcn_cvt_scalef32_pk32_bf6_bf16(x, scale));
 }
+// The inverse block convert, v_cvt_scalef32_pk32_bf16_{fp6,bf6}: 32 packed codes -> 32 bf16 of decode(code) * 2^de.
+// Used for |de| <= 100, where every product is a normal bf16 value.
+__device__ __forceinline__ bool fp6_decode_hw_ok(int de) { return de >= -100 && de <= 100; }
+template <int F> __device__ __forceinline__ u32x16 fp6_block_decode_hw(u32x6 codes, int de) {
+    const float scale = u2f((uint32_t)(127 + de) << 23);
+    if constexpr (F == FMT_E2M3) return __builtin_bit_cast(u32x16, __builtin_amdgcn_cvt_scalef32_pk32_bf16_fp6(codes, scale));
+    else return __builtin_bit_cast(u32x16, __builtin_amdgcn_cvt_scalef32_pk32_bf16_bf6(codes, scale));
+}
 // the same 6 words from the software codes of 16 packed pairs
 template <int F> __device__ __forceinline__ u32x6 fp6_block_sw(const uint32_t (&words)[16], int e8) {
     uint32_t p[16];
@@ -455,6 +463,21 @@ __global__ __launch_bounds__(WWG) void k_mx_dequantize(const uint8_t* payload, c
             x[0] = hw_unpack<F, 0>(q.x); x[1] = hw_unpack<F, 1>(q.x); x[2] = hw_unpack<F, 2>(q.x); x[3] = hw_unpack<F, 3>(q.x);
             x[4] = hw_unpack<F, 0>(q.y); x[5] = hw_unpack<F, 1>(q.y); x[6] = hw_unpack<F, 2>(q.y); x[7] = hw_unpack<F, 3>(q.y);
         } else {
+            if (fp6_decode_hw_ok(de)) {
+                // every lane of the quad reads its block's 24 bytes (same addresses: one fetch) and decodes all 32 codes
+                // with one block convert, then keeps its own 8 values
+                const uint2* blk = reinterpret_cast<const uint2*>(payload + (c >> 2) * 24);
+                const uint2 b0 = blk[0], b1 = blk[1], b2 = blk[2];
+                const u32x16 t = fp6_block_decode_hw<F>(u32x6{b0.x, b0.y, b1.x, b1.y, b2.x, b2.y}, de);
+                const int j = (int)(c & 3);
+                uint4 r;
+                r.x = j == 0 ? t[0] : j == 1 ? t[4] : j == 2 ? t[8] : t[12];
+                r.y = j == 0 ? t[1] : j == 1 ? t[5] : j == 2 ? t[9] : t[13];
+                r.z = j == 0 ? t[2] : j == 1 ? t[6] : j == 2 ? t[10] : t[14];
+                r.w = j == 0 ? t[3] : j == 1 ? t[7] : j == 2 ? t[11] : t[15];
+                store16_rt(out + c, r, streams_out(nchunks * 8));
+                continue;
+            }
             const uint16_t* p = reinterpret_cast<const uint16_t*>(payload + (c >> 2) * 24 + (c & 3) * 6);
             const uint64_t bits = (uint64_t)p[0] | ((uint64_t)p[1] << 16) | ((uint64_t)p[2] << 32);
 #pragma unroll
@@ -496,6 +519,32 @@ __global__ __launch_bounds__(WWG) void k_selftest_hw_fp6(unsigned long long* mis
         uint32_t x = (a[g] ^ b[g]) >> sh;
         if (sh > 26 && g < 5) x |= (a[g + 1] ^ b[g + 1]) << (32 - sh);
         bad += (x & 0x3Fu) != 0;
+    }
+    if (bad) atomicAdd(mismatches + (F == FMT_E2M3 ? 0 : 1), (unsigned long long)bad);
+}
+
+// The inverse convert: the 64 codes (two groups of 32) with every scale exponent it is used with.
+template <int F>
+__global__ __launch_bounds__(WWG) void k_selftest_hw_fp6_decode(unsigned long long* mismatches) {
+    const int idx = blockIdx.x * WWG + threadIdx.x;
+    if (idx >= 2 * 201) return;
+    const int half = idx & 1, de = (idx >> 1) - 100;
+    uint32_t d[6] = {0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+        const uint64_t code = (uint64_t)(half * 32 + j) << ((6 * j) & 31);
+        d[(6 * j) >> 5] |= (uint32_t)code;
+        if (((6 * j) >> 5) < 5) d[((6 * j) >> 5) + 1] |= (uint32_t)(code >> 32);
+    }
+    const u32x16 t = fp6_block_decode_hw<F>(u32x6{d[0], d[1], d[2], d[3], d[4], d[5]}, de);
+    unsigned bad = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t c0 = half * 32 + 2 * i, c1 = c0 + 1;
+        const float v0 = u2f(f2u(fp6_value<F>(c0 & 0x1Fu)) | ((c0 & 0x20u) << 26)), v1 = u2f(f2u(fp6_value<F>(c1 & 0x1Fu)) | ((c1 & 0x20u) << 26));
+        const uint32_t want = store_pair<true>(ldexpf(v0, de), ldexpf(v1, de));
+        bad += ((t[i] ^ want) & 0xFFFFu) != 0;
+        bad += ((t[i] ^ want) >> 16) != 0;
     }
     if (bad) atomicAdd(mismatches + (F == FMT_E2M3 ? 0 : 1), (unsigned long long)bad);
 }
@@ -612,5 +661,7 @@ extern "C" int mor_selftest_hw_fp6(uint64_t* mismatches, void* stream) {
     const unsigned grid = (2048u * 253u + WWG - 1) / WWG;
     k_selftest_hw_fp6<FMT_E2M3><<<grid, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
     k_selftest_hw_fp6<FMT_E3M2><<<grid, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
+    k_selftest_hw_fp6_decode<FMT_E2M3><<<2, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
+    k_selftest_hw_fp6_decode<FMT_E3M2><<<2, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
     return mor_check_launch("k_selftest_hw_fp6");
 }
