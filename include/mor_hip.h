@@ -132,12 +132,13 @@ MOR_API int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t
 MOR_API int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
 
 /*
- * The same for the gfx950 block convert of 32 bf16 values to packed FP6 (used by the MX wire format):
- * every finite bf16 value with every scale exponent against the software codes, and the inverse
- * convert (codes to bf16) for every code and scale exponent it is used with.
- * mismatches[0] = E2M3 count, mismatches[1] = E3M2 count (device pointer, 2 x uint64).
+ * The same for the gfx950 scaled converts the MX wire format uses: the block convert of 32 bf16
+ * values to packed FP6 (every finite bf16 value with every scale exponent, against the software
+ * codes), its inverse, and the FP8 -> bf16 scaled convert of the dequantizer (every finite code
+ * with every scale exponent it is used with).  mismatches[MOR_FMT_*] = count per element format
+ * (device pointer, 4 x uint64).
  */
-MOR_API int mor_selftest_hw_fp6(uint64_t* mismatches, void* stream);
+MOR_API int mor_selftest_hw_wire(uint64_t* mismatches, void* stream);
 
 /*
  * MX wire format: the quantized tensor itself instead of its dequantized bf16 image.

@@ -81,7 +81,7 @@ template <int F> __device__ __forceinline__ uint64_t code_chunk(uint4 v, int e8)
 }
 
 // FP6 by the gfx950 block convert: v_cvt_scalef32_pk32_{fp6,bf6}_bf16 turns 32 bf16 values into 32 packed 6-bit codes
-// of RNE(x / 2^floor(log2(scale))), saturating, sign kept (E2M3 = "fp6", E3M2 = "bf6"); mor_selftest_hw_fp6 compares it
+// of RNE(x / 2^floor(log2(scale))), saturating, sign kept (E2M3 = "fp6", E3M2 = "bf6"); mor_selftest_hw_wire compares it
 // with the software codes over every bf16 value and every scale exponent.  Used when 2^-e8 is a normal float.
 typedef __bf16 bf16x32 __attribute__((ext_vector_type(32)));
 typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
@@ -103,6 +103,11 @@ template <int F> __device__ __forceinline__ u32x16 fp6_block_decode_hw(u32x6 cod
     const float scale = u2f((uint32_t)(127 + de) << 23);
     if constexpr (F == FMT_E2M3) return __builtin_bit_cast(u32x16, __builtin_amdgcn_cvt_scalef32_pk32_bf16_fp6(codes, scale));
     else return __builtin_bit_cast(u32x16, __builtin_amdgcn_cvt_scalef32_pk32_bf16_bf6(codes, scale));
+}
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+template <int F, bool HIGH> __device__ __forceinline__ uint32_t fp8_pair_decode_hw(uint32_t codes, float scale) {
+    if constexpr (F == FMT_E4M3) return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)codes, scale, HIGH));
+    else return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8((int)codes, scale, HIGH));
 }
 // the same 6 words from the software codes of 16 packed pairs
 template <int F> __device__ __forceinline__ u32x6 fp6_block_sw(const uint32_t (&words)[16], int e8) {
@@ -460,6 +465,14 @@ __global__ __launch_bounds__(WWG) void k_mx_dequantize(const uint8_t* payload, c
         float x[8];
         if constexpr (Fmt<F>::hw) {
             const uint2 q = *reinterpret_cast<const uint2*>(payload + c * 8);
+            if (fp6_decode_hw_ok(de)) {          // v_cvt_scalef32_pk_bf16_{fp8,bf8}: two codes -> two bf16 of decode * 2^de
+                const float scale = u2f((uint32_t)(127 + de) << 23);
+                uint4 r;
+                r.x = fp8_pair_decode_hw<F, false>(q.x, scale); r.y = fp8_pair_decode_hw<F, true>(q.x, scale);
+                r.z = fp8_pair_decode_hw<F, false>(q.y, scale); r.w = fp8_pair_decode_hw<F, true>(q.y, scale);
+                store16_rt(out + c, r, streams_out(nchunks * 8));
+                continue;
+            }
             x[0] = hw_unpack<F, 0>(q.x); x[1] = hw_unpack<F, 1>(q.x); x[2] = hw_unpack<F, 2>(q.x); x[3] = hw_unpack<F, 3>(q.x);
             x[4] = hw_unpack<F, 0>(q.y); x[5] = hw_unpack<F, 1>(q.y); x[6] = hw_unpack<F, 2>(q.y); x[7] = hw_unpack<F, 3>(q.y);
         } else {
@@ -520,7 +533,7 @@ __global__ __launch_bounds__(WWG) void k_selftest_hw_fp6(unsigned long long* mis
         if (sh > 26 && g < 5) x |= (a[g + 1] ^ b[g + 1]) << (32 - sh);
         bad += (x & 0x3Fu) != 0;
     }
-    if (bad) atomicAdd(mismatches + (F == FMT_E2M3 ? 0 : 1), (unsigned long long)bad);
+    if (bad) atomicAdd(mismatches + F, (unsigned long long)bad);
 }
 
 // The inverse convert: the 64 codes (two groups of 32) with every scale exponent it is used with.
@@ -546,7 +559,23 @@ __global__ __launch_bounds__(WWG) void k_selftest_hw_fp6_decode(unsigned long lo
         bad += ((t[i] ^ want) & 0xFFFFu) != 0;
         bad += ((t[i] ^ want) >> 16) != 0;
     }
-    if (bad) atomicAdd(mismatches + (F == FMT_E2M3 ? 0 : 1), (unsigned long long)bad);
+    if (bad) atomicAdd(mismatches + F, (unsigned long long)bad);
+}
+
+// v_cvt_scalef32_pk_bf16_{fp8,bf8} (dequantize): the 254 finite-or-not codes as they come, every scale exponent used.
+template <int F>
+__global__ __launch_bounds__(WWG) void k_selftest_hw_fp8_decode(unsigned long long* mismatches) {
+    const int idx = blockIdx.x * WWG + threadIdx.x;
+    if (idx >= 128 * 201) return;
+    const uint32_t c0 = 2u * (idx & 127), c1 = c0 + 1u;
+    const int de = (idx >> 7) - 100;
+    const float v0 = hw_unpack<F, 0>(c0 | (c1 << 8)), v1 = hw_unpack<F, 1>(c0 | (c1 << 8));
+    if (v0 != v0 || v1 != v1 || fabsf(v0) > Fmt<F>::fmax || fabsf(v1) > Fmt<F>::fmax) return;     // NaN / Inf codes are never produced
+    const uint32_t want = store_pair<true>(ldexpf(v0, de), ldexpf(v1, de));
+    const uint32_t got = fp8_pair_decode_hw<F, false>(c0 | (c1 << 8), u2f((uint32_t)(127 + de) << 23));
+    const uint32_t got_hi = fp8_pair_decode_hw<F, true>((c0 | (c1 << 8)) << 16, u2f((uint32_t)(127 + de) << 23));
+    const unsigned bad = (got != want) + (got_hi != want);
+    if (bad) atomicAdd(mismatches + F, (unsigned long long)bad);
 }
 
 }  // namespace mor
@@ -653,15 +682,17 @@ extern "C" int mor_fake_quantize_dual(const void* input, void* output_rows, int3
     return mor_check_launch("k_fq_dual");
 }
 
-extern "C" int mor_selftest_hw_fp6(uint64_t* mismatches, void* stream) {
+extern "C" int mor_selftest_hw_wire(uint64_t* mismatches, void* stream) {
     if (!mismatches) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mismatches is NULL");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = hipMemsetAsync(mismatches, 0, 2 * sizeof(uint64_t), st);
+    hipError_t e = hipMemsetAsync(mismatches, 0, 4 * sizeof(uint64_t), st);
     if (e != hipSuccess) return mor_fail(MOR_ERR_LAUNCH, "hipMemsetAsync: %s", hipGetErrorString(e));
     const unsigned grid = (2048u * 253u + WWG - 1) / WWG;
     k_selftest_hw_fp6<FMT_E2M3><<<grid, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
     k_selftest_hw_fp6<FMT_E3M2><<<grid, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
     k_selftest_hw_fp6_decode<FMT_E2M3><<<2, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
     k_selftest_hw_fp6_decode<FMT_E3M2><<<2, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
-    return mor_check_launch("k_selftest_hw_fp6");
+    k_selftest_hw_fp8_decode<FMT_E4M3><<<(128 * 201 + WWG - 1) / WWG, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
+    k_selftest_hw_fp8_decode<FMT_E5M2><<<(128 * 201 + WWG - 1) / WWG, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
+    return mor_check_launch("k_selftest_hw_wire");
 }

@@ -147,11 +147,12 @@ def test_python_api_round_trip():
     assert p6.shape == (256, 384) and wire.dequantize_mx(p6, s6, wire.E2M3).shape == (256, 512)
 
 
-def test_hw_fp6_block_convert_selftest(G):
-    """v_cvt_scalef32_pk32_{fp6,bf6}_bf16 against the software codes: 65 280 finite bf16 values x 253 scale exponents."""
+def test_hw_scaled_converts_selftest(G):
+    """The gfx950 scaled converts of the wire-format kernels against the software codes / values: FP6 block convert
+    (65 280 finite bf16 values x 253 scale exponents), its inverse and the FP8 decode (every code x 201 exponents)."""
     from mor_amd import _cabi
     L = _cabi.lib()
-    bad = torch.full((2,), -1, dtype=torch.int64, device="cuda")
-    _cabi.check(L.mor_selftest_hw_fp6(bad.data_ptr(), None))
+    bad = torch.full((4,), -1, dtype=torch.int64, device="cuda")
+    _cabi.check(L.mor_selftest_hw_wire(bad.data_ptr(), None))
     torch.cuda.synchronize()
-    assert bad.tolist() == [0, 0]
+    assert bad.tolist() == [0, 0, 0, 0]
