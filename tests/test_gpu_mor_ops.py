@@ -269,3 +269,43 @@ def test_ops_trace_under_torch_compile(mor):
     got = torch.compile(f, backend="aot_eager", fullgraph=True)(w)
     got.backward()
     assert torch.equal(got, want) and torch.equal(w.grad, g_eager) and torch.all(g_eager == 1)
+
+
+def test_concurrent_streams_and_host_threads(mor):
+    """The library keeps no state between calls: four host threads, each on its own stream with its own tensors,
+    interleave different ops and get what a single-threaded run gets."""
+    import threading
+    xs = [random_bf16(100 + i, -8.0, 8.0, 512, 1024).cuda() for i in range(4)]
+
+    def work(x):
+        a = mor.ops.fake_quantize(x, 512, 1024, 128, 128, clamp_threshold=1e-15, mode=1, sf_type=1)
+        b = mor.ops.fake_quantize(x, 512, 1024, 1, 32, clamp_threshold=0.0, mode=2, sf_type=2)
+        c = mor.ops.fake_quantize_block_scaling(x, 512, 1024, 128, 128, e4m3_threshold=0.045, ss_mode=1)
+        d = mor.ops.fake_quantize_channel_scaling(x, 512, 1024, 1, 1024, e4m3_threshold=0.045, ss_mode=3)
+        e = mor.ops.fake_quantize_e8mx(x, 512, 1024, 128, 128, quantize_type=2, scaling_strategy=1)
+        return list(a) + list(b) + list(c) + list(d) + [e]
+
+    want = [work(x) for x in xs]
+    torch.cuda.synchronize()
+    got = [None] * 4
+    errors = []
+
+    def run(i):
+        try:
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                for _ in range(20):
+                    got[i] = work(xs[i])
+            s.synchronize()
+        except Exception as exc:                      # surfaced below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(4):
+        for a, b in zip(got[i], want[i]):
+            assert torch.equal(a, b), i
