@@ -364,4 +364,40 @@ __device__ __forceinline__ void acc_amin(uint32_t& amin_m1, uint32_t w) {
 }
 constexpr uint32_t AMIN_INIT_M1 = 0x7F7F0000u - 1u;   // bf16 max, FQ:409-412
 
+
+// ---------------------------------------------------------------- gfx950 block converts (32 values per lane)
+// FP6 by the gfx950 block convert: v_cvt_scalef32_pk32_{fp6,bf6}_bf16 turns 32 bf16 values into 32 packed 6-bit codes
+// of RNE(x / 2^floor(log2(scale))), saturating, sign kept (E2M3 = "fp6", E3M2 = "bf6"); the library's selftest compares
+// it with the software codes over every bf16 value and every scale exponent.  Used when 2^-e8 is a normal float.
+typedef __bf16 bf16x32 __attribute__((ext_vector_type(32)));
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x6 __attribute__((ext_vector_type(6)));
+__device__ __forceinline__ bool fp6_hw_ok(int e8) { return e8 >= -126 && e8 <= 126; }
+template <int F> __device__ __forceinline__ u32x6 fp6_block_hw(const uint32_t (&words)[16], int e8) {
+    const float scale = u2f((uint32_t)(127 - e8) << 23);
+    u32x16 t;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) t[i] = words[i];
+    const bf16x32 x = __builtin_bit_cast(bf16x32, t);
+    if constexpr (F == FMT_E2M3) return __builtin_bit_cast(u32x6, __builtin_amdgcn_cvt_scalef32_pk32_fp6_bf16(x, scale));
+    else return __builtin_bit_cast(u32x6, __builtin_amdgcn_cvt_scalef32_pk32_bf6_bf16(x, scale));
+}
+// The inverse block convert, v_cvt_scalef32_pk32_bf16_{fp6,bf6}: 32 packed codes -> 32 bf16 of decode(code) * 2^de.
+// Used for |de| <= 100, where every product is a normal bf16 value.
+__device__ __forceinline__ bool fp6_decode_hw_ok(int de) { return de >= -100 && de <= 100; }
+template <int F> __device__ __forceinline__ u32x16 fp6_block_decode_hw(u32x6 codes, int de) {
+    const float scale = u2f((uint32_t)(127 + de) << 23);
+    if constexpr (F == FMT_E2M3) return __builtin_bit_cast(u32x16, __builtin_amdgcn_cvt_scalef32_pk32_bf16_fp6(codes, scale));
+    else return __builtin_bit_cast(u32x16, __builtin_amdgcn_cvt_scalef32_pk32_bf16_bf6(codes, scale));
+}
+// quad_perm [J,J,J,J]: every lane of a quad reads lane J of its quad
+template <int J> __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) { return dpp_u<J * 0x55>(v); }
+// the 4 chunks (16 words) of a quad's block in every lane of the quad
+__device__ __forceinline__ void quad_gather(uint4 v, uint32_t (&w)[16]) {
+    w[0] = quad_bcast<0>(v.x); w[1] = quad_bcast<0>(v.y); w[2] = quad_bcast<0>(v.z); w[3] = quad_bcast<0>(v.w);
+    w[4] = quad_bcast<1>(v.x); w[5] = quad_bcast<1>(v.y); w[6] = quad_bcast<1>(v.z); w[7] = quad_bcast<1>(v.w);
+    w[8] = quad_bcast<2>(v.x); w[9] = quad_bcast<2>(v.y); w[10] = quad_bcast<2>(v.z); w[11] = quad_bcast<2>(v.w);
+    w[12] = quad_bcast<3>(v.x); w[13] = quad_bcast<3>(v.y); w[14] = quad_bcast<3>(v.z); w[15] = quad_bcast<3>(v.w);
+}
+
 }  // namespace mor

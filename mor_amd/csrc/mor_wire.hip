@@ -80,30 +80,6 @@ template <int F> __device__ __forceinline__ uint64_t code_chunk(uint4 v, int e8)
            ((uint64_t)code_pair<F>(v.z, e8) << (2 * pb)) | ((uint64_t)code_pair<F>(v.w, e8) << (3 * pb));
 }
 
-// FP6 by the gfx950 block convert: v_cvt_scalef32_pk32_{fp6,bf6}_bf16 turns 32 bf16 values into 32 packed 6-bit codes
-// of RNE(x / 2^floor(log2(scale))), saturating, sign kept (E2M3 = "fp6", E3M2 = "bf6"); mor_selftest_hw_wire compares it
-// with the software codes over every bf16 value and every scale exponent.  Used when 2^-e8 is a normal float.
-typedef __bf16 bf16x32 __attribute__((ext_vector_type(32)));
-typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x6 __attribute__((ext_vector_type(6)));
-__device__ __forceinline__ bool fp6_hw_ok(int e8) { return e8 >= -126 && e8 <= 126; }
-template <int F> __device__ __forceinline__ u32x6 fp6_block_hw(const uint32_t (&words)[16], int e8) {
-    const float scale = u2f((uint32_t)(127 - e8) << 23);
-    u32x16 t;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) t[i] = words[i];
-    const bf16x32 x = __builtin_bit_cast(bf16x32, t);
-    if constexpr (F == FMT_E2M3) return __builtin_bit_cast(u32x6, __builtin_amdgcn_cvt_scalef32_pk32_fp6_bf16(x, scale));
-    else return __builtin_bit_cast(u32x6, __builtin_amdgcn_cvt_scalef32_pk32_bf6_bf16(x, scale));
-}
-// The inverse block convert, v_cvt_scalef32_pk32_bf16_{fp6,bf6}: 32 packed codes -> 32 bf16 of decode(code) * 2^de.
-// Used for |de| <= 100, where every product is a normal bf16 value.
-__device__ __forceinline__ bool fp6_decode_hw_ok(int de) { return de >= -100 && de <= 100; }
-template <int F> __device__ __forceinline__ u32x16 fp6_block_decode_hw(u32x6 codes, int de) {
-    const float scale = u2f((uint32_t)(127 + de) << 23);
-    if constexpr (F == FMT_E2M3) return __builtin_bit_cast(u32x16, __builtin_amdgcn_cvt_scalef32_pk32_bf16_fp6(codes, scale));
-    else return __builtin_bit_cast(u32x16, __builtin_amdgcn_cvt_scalef32_pk32_bf16_bf6(codes, scale));
-}
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 template <int F, bool HIGH> __device__ __forceinline__ uint32_t fp8_pair_decode_hw(uint32_t codes, float scale) {
     if constexpr (F == FMT_E4M3) return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)codes, scale, HIGH));
@@ -139,7 +115,6 @@ __device__ __forceinline__ float chunk_amax(uint4 v) {
 // FP8: 8 bytes per lane.  FP6: the quad's 16 words are broadcast to its lanes (DPP), every lane converts the whole
 // block with one instruction and lanes 0..2 store 8 of the 24 bytes each; outside the range of the block convert the
 // software codes are merged across the quad instead.
-template <int J> __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) { return dpp_u<J * 0x55>(v); }
 template <int F> __device__ __forceinline__ void emit_chunk(uint8_t* payload, int64_t c, uint4 v, int e8, bool ok) {
     if constexpr (Fmt<F>::hw) {
         const uint64_t codes = code_chunk<F>(v, e8);
@@ -149,10 +124,7 @@ template <int F> __device__ __forceinline__ void emit_chunk(uint8_t* payload, in
         uint32_t lo, hi;
         if (fp6_hw_ok(e8)) {                                     // uniform over the quad (e8 is the block's)
             uint32_t w[16];
-            w[0] = quad_bcast<0>(v.x); w[1] = quad_bcast<0>(v.y); w[2] = quad_bcast<0>(v.z); w[3] = quad_bcast<0>(v.w);
-            w[4] = quad_bcast<1>(v.x); w[5] = quad_bcast<1>(v.y); w[6] = quad_bcast<1>(v.z); w[7] = quad_bcast<1>(v.w);
-            w[8] = quad_bcast<2>(v.x); w[9] = quad_bcast<2>(v.y); w[10] = quad_bcast<2>(v.z); w[11] = quad_bcast<2>(v.w);
-            w[12] = quad_bcast<3>(v.x); w[13] = quad_bcast<3>(v.y); w[14] = quad_bcast<3>(v.z); w[15] = quad_bcast<3>(v.w);
+            quad_gather(v, w);
             const u32x6 d = fp6_block_hw<F>(w, e8);
             lo = j == 0 ? d[0] : j == 1 ? d[2] : d[4];
             hi = j == 0 ? d[1] : j == 1 ? d[3] : d[5];
