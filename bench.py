@@ -129,6 +129,11 @@ def main():
         print("bench.py measures one GPU: every quantization block is independent, so more GPUs only shard rows; "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("mor_amd_build", os.path.join(ROOT, "mor_amd", "build.py"))
+    build_mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build_mod)
+    build_mod.ensure_built()                # nothing to do when the libraries travelled with the tree
     import torch
     from mor_amd import _cabi
     if not torch.cuda.is_available():

@@ -52,6 +52,14 @@ def build_torch_binding(verbose=False):
     return TORCH_BINDING_OUT
 
 
+def ensure_built(verbose=False):
+    """Builds what is missing (used by the tests, the smoke check and the benchmark; build() always rebuilds)."""
+    if not os.path.exists(OUT):
+        build_hip(verbose)
+    if not os.path.exists(TORCH_BINDING_OUT):
+        build_torch_binding(verbose)
+
+
 if __name__ == "__main__":
     print(build_hip(verbose=True))
     print(build_torch_binding(verbose=True))

@@ -11,6 +11,12 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    # the libraries are built beforehand and travel with the tree; build them only if nothing is there
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("mor_amd_build", os.path.join(ROOT, "mor_amd", "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    mod.ensure_built()
 
 
 @pytest.fixture(scope="session")
