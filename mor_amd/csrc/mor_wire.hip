@@ -174,21 +174,22 @@ __global__ __launch_bounds__(WWG) void k_mx_quantize(const uint4* in, uint8_t* p
 // both orientations from one read.  Tile TR rows x 128 columns (TR = 64 or 128); rows % 32 == 0, cols % 32 == 0.
 constexpr int TILE_C = 128;
 constexpr int TILE_ROWS = 128;
+constexpr int DUAL_THREADS = 512;
 
-template <int F, int TR>
-__global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_payload, uint8_t* row_scales,
+template <int F, int TR, int DT>
+__global__ __launch_bounds__(DT) void k_mx_dual(const uint4* in, uint8_t* row_payload, uint8_t* row_scales,
                                                  uint8_t* col_payload, uint8_t* col_scales, int64_t rows, int64_t cols) {
     constexpr int PITCH = TILE_C + 8;             // bf16 elements per LDS row; keeps the row starts 16-byte aligned
-    constexpr int NV = TR * (TILE_C / 8) / WWG;   // 16-byte chunks per thread
+    constexpr int NV = TR * (TILE_C / 8) / DT;   // 16-byte chunks per thread
     constexpr int RB = TR / 32;                   // row blocks per tile column
-    constexpr int BPT = TILE_C * RB / WWG;        // column blocks per thread
+    constexpr int BPT = TILE_C * RB / DT;        // column blocks per thread
     constexpr int blk_bytes = 32 * Wire<F>::bits / 8;
     constexpr int SEG = Fmt<F>::hw ? 16 : 8;      // bytes per lane of the column stores (both divide blk_bytes)
     constexpr int CODE_PITCH = (RB * blk_bytes + 16 + 15) / 16 * 16;   // bytes per column of the code tile (padded, 16-byte aligned)
     constexpr int SEGS = RB * blk_bytes / SEG;    // per column
     // one buffer, two uses: the bf16 tile, then the codes of the column blocks (smaller)
     __shared__ __attribute__((aligned(16))) uint16_t tile[TR * PITCH];
-    __shared__ uint32_t s_cscale[TILE_C];
+    __shared__ __attribute__((aligned(4))) uint8_t s_cscale[TILE_C * 4];
     uint8_t* codes = reinterpret_cast<uint8_t*>(tile);
     static_assert(TILE_C * CODE_PITCH <= TR * PITCH * 2, "the code tile must fit the bf16 tile");
     const int tid = threadIdx.x;
@@ -202,14 +203,14 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
     bool ok[NV];
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
-        const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+        const int ch = k * DT + tid, r = ch >> 4, cc = ch & 15;
         ok[k] = (r < rows_valid) && (cc * 8 < cols_valid);
         v[k] = make_uint4(0, 0, 0, 0);
         if (ok[k]) v[k] = in[(R0 + r) * row_chunks + (C0 >> 3) + cc];
     }
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
-        const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+        const int ch = k * DT + tid, r = ch >> 4, cc = ch & 15;
         *reinterpret_cast<uint4*>(&tile[r * PITCH + cc * 8]) = v[k];
     }
     __syncthreads();
@@ -230,7 +231,7 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
     const bool dword_row_scales = (cols & 127) == 0;
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
-        const int ch = k * WWG + tid, r = ch >> 4, cc = ch & 15;
+        const int ch = k * DT + tid, r = ch >> 4, cc = ch & 15;
         const float amax = group_max_t<4>(chunk_amax(v[k]), 4);
         const int e8 = wire_e8<F>(amax);
         const int64_t cidx = (R0 + r) * row_chunks + (C0 >> 3) + cc;       // chunk index in the row-major payload
@@ -243,7 +244,6 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
     }
     __syncthreads();                              // every thread has its column blocks in registers: reuse the buffer
 
-    uint32_t my_scales = 0;
 #pragma unroll
     for (int h = 0; h < BPT; ++h) {
         const int rb = (tid >> 7) * BPT + h;
@@ -251,7 +251,7 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc_amax(amax, w[h][i]);
         const int e8 = wire_e8<F>(amax);
-        my_scales |= (uint32_t)(127 - e8) << (8 * h);
+        s_cscale[c * 4 + rb] = (uint8_t)(127 - e8);
         uint8_t* dst = codes + c * CODE_PITCH + rb * blk_bytes;
         if constexpr (Fmt<F>::hw) {
             uint32_t q[8];
@@ -266,7 +266,6 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
             *reinterpret_cast<uint2*>(dst + 16) = make_uint2(d[4], d[5]);
         }
     }
-    if (tid >= TILE_C) s_cscale[c] = my_scales;
     __syncthreads();
 
     // the transposed payload: a column of the tile is RB * blk_bytes contiguous bytes, SEGS lanes store one column
@@ -275,16 +274,16 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
     if (SEG == 16 || ((col_row_bytes & 15) == 0 && rows_valid == TR)) {      // 16 bytes per lane wherever they are aligned
         constexpr int S16 = RB * blk_bytes / 16;
 #pragma unroll
-        for (int i = 0; i < (TILE_C * S16 + WWG - 1) / WWG; ++i) {
-            const int idx = i * WWG + tid, col = idx / S16, seg = idx % S16;
+        for (int i = 0; i < (TILE_C * S16 + DT - 1) / DT; ++i) {
+            const int idx = i * DT + tid, col = idx / S16, seg = idx % S16;
             if (col < cols_valid && seg * 16 < valid_bytes && idx < TILE_C * S16)
                 store16_rt(reinterpret_cast<uint4*>(col_payload + (C0 + col) * col_row_bytes + (R0 / 32) * blk_bytes + seg * 16),
                            *reinterpret_cast<const uint4*>(codes + col * CODE_PITCH + seg * 16), nt);
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < TILE_C * SEGS / WWG; ++i) {
-            const int idx = i * WWG + tid, col = idx / SEGS, seg = idx % SEGS;
+        for (int i = 0; i < TILE_C * SEGS / DT; ++i) {
+            const int idx = i * DT + tid, col = idx / SEGS, seg = idx % SEGS;
             if (col < cols_valid && seg * SEG < valid_bytes)
                 *reinterpret_cast<uint2*>(col_payload + (C0 + col) * col_row_bytes + (R0 / 32) * blk_bytes + seg * SEG) =
                     *reinterpret_cast<const uint2*>(codes + col * CODE_PITCH + seg * SEG);
@@ -292,7 +291,7 @@ __global__ __launch_bounds__(WWG) void k_mx_dual(const uint4* in, uint8_t* row_p
     }
     // scale bytes of the column blocks: RB per column and tile
     if (tid < TILE_C && c < cols_valid) {
-        const uint32_t sall = my_scales | (s_cscale[c] << (8 * BPT));
+        const uint32_t sall = *reinterpret_cast<const uint32_t*>(&s_cscale[c * 4]);
         uint8_t* dst = col_scales + (C0 + c) * (rows / 32) + R0 / 32;
         if (RB == 4 && (rows & 127) == 0) *reinterpret_cast<uint32_t*>(dst) = sall;
         else if (RB == 2 && (rows & 63) == 0) *reinterpret_cast<uint16_t*>(dst) = (uint16_t)sall;
@@ -599,10 +598,10 @@ extern "C" int mor_mx_quantize_dual(const void* input, void* row_payload, void* 
     uint8_t *rp = static_cast<uint8_t*>(row_payload), *rs = static_cast<uint8_t*>(row_scales);
     uint8_t *cp = static_cast<uint8_t*>(col_payload), *cs = static_cast<uint8_t*>(col_scales);
     switch (fmt) {
-        case MOR_FMT_E4M3: k_mx_dual<FMT_E4M3, TILE_ROWS><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
-        case MOR_FMT_E5M2: k_mx_dual<FMT_E5M2, TILE_ROWS><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
-        case MOR_FMT_E3M2: k_mx_dual<FMT_E3M2, TILE_ROWS><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
-        default: k_mx_dual<FMT_E2M3, TILE_ROWS><<<(unsigned)tiles, WWG, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        case MOR_FMT_E4M3: k_mx_dual<FMT_E4M3, TILE_ROWS, DUAL_THREADS><<<(unsigned)tiles, DUAL_THREADS, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        case MOR_FMT_E5M2: k_mx_dual<FMT_E5M2, TILE_ROWS, DUAL_THREADS><<<(unsigned)tiles, DUAL_THREADS, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        case MOR_FMT_E3M2: k_mx_dual<FMT_E3M2, TILE_ROWS, DUAL_THREADS><<<(unsigned)tiles, DUAL_THREADS, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
+        default: k_mx_dual<FMT_E2M3, TILE_ROWS, DUAL_THREADS><<<(unsigned)tiles, DUAL_THREADS, 0, st>>>(in, rp, rs, cp, cs, rows, cols); break;
     }
     return mor_check_launch("k_mx_dual");
 }
