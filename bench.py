@@ -200,8 +200,9 @@ def main():
         "metric": "fake-quant HBM GB/s (rd+wr), MX 1x32 E8M0 block scaling on 8192x8192 bf16 (E4M3+E5M2+E2M3)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 in/out, fp32 + fp8/fp6 arithmetic", "data": "synthetic",
+        "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"configs[1]: MX block scaling {rows}x{cols} bf16, 1x32 blocks, E8M0 scale, E4M3+E5M2+E2M3 per step",
+                   "arithmetic": "bf16 tensors, fp32 / integer arithmetic, gfx950 fp8 / fp6 converts",
                    "elements_per_s": round(3 * nelem / (ms_per_step * 1e-3), 0), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": roofline,
         "cpu_baseline": cpu,
