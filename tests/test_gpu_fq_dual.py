@@ -45,6 +45,21 @@ def test_both_orientations_match_oracle(G, mode, sf):
     assert np.all(meta == -7) and np.all(meta_t == -7) and np.array_equal(out, want)
 
 
+# tile grids (128 x 128 tiles) that take each of the workgroup -> tile orders the kernel chooses between
+@pytest.mark.parametrize("rows,cols,mode,sf", [(1024, 512, 2, 2), (2048, 1024, 3, 1), (4096, 1024, 2, 1), (1024, 4096, 3, 2),
+                                               (2048, 4096, 2, 2), (8192, 512, 3, 2), (256, 8192, 2, 1), (128, 8192, 2, 2),
+                                               (1152, 1280, 3, 1)])
+def test_tile_orders_match_oracle(G, rows, cols, mode, sf):
+    print("fq_dual tile order", rows, cols, mode, sf, flush=True)
+    a = data_gen.c2_student_t(rows, cols, seed=rows + cols)
+    want, wmeta = O.fake_quantize(a, 1, 32, 0.0, mode, sf)
+    want_t, wmeta_t = O.fake_quantize(np.ascontiguousarray(a.T), 1, 32, 0.0, mode, sf)
+    out, meta, out_t, meta_t = G.fake_quantize_dual(a, mode, sf)
+    for got, exp, what in ((out, want, "rows"), (out_t, want_t, "columns"), (meta, wmeta, "meta"), (meta_t, wmeta_t, "meta_t")):
+        bad = np.argwhere(got != exp)
+        assert len(bad) == 0, (what, len(bad), tuple(bad[0]))
+
+
 def test_argument_checks(G):
     from mor_amd import _cabi
     L = _cabi.lib()

@@ -59,6 +59,24 @@ def test_dual_matches_oracle_on_the_tensor_and_its_transpose(G, fmt):
         assert first_diff(cp, tp) is None, (name, "column payload", first_diff(cp, tp))
 
 
+# tile grids (128 x 128 tiles) that take each of the workgroup -> tile orders the dual kernels choose between
+TILE_ORDER_SHAPES = [(1024, 512), (2048, 1024), (1024, 2048), (4096, 1024), (1024, 4096), (2048, 4096), (8192, 512),
+                     (256, 8192), (128, 8192), (1152, 1280)]
+
+
+@pytest.mark.parametrize("k", range(len(TILE_ORDER_SHAPES)))
+def test_dual_tile_orders_match_oracle(G, k):
+    rows, cols = TILE_ORDER_SHAPES[k]
+    fmt = FORMATS[k % 4]
+    print("mx_quantize_dual tile order", rows, cols, fmt, flush=True)
+    a = data_gen.c2_student_t(rows, cols, seed=60 + k)
+    wp, ws = O.mx_quantize(a, fmt)
+    tp, ts = O.mx_quantize(np.ascontiguousarray(a.T), fmt)
+    rp, rs, cp, cs = G.mx_quantize_dual(a, fmt)
+    assert first_diff(rs, ws) is None and first_diff(rp, wp) is None, ("rows", first_diff(rs, ws), first_diff(rp, wp))
+    assert first_diff(cs, ts) is None and first_diff(cp, tp) is None, ("columns", first_diff(cs, ts), first_diff(cp, tp))
+
+
 @pytest.mark.parametrize("fmt", FORMATS)
 def test_dequantize_matches_oracle(G, fmt):
     for name, a in cases():
