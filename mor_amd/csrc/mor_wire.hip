@@ -254,9 +254,11 @@ __global__ __launch_bounds__(DT) void k_mx_dual(const uint4* in, uint8_t* row_pa
             w[h][i] = (uint32_t)tile[(rb * 32 + 2 * i) * PITCH + c] | ((uint32_t)tile[(rb * 32 + 2 * i + 1) * PITCH + c] << 16);
     }
     // blocks along rows, from registers (the global stores overlap the LDS latency above).  The transposed payload
-    // is streamed out while the input fits the 256 MB last-level cache (measured 54.7 -> 49.6 us at 8192^2); beyond
-    // that everything streams anyway and plain stores are faster (215 against 229 us at 16384 x 14336).
-    const bool nt = streams_out(rows * cols) && rows * cols <= ((int64_t)128 << 20);
+    // is streamed out while the input fits the 256 MB last-level cache (measured 49.5 -> 44.9 us at 8192^2); beyond
+    // that everything streams anyway and plain stores are faster.  6-bit codes keep plain stores: a tile's part of
+    // a column is 96 bytes, three quarters of a memory line, and streamed parts reach memory before the neighbouring
+    // tile's part joins them (8192^2: 49.4 us streamed, 47.3 plain; 16384 x 14336: 265 against 201 us).
+    const bool nt = Wire<F>::bits == 8 && streams_out(rows * cols) && rows * cols <= ((int64_t)128 << 20);
     const bool dword_row_scales = (cols & 127) == 0;
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
