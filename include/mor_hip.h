@@ -127,7 +127,9 @@ MOR_API int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t
 /*
  * Exhaustive on-device comparison of the gfx950 FP8 convert instructions with the software
  * cast over all 2^32 fp32 inputs whose magnitude does not exceed the format maximum.
- * mismatches[0] = E4M3 count, mismatches[1] = E5M2 count (device pointer, 2 x uint64).
+ * mismatches[0] = E4M3 count, mismatches[1] = E5M2 count, mismatches[2] = count of inputs for which
+ * the scaled pair converts (codes of both formats in one register, two values decoded at once)
+ * differ from the plain converts (device pointer, 3 x uint64).
  */
 MOR_API int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
 

@@ -143,6 +143,29 @@ template <int F, int BYTE> __device__ __forceinline__ float hw_unpack(uint32_t p
     else return __builtin_amdgcn_cvt_f32_bf8((int)p, BYTE);
 }
 
+// gfx950 scaled converts on fp32 pairs: both fp8 codes of a pair of values in one register, E4M3 codes of (a, b) in
+// the low word and E5M2 codes of (128 a, 128 b) in the high word (the scale operand of the convert divides by 2^-7),
+// and both values of a word decoded by one instruction.  mor_selftest_hw_cast compares them with the plain converts
+// over every fp32 value in range.
+typedef short s16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t hw_pack2_both(float a, float b, uint32_t old) {
+    s16x2 p = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(__builtin_bit_cast(s16x2, old), a, b, 1.0f, false);
+    p = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(p, a, b, 0x1p-7f, true);
+    return __builtin_bit_cast(uint32_t, p);
+}
+__device__ __forceinline__ f32x2 hw_unpack2_e4m3_low(uint32_t p) { return __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(p, 1.0f, false); }
+__device__ __forceinline__ f32x2 hw_unpack2_e5m2_high_div128(uint32_t p) { return __builtin_amdgcn_cvt_scalef32_pk_f32_bf8(p, 0x1p-7f, true); }
+template <int F> __device__ __forceinline__ uint32_t hw_pack2_low(float a, float b) {
+    const s16x2 z = {0, 0};
+    if constexpr (F == FMT_E4M3) return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(z, a, b, 1.0f, false));
+    else return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(z, a, b, 1.0f, false));
+}
+template <int F> __device__ __forceinline__ f32x2 hw_unpack2_low(uint32_t p) {
+    if constexpr (F == FMT_E4M3) return __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(p, 1.0f, false);
+    else return __builtin_amdgcn_cvt_scalef32_pk_f32_bf8(p, 1.0f, false);
+}
+
 // ---------------------------------------------------------------- scale-quantize-dequantize-descale
 // FQ:248-306 with E8_RZ: the power of two is taken from the exponent field of the fp32 scale and
 // added to / subtracted from exponent fields, clamping at 0 and keeping the mantissa.
@@ -324,6 +347,15 @@ template <int GT> __device__ __forceinline__ float group_max_t(float v, int G) {
         return v;
     }
 }
+__device__ __forceinline__ uint32_t group_umax(uint32_t v, int G) {
+    if (G >= 2) v = max(v, dpp_u<DPP_XOR1>(v));
+    if (G >= 4) v = max(v, dpp_u<DPP_XOR2>(v));
+    if (G >= 8) v = max(v, dpp_u<DPP_HALF_MIRROR>(v));
+    if (G >= 16) v = max(v, dpp_u<DPP_MIRROR>(v));
+    if (G >= 32) v = max(v, (uint32_t)__shfl_xor((int)v, 16));
+    if (G >= 64) v = max(v, (uint32_t)__shfl_xor((int)v, 32));
+    return v;
+}
 __device__ __forceinline__ uint32_t group_umin(uint32_t v, int G) {
     if (G >= 2) v = min(v, dpp_u<DPP_XOR1>(v));
     if (G >= 4) v = min(v, dpp_u<DPP_XOR2>(v));
@@ -363,6 +395,31 @@ __device__ __forceinline__ void acc_amin(uint32_t& amin_m1, uint32_t w) {
     amin_m1 = min(min(amin_m1, a), b);
 }
 constexpr uint32_t AMIN_INIT_M1 = 0x7F7F0000u - 1u;   // bf16 max, FQ:409-412
+
+// The same on both halves of a word at once with packed 16-bit integer instructions: bf16 magnitudes order as their
+// bit patterns do.  amax2 holds two running maxima of magnitudes, amin2_m1 two running minima of (magnitude - 1),
+// where zero wraps to 0xFFFF and so never wins.  A NaN (magnitude above 0x7F80) would win the maximum, which the
+// float maximum of the reference (FQ:430) does not allow: callers send such blocks to the exact path.
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
+__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
+__device__ __forceinline__ uint32_t pk_sub_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, a) - __builtin_bit_cast(u16x2, b));
+}
+__device__ __forceinline__ void acc_amax_pk(uint32_t& amax2, uint32_t w) { amax2 = pk_max_u16(amax2, w & 0x7FFF7FFFu); }
+__device__ __forceinline__ void acc_amin_pk(uint32_t& amin2_m1, uint32_t w) {
+    amin2_m1 = pk_min_u16(amin2_m1, pk_sub_u16(w & 0x7FFF7FFFu, 0x00010001u));
+}
+constexpr uint32_t AMIN2_INIT_M1 = 0x7F7E7F7Eu;
+// fp32 bit pattern of the larger half / (magnitude - 1) of the smaller half in the 32-bit form acc_amin keeps
+__device__ __forceinline__ uint32_t amax_bits_of(uint32_t amax2) { return max(amax2 << 16, amax2 & 0xFFFF0000u); }
+__device__ __forceinline__ uint32_t amin_m1_of(uint32_t amin2_m1) { return (min(amin2_m1 & 0xFFFFu, amin2_m1 >> 16) << 16) | 0xFFFFu; }
+// keeps the compiler from carrying unpacked copies of a data register from one pass over the block to the next
+__device__ __forceinline__ void opaque(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
 
 
 // ---------------------------------------------------------------- gfx950 block converts (32 values per lane)

@@ -107,10 +107,8 @@ __device__ __forceinline__ void err_terms_exact(float x, bool e8, const Scale& s
 // ------------------------------------------------------------------------------------------------
 // quantize one packed word with an fp32 scale: |x| * s, hardware convert, divide by s, round-half-up store, sign
 template <int F> __device__ __forceinline__ uint32_t fq_pair_div(uint32_t w, float s, float r) {
-    const uint32_t p = hw_pack2<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s);
-    const float q0 = div_by_scale(hw_unpack<F, 0>(p), s, r);
-    const float q1 = div_by_scale(hw_unpack<F, 1>(p), s, r);
-    return store_pair<false>(q0, q1) | (w & 0x80008000u);
+    const f32x2 c = hw_unpack2_low<F>(hw_pack2_low<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s));
+    return store_pair<false>(div_by_scale(c.x, s, r), div_by_scale(c.y, s, r)) | (w & 0x80008000u);
 }
 template <int F> __device__ __forceinline__ uint4 fq_vec_div(uint4 v, float s, float r) {
     uint4 o;
@@ -129,8 +127,9 @@ template <int F> __device__ __forceinline__ uint4 fq_vec_div(uint4 v, float s, f
 // depend on less than 1e-5 are recomputed with the reference's divisions by the caller.  The sums are only wanted
 // for blocks with amax / min non-zero |x| <= 939524096 (FQ:637), so a non-zero element scales to at least
 // 448 / 939524096 and no reciprocal overflows.
+// `codes` carries the register of the fp8 codes from one word to the next (the converts write half of it).
 template <bool E8>
-__device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float& e4, float& e5) {
+__device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float& e4, float& e5, uint32_t& codes) {
     float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
     if constexpr (E8) {
         const int e84 = s4.e8, e85 = s4.e8 + 7;
@@ -147,16 +146,16 @@ __device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float
         e4 = fmaf(fabsf(qb4 - b), yb, e4);
         e5 = fmaf(fabsf(qb5 - b), yb, e5);
     } else {
-        const float va = a * s4.s, vb = b * s4.s;
-        const uint32_t p4 = hw_pack2<FMT_E4M3>(va, vb);
-        const uint32_t p5 = hw_pack2<FMT_E5M2>(va * 128.0f, vb * 128.0f);
-        // a zero element has c = y = 0: its term is 0 * rcp(2^-100) = 0 without a select
-        const float ya = __builtin_amdgcn_rcpf(fmaxf(va, 0x1p-100f));
-        const float yb = __builtin_amdgcn_rcpf(fmaxf(vb, 0x1p-100f));
-        e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 0>(p4) - va), ya, e4);
-        e5 = fmaf(fabsf(fmaf(hw_unpack<FMT_E5M2, 0>(p5), 0.0078125f, -va)), ya, e5);
-        e4 = fmaf(fabsf(hw_unpack<FMT_E4M3, 1>(p4) - vb), yb, e4);
-        e5 = fmaf(fabsf(fmaf(hw_unpack<FMT_E5M2, 1>(p5), 0.0078125f, -vb)), yb, e5);
+        // y + 2^-100 is y for every non-zero element of such a block and keeps the reciprocal of a zero element
+        // finite: its codes are 0 and c - x s = 0 (one fma, x s not rounded), so its term is 0 without a select
+        const float va = fmaf(a, s4.s, 0x1p-100f), vb = fmaf(b, s4.s, 0x1p-100f);
+        codes = hw_pack2_both(va, vb, codes);
+        const f32x2 c4 = hw_unpack2_e4m3_low(codes), c5 = hw_unpack2_e5m2_high_div128(codes);
+        const float ya = __builtin_amdgcn_rcpf(va), yb = __builtin_amdgcn_rcpf(vb);
+        e4 = fmaf(fabsf(fmaf(-a, s4.s, c4.x)), ya, e4);
+        e5 = fmaf(fabsf(fmaf(-a, s4.s, c5.x)), ya, e5);
+        e4 = fmaf(fabsf(fmaf(-b, s4.s, c4.y)), yb, e4);
+        e5 = fmaf(fabsf(fmaf(-b, s4.s, c5.y)), yb, e5);
     }
 }
 
@@ -237,8 +236,9 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
             bool exact = true;
             if constexpr (FAST && !EMU) {
                 if (allow_fast && s4.fast && s4.e8 >= -90 && s4.e8 <= 90) {
-                    if (e8) for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<true>((uint32_t)bin[at], s4, e4, e5); });
-                    else for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<false>((uint32_t)bin[at], s4, e4, e5); });
+                    uint32_t codes = 0;
+                    if (e8) for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<true>((uint32_t)bin[at], s4, e4, e5, codes); });
+                    else for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<false>((uint32_t)bin[at], s4, e4, e5, codes); });
                     e4 = wave_sum(e4);
                     e5 = wave_sum(e5);
                     __syncthreads();
@@ -492,25 +492,29 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
     }
 
     // pass 1 (registers): amax and min over non-zero magnitudes, FQ:407-485
-    float amax = 0.0f;
-    uint32_t amin_m1 = AMIN_INIT_M1;
+    // (packed 16-bit integer maxima / minima of both halves of a word; the data stays packed in its registers)
+    uint32_t amax2 = 0, amin2_m1 = AMIN2_INIT_M1;
 #pragma unroll
     for (int k = 0; k < NV; ++k)
         if (ok[k]) {
-            acc_amax(amax, v[k].x); acc_amax(amax, v[k].y); acc_amax(amax, v[k].z); acc_amax(amax, v[k].w);
-            if constexpr (MOR) { acc_amin(amin_m1, v[k].x); acc_amin(amin_m1, v[k].y); acc_amin(amin_m1, v[k].z); acc_amin(amin_m1, v[k].w); }
+            acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+            if constexpr (MOR) { acc_amin_pk(amin2_m1, v[k].x); acc_amin_pk(amin2_m1, v[k].y); acc_amin_pk(amin2_m1, v[k].z); acc_amin_pk(amin2_m1, v[k].w); }
+            opaque(v[k]);
         }
-    amax = group_max(amax, 64);
-    if constexpr (MOR) amin_m1 = group_umin(amin_m1, 64);
-    if (lane == 0) { s_f[0][wave] = amax; s_u[wave] = amin_m1; }
+    uint32_t amax_b = group_umax(amax_bits_of(amax2), 64);
+    uint32_t amin_m1 = AMIN_INIT_M1;
+    if constexpr (MOR) amin_m1 = group_umin(amin_m1_of(amin2_m1), 64);
+    if (lane == 0) { s_f[0][wave] = u2f(amax_b); s_u[wave] = amin_m1; }
     __syncthreads();
-    amax = fmaxf(fmaxf(s_f[0][0], s_f[0][1]), fmaxf(s_f[0][2], s_f[0][3]));
+    amax_b = max(max(f2u(s_f[0][0]), f2u(s_f[0][1])), max(f2u(s_f[0][2]), f2u(s_f[0][3])));
     amin_m1 = min(min(s_u[0], s_u[1]), min(s_u[2], s_u[3]));
+    const float amax = u2f(amax_b);
     const float amin = u2f(amin_m1 + 1u);
 
     // scales of the two fp8 formats; the fp6 scales differ from s4 by 2^4 / 2^6, inside the margin of `fast`
     const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
-    if (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast)) {           // uniform over the workgroup
+    // (a NaN in the block shows as amax_b above the bits of infinity: the exact path takes its maximum as the reference does)
+    if (amax_b > 0x7F800000u || (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast))) {           // uniform over the workgroup
         generic_block<false>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
                              sh, qa, E8, bid, s_f, s_u);
         return;
@@ -524,14 +528,17 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
         if (qt == Q_UNKNOWN) {
             // pass 2 (registers): the two error sums, FQ:487-584.  amax > 0 here.
             __syncthreads();                     // s_f[0] has been read by every wave
+            uint32_t codes = 0;
 #pragma unroll
             for (int k = 0; k < NV; ++k)
                 if (ok[k]) {
-                    err_pair_fast<E8>(v[k].x, s4, e4, e5);
-                    err_pair_fast<E8>(v[k].y, s4, e4, e5);
-                    err_pair_fast<E8>(v[k].z, s4, e4, e5);
-                    err_pair_fast<E8>(v[k].w, s4, e4, e5);
+                    err_pair_fast<E8>(v[k].x, s4, e4, e5, codes);
+                    err_pair_fast<E8>(v[k].y, s4, e4, e5, codes);
+                    err_pair_fast<E8>(v[k].z, s4, e4, e5, codes);
+                    err_pair_fast<E8>(v[k].w, s4, e4, e5, codes);
                 }
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) opaque(v[k]);
             e4 = wave_sum(e4);
             e5 = wave_sum(e5);
             if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
@@ -643,7 +650,7 @@ __global__ __launch_bounds__(WG) void k_block_stats(const uint16_t* __restrict__
 // ------------------------------------------------------------------------------------------------
 // Exhaustive check of the hardware converts against the software model, in range.
 __global__ __launch_bounds__(WG) void k_selftest_hw_cast(unsigned long long* mism) {
-    unsigned long long bad4 = 0, bad5 = 0;
+    unsigned long long bad4 = 0, bad5 = 0, bad_scaled = 0;
     const uint64_t stride = (uint64_t)gridDim.x * WG;
     for (uint64_t i = (uint64_t)blockIdx.x * WG + threadIdx.x; i < (1ull << 32); i += stride) {
         float v = u2f((uint32_t)i);
@@ -656,9 +663,30 @@ __global__ __launch_bounds__(WG) void k_selftest_hw_cast(unsigned long long* mis
             uint32_t hw = f2u(hw_unpack<FMT_E5M2, 1>(hw_pack2<FMT_E5M2>(0.0f, v)));
             bad5 += (hw != f2u(cast_hwmodel_exact<FMT_E5M2>(v)));
         }
+        // the scaled converts against the plain ones: codes and decoded values, both lanes of the pair
+        if (a <= 448.0f) {
+            const float o = u2f((uint32_t)i ^ 0x00400000u);              // the other value of the pair (same exponent)
+            const uint32_t both = hw_pack2_both(v, o, 0xA5A5A5A5u);
+            const uint32_t p4 = hw_pack2<FMT_E4M3>(v, o), p5 = hw_pack2<FMT_E5M2>(v * 128.0f, o * 128.0f);
+            const f32x2 c4 = hw_unpack2_e4m3_low(both), c5 = hw_unpack2_e5m2_high_div128(both);
+            bool ok = ((both & 0xFFFFu) == (p4 & 0xFFFFu)) && ((both >> 16) == (p5 & 0xFFFFu));
+            ok = ok && f2u(c4.x) == f2u(hw_unpack<FMT_E4M3, 0>(p4)) && f2u(c4.y) == f2u(hw_unpack<FMT_E4M3, 1>(p4));
+            ok = ok && f2u(c5.x) == f2u(hw_unpack<FMT_E5M2, 0>(p5) * 0.0078125f) && f2u(c5.y) == f2u(hw_unpack<FMT_E5M2, 1>(p5) * 0.0078125f);
+            const uint32_t l4 = hw_pack2_low<FMT_E4M3>(v, o);
+            const f32x2 d4 = hw_unpack2_low<FMT_E4M3>(l4);
+            ok = ok && ((l4 & 0xFFFFu) == (p4 & 0xFFFFu)) && f2u(d4.x) == f2u(c4.x) && f2u(d4.y) == f2u(c4.y);
+            bad_scaled += !ok;
+        }
+        if (a <= 57344.0f) {
+            const float o = u2f((uint32_t)i ^ 0x00400000u);
+            const uint32_t p5 = hw_pack2<FMT_E5M2>(v, o), l5 = hw_pack2_low<FMT_E5M2>(v, o);
+            const f32x2 d5 = hw_unpack2_low<FMT_E5M2>(l5);
+            bad_scaled += !(((l5 & 0xFFFFu) == (p5 & 0xFFFFu)) && f2u(d5.x) == f2u(hw_unpack<FMT_E5M2, 0>(p5)) && f2u(d5.y) == f2u(hw_unpack<FMT_E5M2, 1>(p5)));
+        }
     }
     if (bad4) atomicAdd(&mism[0], bad4);
     if (bad5) atomicAdd(&mism[1], bad5);
+    if (bad_scaled) atomicAdd(&mism[2], bad_scaled);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -797,7 +825,12 @@ static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, i
     // Tensors whose traffic exceeds twice the 256 MB last-level cache stream their loads as well.
     const int64_t out_bytes = sh.rows * sh.cols * 2;
     const int ntm = (2 * out_bytes > ((int64_t)512 << 20)) ? 1 : (out_bytes >= ((int64_t)4 << 20)) ? 2 : 0;
-#define MOR_WGBLOCK(FULL, NT) k_wgblock<MOR, E8, NV, FULL, NT><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift)
+    // Large grids run 3 workgroups per CU (unused dynamic LDS caps the occupancy the registers would allow at 5):
+    // fewer tiles in flight keep the memory system on fewer DRAM pages at a time (16384 x 14336 MoR: 176.8 -> 170.8 us,
+    // 8192^2 block E4M3: 41.4 -> 40.1 us), while a grid that fits the chip at once wants every slot (4096^2: 9.2
+    // against 10.8 us).
+    const size_t dyn_lds = (NV == 8 && grid >= 4096) ? 53000 : 0;
+#define MOR_WGBLOCK(FULL, NT) k_wgblock<MOR, E8, NV, FULL, NT><<<grid, WG, dyn_lds, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift)
     if (full) {
         if (ntm == 1) MOR_WGBLOCK(true, 1); else if (ntm == 2) MOR_WGBLOCK(true, 2); else MOR_WGBLOCK(true, 0);
     } else {
@@ -967,7 +1000,7 @@ extern "C" int mor_e4m3_with_e8_scale(const float* input, float* output, int64_t
 extern "C" int mor_selftest_hw_cast(uint64_t* mismatches, void* stream) {
     if (!mismatches) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mismatches is NULL");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    k_fill_i32<<<1, WG, 0, st>>>(reinterpret_cast<int32_t*>(mismatches), 4, 0);
+    k_fill_i32<<<1, WG, 0, st>>>(reinterpret_cast<int32_t*>(mismatches), 6, 0);
     k_selftest_hw_cast<<<256 * 16, WG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
     return mor_check_launch("k_selftest_hw_cast");
 }
