@@ -339,8 +339,13 @@ def c5_sweep(torch, run, K, W):
     cache = {}
 
     def timed(key, fn):
+        # short kernels are timed over about 3 ms of back-to-back launches: a burst of a few hundred microseconds
+        # ends before the clocks have left their idle state
         if key not in cache:
-            cache[key] = time_launches(torch, fn, K, W)[0]
+            ms = time_launches(torch, fn, K, W)[0]
+            if ms * K < 3.0:
+                ms = time_launches(torch, fn, min(400, int(3.0 / ms) + 1), W)[0]
+            cache[key] = ms
         return cache[key]
 
     def view(src, r, c):

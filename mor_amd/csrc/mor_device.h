@@ -275,9 +275,8 @@ template <int F, bool CLAMP> __device__ __forceinline__ uint32_t fp32_pair_fast(
             v0 = fminf(v0, Fmt<F>::fmax);
             v1 = fminf(v1, Fmt<F>::fmax);
         }
-        const uint32_t p = hw_pack2<F>(v0, v1);
-        const float q0 = div_by_scale(hw_unpack<F, 0>(p), s, r), q1 = div_by_scale(hw_unpack<F, 1>(p), s, r);
-        return store_pair<false>(q0, q1) | (w & 0x80008000u);
+        const f32x2 c = hw_unpack2_low<F>(hw_pack2_low<F>(v0, v1));
+        return store_pair<false>(div_by_scale(c.x, s, r), div_by_scale(c.y, s, r)) | (w & 0x80008000u);
     } else {
         const float d0 = cast_sw_exact<F>(a), d1 = cast_sw_exact<F>(b);
         const uint32_t sign = ((d0 != 0.0f) ? (w & 0x8000u) : 0u) | ((d1 != 0.0f) ? (w & 0x80000000u) : 0u);

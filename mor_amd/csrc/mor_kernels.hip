@@ -1298,8 +1298,8 @@ __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, fl
         qa = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p)) - e8s, 0));
         qb = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p)) - e8s, 0));
     } else {
-        uint32_t p = hw_pack2<FMT_E4M3>(a * sc.s, b * sc.s);
-        float ca = hw_unpack<FMT_E4M3, 0>(p), cb = hw_unpack<FMT_E4M3, 1>(p);
+        const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc.s, b * sc.s));
+        const float ca = c.x, cb = c.y;
         float ta = ca * rs, tb = cb * rs;
         qa = fmaf(fmaf(-ta, sc.s, ca), rs, ta);
         qb = fmaf(fmaf(-tb, sc.s, cb), rs, tb);
