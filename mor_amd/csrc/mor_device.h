@@ -414,6 +414,10 @@ __device__ __forceinline__ void acc_amin_pk(uint32_t& amin2_m1, uint32_t w) {
     amin2_m1 = pk_min_u16(amin2_m1, pk_sub_u16(w & 0x7FFF7FFFu, 0x00010001u));
 }
 constexpr uint32_t AMIN2_INIT_M1 = 0x7F7E7F7Eu;
+// two running counts of non-zero magnitudes (each half adds 1 when its magnitude is not 0); at most 65535 words per lane
+__device__ __forceinline__ void acc_nnz_pk(uint32_t& nnz2, uint32_t w) {
+    nnz2 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, nnz2) + __builtin_bit_cast(u16x2, pk_min_u16(w & 0x7FFF7FFFu, 0x00010001u)));
+}
 // fp32 bit pattern of the larger half / (magnitude - 1) of the smaller half in the 32-bit form acc_amin keeps
 __device__ __forceinline__ uint32_t amax_bits_of(uint32_t amax2) { return max(amax2 << 16, amax2 & 0xFFFF0000u); }
 __device__ __forceinline__ uint32_t amin_m1_of(uint32_t amin2_m1) { return (min(amin2_m1 & 0xFFFFu, amin2_m1 >> 16) << 16) | 0xFFFFu; }

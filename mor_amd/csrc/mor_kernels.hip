@@ -1288,31 +1288,30 @@ __device__ __forceinline__ float bs_element(float x, const Scale& sc, float& err
 // Fast version on magnitudes for scales in the fast range: hardware convert; q = c / s by a reciprocal-multiply
 // with one exact-residual correction (r = 1 / s correctly rounded, the result is then the rounded quotient);
 // error term |q - x| / x through the hardware reciprocal (relative 1e-7, tolerance on the sum 1e-6).
+// No selects: a zero element has q = 0, so its term is 0 * min(1 / 0, FLT_MAX) = 0 and its magnitude bits are 0;
+// the sign of the input is kept for non-zero halves only (zero inputs come back as +0, FQ:1133-1134), through a
+// packed 16-bit mask.
 template <bool E8>
 __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, float rs, float& err) {
-    float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
+    const float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
     float qa, qb;
     if constexpr (E8) {
         const int e8s = sc.e8 << 23;
         uint32_t p = hw_pack2<FMT_E4M3>(ldexpf(a, sc.e8), ldexpf(b, sc.e8));
         qa = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p)) - e8s, 0));
         qb = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p)) - e8s, 0));
+        qa = (a == 0.0f) ? 0.0f : qa;                // the exponent arithmetic turns a zero code into 2^-e8 (e8 < 0), and
+        qb = (b == 0.0f) ? 0.0f : qb;                // zero inputs are skipped by the reference (FQ:1133)
     } else {
         const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc.s, b * sc.s));
-        const float ca = c.x, cb = c.y;
-        float ta = ca * rs, tb = cb * rs;
-        qa = fmaf(fmaf(-ta, sc.s, ca), rs, ta);
-        qb = fmaf(fmaf(-tb, sc.s, cb), rs, tb);
+        qa = div_by_scale(c.x, sc.s, rs);
+        qb = div_by_scale(c.y, sc.s, rs);
     }
-    const bool za = (a == 0.0f), zb = (b == 0.0f);
-    float ya = za ? 0.0f : __builtin_amdgcn_rcpf(a);
-    float yb = zb ? 0.0f : __builtin_amdgcn_rcpf(b);
+    const float ya = fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), yb = fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f);
     err = fmaf(fabsf(qa - a), ya, err);
     err = fmaf(fabsf(qb - b), yb, err);
-    // zero inputs come back as +0 (FQ:1133-1134); everything else keeps the input's sign
-    uint32_t lo = za ? 0u : ((rhu_bits(qa) >> 16) | (w & 0x8000u));
-    uint32_t hi = zb ? 0u : ((rhu_bits(qb) & 0xFFFF0000u) | (w & 0x80000000u));
-    return lo | hi;
+    const uint32_t nonzero = pk_min_u16(w & 0x7FFF7FFFu, 0x00010001u);        // 1 in each half that is not +-0
+    return store_pair<false>(qa, qb) | (w & (nonzero << 15));
 }
 
 // pass 2 / pass 4: quantize every element with its block's scale (looked up per chunk, or per column in column
@@ -1527,44 +1526,83 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
     const uint32_t row_stride = (uint32_t)(sh.cols >> 3);
     const int nch = (int)sh.brows * cpr;
     const bool nt = streams_out(sh.rows * sh.cols);
+    // chunk k * 256 + tid of a block is at off_k(k) + off_tid; cpr is a power of two, so off_k is uniform (no per-lane
+    // index arithmetic is carried through the loop over blocks)
+    const uint32_t off_tid = cpr_shift <= 8 ? (uint32_t)(tid >> cpr_shift) * row_stride + (uint32_t)(tid & (cpr - 1)) : (uint32_t)tid;
+    auto off_k = [&](int k) -> uint32_t {
+        return cpr_shift <= 8 ? (uint32_t)(k << (8 - cpr_shift)) * row_stride
+                              : (uint32_t)(k >> (cpr_shift - 8)) * row_stride + (uint32_t)((k & ((1 << (cpr_shift - 8)) - 1)) << 8);
+    };
     float gmax = 0.0f, err = 0.0f;
     int nnz_total = 0;
     for (int64_t bid = blockIdx.x; bid < nblocks; bid += gridDim.x) {
         const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
         const int64_t base = by * sh.brows * row_stride + ((bx * sh.bcols) >> 3);
         uint4 v[NV];
-        uint32_t off[NV];
         bool ok[NV];
-        float amax = 0.0f;
-        int nnz = 0;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            const int ch = k * WG + tid;
-            const int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
-            ok[k] = FULL || (ch < nch);
-            off[k] = (uint32_t)r * row_stride + (uint32_t)(ch - r * cpr);
+            ok[k] = FULL || (k * WG + tid < nch);
             v[k] = make_uint4(0, 0, 0, 0);
-            if (ok[k]) v[k] = in[base + off[k]];
+            if (ok[k]) v[k] = in[base + off_k(k) + off_tid];
         }
+        // amax and the non-zero count.  Large blocks: on packed 16-bit magnitudes, the data staying packed in its
+        // registers from pass to pass (NV = 8: 100 registers instead of 220).  Small blocks: float maxima, whose
+        // unpacked magnitudes the quantize pass then uses again (measured faster for NV <= 2).
+        constexpr bool PACKED = NV > 2;
+        uint32_t amax_b, nnz2 = 0;
+        if constexpr (PACKED) {
+            uint32_t amax2 = 0;
 #pragma unroll
-        for (int k = 0; k < NV; ++k) acc_amax_nnz(amax, nnz, v[k]);
-        amax = group_max(amax, 64);
+            for (int k = 0; k < NV; ++k) {
+                acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+                acc_nnz_pk(nnz2, v[k].x); acc_nnz_pk(nnz2, v[k].y); acc_nnz_pk(nnz2, v[k].z); acc_nnz_pk(nnz2, v[k].w);
+                opaque(v[k]);
+            }
+            amax_b = group_umax(amax_bits_of(amax2), 64);
+        } else {
+            float amaxf = 0.0f;
+            int nnzf = 0;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) acc_amax_nnz(amaxf, nnzf, v[k]);
+            nnz2 = (uint32_t)nnzf;
+            amax_b = f2u(group_max(amaxf, 64));
+        }
         __syncthreads();                          // the previous block's readers of s_f are done
-        if (lane == 0) s_f[wave] = amax;
+        if (lane == 0) s_f[wave] = u2f(amax_b);
         __syncthreads();
-        amax = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        amax_b = max(max(f2u(s_f[0]), f2u(s_f[1])), max(f2u(s_f[2]), f2u(s_f[3])));
+        float amax = u2f(amax_b);
+        if (amax_b > 0x7F800000u) {               // a NaN in the block: the float maximum of the reference skips it (rare)
+            amax = 0.0f;
+#pragma unroll 1
+            for (int ch = tid; ch < nch; ch += WG) {              // from memory again: no second use of the registers
+                const int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
+                const uint4 x = in[base + (uint32_t)r * row_stride + (uint32_t)(ch - r * cpr)];
+                acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
+            }
+            amax = group_max(amax, 64);
+            __syncthreads();
+            if (lane == 0) s_f[wave] = amax;
+            __syncthreads();
+            amax = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        }
         gmax = fmaxf(gmax, amax);
-        nnz_total += nnz;
+        nnz_total += (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
         const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
         if (sc.fast || !(amax > 0.0f)) {          // an all-zero block gives +0 whatever its (clamped) scale is
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
+                if constexpr (PACKED) opaque(v[k]);   // one vector at a time: work hoisted from all of them doubles the registers
                 uint4 q;
                 q.x = bs_pair_fast<E8>(v[k].x, sc, sc.r, err);
                 q.y = bs_pair_fast<E8>(v[k].y, sc, sc.r, err);
                 q.z = bs_pair_fast<E8>(v[k].z, sc, sc.r, err);
                 q.w = bs_pair_fast<E8>(v[k].w, sc, sc.r, err);
-                if (ok[k] && write) store16_rt(out + base + off[k], q, nt);
+                // this vector's results and error terms are finished here: not once in each branch of the store, and
+                // not, with all the magnitudes and quotients alive, after the last store
+                if constexpr (PACKED) { opaque(q); asm volatile("" : "+v"(err)); }
+                if (ok[k] && write) store16_rt(out + base + off_k(k) + off_tid, q, nt);
             }
         } else {
             const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in);
@@ -1842,10 +1880,10 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
     // block-local scales: one pass out of place; in place one pass for the decision and one gated pass that writes
     const int64_t blk_chunks = (bcols % 8 == 0) ? brows * (bcols / 8) : 0;
     // (in place, large blocks are faster through the general three-pass path: measured 109 against 102 us)
-    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG / 2 && blk_chunks <= (inplace ? 2 : 8) * WG
-        && brows * (cols / 8) < 0x7FFFFFFFll) {
+    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG && blk_chunks <= (inplace ? 2 : 8) * WG
+        && brows * (cols / 8) < 0x7FFFFFFFll && is_pow2(bcols / 8)) {
         const int cpr = (int)(bcols / 8);
-        const int shift = is_pow2(cpr) ? ilog2(cpr) : -1;
+        const int shift = ilog2(cpr);
         const int nv = (int)cdiv(blk_chunks, WG);
         const int NVc = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
         const bool full = blk_chunks == (int64_t)NVc * WG;
