@@ -1479,20 +1479,41 @@ __global__ __launch_bounds__(WG) void k_bs_finalize(const uint32_t* ws, int npar
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float gamax = u2f(ws[0]);
     int gnnz = (int)ws[1];
-    if (npart_stats > 0) {
-        gamax = reduce_partial_amax(ws, npart_stats, s_f);
+    float acc = 0.0f;
+    if (npart_stats > 0 && npart_stats == npartials) {
+        // the three partial arrays in one sweep, all loads of a batch in flight (three sweeps in a row were 6.4 us
+        // of one workgroup's load latency); every sum keeps the order of the separate sweeps
+        const float* pa = reinterpret_cast<const float*>(ws) + WS_PAMAX;
         const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
+        float a = 0.0f;
         int n = 0;
 #pragma unroll 8
-        for (int i = threadIdx.x; i < npart_stats; i += WG) n += pn[i];
+        for (int i = threadIdx.x; i < npartials; i += WG) {
+            a = fmaxf(a, pa[i]);
+            n += pn[i];
+            acc += part[i];
+        }
+        a = group_max(a, 64);
         n = wave_sum_i(n);
-        if (lane == 0) s_i[wave] = n;
+        if (lane == 0) { s_f[wave] = a; s_i[wave] = n; }
         __syncthreads();
+        gamax = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
         gnnz = s_i[0] + s_i[1] + s_i[2] + s_i[3];
-    }
-    float acc = 0.0f;
+    } else {
+        if (npart_stats > 0) {
+            gamax = reduce_partial_amax(ws, npart_stats, s_f);
+            const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
+            int n = 0;
 #pragma unroll 8
-    for (int i = threadIdx.x; i < npartials; i += WG) acc += part[i];
+            for (int i = threadIdx.x; i < npart_stats; i += WG) n += pn[i];
+            n = wave_sum_i(n);
+            if (lane == 0) s_i[wave] = n;
+            __syncthreads();
+            gnnz = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+        }
+#pragma unroll 8
+        for (int i = threadIdx.x; i < npartials; i += WG) acc += part[i];
+    }
     acc = wave_sum(acc);
     __syncthreads();
     if (lane == 0) s_f[wave] = acc;
@@ -1887,7 +1908,7 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
         const int nv = (int)cdiv(blk_chunks, WG);
         const int NVc = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
         const bool full = blk_chunks == (int64_t)NVc * WG;
-        const int grid = (int)std::min<int64_t>(nb, MAX_PARTIALS);
+        const int grid = (int)std::min<int64_t>(nb, 4096);      // partials: one per workgroup (the finalize kernel reads them all)
         const uint4* i4 = static_cast<const uint4*>(input);
         uint4* o4 = static_cast<uint4*>(output);
 #define MOR_BS_FUSED(E8, NV, PHASE) do { \
@@ -1901,7 +1922,7 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
         if (inplace) MOR_BS_FUSED_ALL(2);
         else {
             const int64_t n_all = rows * cols;
-            k_copy_if<<<grid_for(n_all / 8, 16), WG, 0, st>>>(in16, out16, meta, 3, n_all, n_all / 8);
+            k_copy_if<<<grid_for(n_all / 8, 4), WG, 0, st>>>(in16, out16, meta, 3, n_all, n_all / 8);
         }
 #undef MOR_BS_FUSED_ALL
 #undef MOR_BS_FUSED
@@ -1920,7 +1941,7 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
             else k_bs_fused_rows<false><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, G, (int)ss_mode, meta, phase);
             if (phase != 2) k_bs_finalize<<<1, WG, 0, st>>>(ws, grid, grid, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
         }
-        if (!inplace) k_copy_if<<<grid_for(nchunks, 16), WG, 0, st>>>(in16, out16, meta, 3, rows * cols, nchunks);
+        if (!inplace) k_copy_if<<<grid_for(nchunks, 4), WG, 0, st>>>(in16, out16, meta, 3, rows * cols, nchunks);
         return mor_check_launch("mor_block_scaling (single pass, row blocks)");
     }
 
@@ -1974,7 +1995,7 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
     }
     if (!inplace) {
         const int64_t nvec = vec ? n / 8 : 0;
-        k_copy_if<<<grid_for(nvec > 0 ? nvec : n, 16), WG, 0, st>>>(in16, out16, meta, 3, n, nvec);
+        k_copy_if<<<grid_for(nvec > 0 ? nvec : n, 4), WG, 0, st>>>(in16, out16, meta, 3, n, nvec);
     }
     return mor_check_launch("mor_block_scaling");
 }
