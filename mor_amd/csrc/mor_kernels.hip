@@ -1291,7 +1291,8 @@ __device__ __forceinline__ float bs_element(float x, const Scale& sc, float& err
 // No selects: a zero element has q = 0, so its term is 0 * min(1 / 0, FLT_MAX) = 0 and its magnitude bits are 0;
 // the sign of the input is kept for non-zero halves only (zero inputs come back as +0, FQ:1133-1134), through a
 // packed 16-bit mask.
-template <bool E8>
+// ERR / OUT: whether the error terms / the output word are wanted (the in-place phases need one of them each).
+template <bool E8, bool ERR = true, bool OUT = true>
 __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, float rs, float& err) {
     const float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
     float qa, qb;
@@ -1307,11 +1308,23 @@ __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, fl
         qa = div_by_scale(c.x, sc.s, rs);
         qb = div_by_scale(c.y, sc.s, rs);
     }
-    const float ya = fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), yb = fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f);
-    err = fmaf(fabsf(qa - a), ya, err);
-    err = fmaf(fabsf(qb - b), yb, err);
+    if constexpr (ERR) {
+        const float ya = fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), yb = fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f);
+        err = fmaf(fabsf(qa - a), ya, err);
+        err = fmaf(fabsf(qb - b), yb, err);
+    }
+    if constexpr (!OUT) return 0u;
     const uint32_t nonzero = pk_min_u16(w & 0x7FFF7FFFu, 0x00010001u);        // 1 in each half that is not +-0
     return store_pair<false>(qa, qb) | (w & (nonzero << 15));
+}
+template <bool E8, bool ERR, bool OUT>
+__device__ __forceinline__ uint4 bs_vec_fast(uint4 v, const Scale& sc, float& err) {
+    uint4 q;
+    q.x = bs_pair_fast<E8, ERR, OUT>(v.x, sc, sc.r, err);
+    q.y = bs_pair_fast<E8, ERR, OUT>(v.y, sc, sc.r, err);
+    q.z = bs_pair_fast<E8, ERR, OUT>(v.z, sc, sc.r, err);
+    q.w = bs_pair_fast<E8, ERR, OUT>(v.w, sc, sc.r, err);
+    return q;
 }
 
 // pass 2 / pass 4: quantize every element with its block's scale (looked up per chunk, or per column in column
@@ -1349,7 +1362,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
                 if (!EMU && sc.fast) {
                     const float rs = 1.0f / sc.s;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) w[j] = bs_pair_fast<E8>(w[j], sc, rs, err);
+                    for (int j = 0; j < 4; ++j) w[j] = bs_pair_fast<E8, ERR, WRITE>(w[j], sc, rs, err);
                 } else {
 #pragma unroll 1
                     for (int j = 0; j < 4; ++j) {
@@ -1612,18 +1625,32 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
         nnz_total += (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
         const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
         if (sc.fast || !(amax > 0.0f)) {          // an all-zero block gives +0 whatever its (clamped) scale is
+            // For large blocks every vector is finished before the next begins (register barriers): otherwise the
+            // compiler hoists work from all of them, and sinks the whole chain of error terms below the last store
+            // with every magnitude and quotient alive, which doubles the registers.
+            if (phase == 1) {                      // decision pass of the in-place variant: error terms only
 #pragma unroll
-            for (int k = 0; k < NV; ++k) {
-                if constexpr (PACKED) opaque(v[k]);   // one vector at a time: work hoisted from all of them doubles the registers
-                uint4 q;
-                q.x = bs_pair_fast<E8>(v[k].x, sc, sc.r, err);
-                q.y = bs_pair_fast<E8>(v[k].y, sc, sc.r, err);
-                q.z = bs_pair_fast<E8>(v[k].z, sc, sc.r, err);
-                q.w = bs_pair_fast<E8>(v[k].w, sc, sc.r, err);
-                // this vector's results and error terms are finished here: not once in each branch of the store, and
-                // not, with all the magnitudes and quotients alive, after the last store
-                if constexpr (PACKED) { opaque(q); asm volatile("" : "+v"(err)); }
-                if (ok[k] && write) store16_rt(out + base + off_k(k) + off_tid, q, nt);
+                for (int k = 0; k < NV; ++k) {
+                    if constexpr (PACKED) opaque(v[k]);
+                    bs_vec_fast<E8, true, false>(v[k], sc, err);
+                    if constexpr (PACKED) asm volatile("" : "+v"(err));
+                }
+            } else if (phase == 2) {               // write pass of the in-place variant: no error terms
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    if constexpr (PACKED) opaque(v[k]);
+                    uint4 q = bs_vec_fast<E8, false, true>(v[k], sc, err);
+                    if constexpr (PACKED) opaque(q);
+                    if (ok[k]) store16_rt(out + base + off_k(k) + off_tid, q, nt);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    if constexpr (PACKED) opaque(v[k]);
+                    uint4 q = bs_vec_fast<E8, true, true>(v[k], sc, err);
+                    if constexpr (PACKED) { opaque(q); asm volatile("" : "+v"(err)); }
+                    if (ok[k]) store16_rt(out + base + off_k(k) + off_tid, q, nt);
+                }
             }
         } else {
             const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in);
@@ -1690,10 +1717,9 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
             const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
             float e = 0.0f;
             uint4 q;
-            q.x = bs_pair_fast<E8>(v[k].x, sc, sc.r, e);
-            q.y = bs_pair_fast<E8>(v[k].y, sc, sc.r, e);
-            q.z = bs_pair_fast<E8>(v[k].z, sc, sc.r, e);
-            q.w = bs_pair_fast<E8>(v[k].w, sc, sc.r, e);
+            if (phase == 1) q = bs_vec_fast<E8, true, false>(v[k], sc, e);          // in place: decision pass,
+            else if (phase == 2) q = bs_vec_fast<E8, false, true>(v[k], sc, e);     // write pass
+            else q = bs_vec_fast<E8, true, true>(v[k], sc, e);
             if (sc.fast || !(amax > 0.0f)) {      // an all-zero block gives +0 whatever its (clamped) scale is
                 err += e;
                 if (c < nchunks && write) store16_rt(out + c, q, nt);
@@ -1900,8 +1926,10 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
 
     // block-local scales: one pass out of place; in place one pass for the decision and one gated pass that writes
     const int64_t blk_chunks = (bcols % 8 == 0) ? brows * (bcols / 8) : 0;
-    // (in place, large blocks are faster through the general three-pass path: measured 109 against 102 us)
-    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG && blk_chunks <= (inplace ? 2 : 8) * WG
+    // (a decision pass that computes no output words and a write pass that computes no error terms; 128 x 128 blocks
+    // in place at 8192^2: 83 us against 99 through the general three-pass path; blocks that fill less than a workgroup
+    // take the general path)
+    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG && blk_chunks <= 8 * WG
         && brows * (cols / 8) < 0x7FFFFFFFll && is_pow2(bcols / 8)) {
         const int cpr = (int)(bcols / 8);
         const int shift = ilog2(cpr);
