@@ -421,6 +421,13 @@ __device__ __forceinline__ void acc_nnz_pk(uint32_t& nnz2, uint32_t w) {
 // fp32 bit pattern of the larger half / (magnitude - 1) of the smaller half in the 32-bit form acc_amin keeps
 __device__ __forceinline__ uint32_t amax_bits_of(uint32_t amax2) { return max(amax2 << 16, amax2 & 0xFFFF0000u); }
 __device__ __forceinline__ uint32_t amin_m1_of(uint32_t amin2_m1) { return (min(amin2_m1 & 0xFFFFu, amin2_m1 >> 16) << 16) | 0xFFFFu; }
+// whether one of the 8 values of a vector is a NaN (the fast arithmetic is only exact for finite values; an infinity
+// shows in the block's scale instead)
+__device__ __forceinline__ bool vec_has_nan(uint4 v) {
+    uint32_t m = 0;
+    acc_amax_pk(m, v.x); acc_amax_pk(m, v.y); acc_amax_pk(m, v.z); acc_amax_pk(m, v.w);
+    return amax_bits_of(m) > 0x7F800000u;
+}
 // keeps the compiler from carrying unpacked copies of a data register from one pass over the block to the next
 __device__ __forceinline__ void opaque(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
 

@@ -1044,9 +1044,11 @@ __global__ void k_zero_f32(float* p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) p[i] = 0.0f;
 }
 
+// FQ:998-999: an element counts when |x| > 0 as floats, so a NaN does not
 __device__ __forceinline__ int nnz_word(uint32_t w) {
-    return ((w & 0x7FFFu) != 0) + ((w & 0x7FFF0000u) != 0);
+    return (fabsf(bf16_lo(w)) > 0.0f) + (fabsf(bf16_hi(w)) > 0.0f);
 }
+__device__ __forceinline__ int nan_word(uint32_t w) { return ((w & 0x7FFFu) > 0x7F80u) + ((w & 0x7FFF0000u) > 0x7F800000u); }
 __device__ __forceinline__ void acc_amax_nnz(float& amax, int& nnz, uint4 v) {
     acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
     nnz += nnz_word(v.x) + nnz_word(v.y) + nnz_word(v.z) + nnz_word(v.w);
@@ -1153,7 +1155,7 @@ __global__ __launch_bounds__(WG) void k_bs_amax_block(const uint16_t* in, uint32
                 int64_t r = i / sh.bcols, c = i - r * sh.bcols;
                 uint32_t a = ((uint32_t)in[(r0 + r) * sh.cols + c0 + c] << 16) & 0x7FFFFFFFu;
                 amax = fmaxf(amax, u2f(a));
-                nnz += ((a & 0x7FFF0000u) != 0);
+                nnz += (u2f(a) > 0.0f);
             }
         }
         amax = group_max(amax, 64);
@@ -1359,7 +1361,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
             } else {
                 const uint32_t bx = div_u32(cc, d_bchunks);
                 const Scale sc = make_scale(scales[(int64_t)by * sh.gx + bx]);
-                if (!EMU && sc.fast) {
+                if (!EMU && sc.fast && !vec_has_nan(v)) {
                     const float rs = 1.0f / sc.s;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) w[j] = bs_pair_fast<E8, ERR, WRITE>(w[j], sc, rs, err);
@@ -1434,6 +1436,14 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
                     for (int k = 0; k < 4; ++k) {
                         uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
                         float row_err = 0.0f;
+                        if (vec_has_nan(v[k])) {          // a NaN among the 8 values: the exact arithmetic for this vector (rare)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                float q0 = bs_element<false, false>(bf16_lo(w[j]), sc[2 * j], row_err);
+                                float q1 = bs_element<false, false>(bf16_hi(w[j]), sc[2 * j + 1], row_err);
+                                w[j] = store_pair<false>(q0, q1);
+                            }
+                        } else
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
                             const float a = fabsf(bf16_lo(w[j])), b = fabsf(bf16_hi(w[j]));
@@ -1595,26 +1605,33 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
             }
             amax_b = group_umax(amax_bits_of(amax2), 64);
         } else {
-            float amaxf = 0.0f;
+            uint32_t amax2 = 0;
             int nnzf = 0;
 #pragma unroll
-            for (int k = 0; k < NV; ++k) acc_amax_nnz(amaxf, nnzf, v[k]);
+            for (int k = 0; k < NV; ++k) {
+                acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+                nnzf += nnz_word(v[k].x) + nnz_word(v[k].y) + nnz_word(v[k].z) + nnz_word(v[k].w);
+            }
             nnz2 = (uint32_t)nnzf;
-            amax_b = f2u(group_max(amaxf, 64));
+            amax_b = group_umax(amax_bits_of(amax2), 64);
         }
         __syncthreads();                          // the previous block's readers of s_f are done
         if (lane == 0) s_f[wave] = u2f(amax_b);
         __syncthreads();
         amax_b = max(max(f2u(s_f[0]), f2u(s_f[1])), max(f2u(s_f[2]), f2u(s_f[3])));
         float amax = u2f(amax_b);
-        if (amax_b > 0x7F800000u) {               // a NaN in the block: the float maximum of the reference skips it (rare)
+        const bool has_nan = amax_b > 0x7F800000u;
+        if (has_nan) {                            // the float maximum and the count of the reference skip a NaN (rare)
             amax = 0.0f;
+            int nans = 0;
 #pragma unroll 1
             for (int ch = tid; ch < nch; ch += WG) {              // from memory again: no second use of the registers
                 const int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
                 const uint4 x = in[base + (uint32_t)r * row_stride + (uint32_t)(ch - r * cpr)];
                 acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
+                if constexpr (PACKED) nans += nan_word(x.x) + nan_word(x.y) + nan_word(x.z) + nan_word(x.w);
             }
+            nnz_total -= nans;                    // the packed count took them for non-zero values
             amax = group_max(amax, 64);
             __syncthreads();
             if (lane == 0) s_f[wave] = amax;
@@ -1624,7 +1641,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
         gmax = fmaxf(gmax, amax);
         nnz_total += (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
         const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
-        if (sc.fast || !(amax > 0.0f)) {          // an all-zero block gives +0 whatever its (clamped) scale is
+        if (!has_nan && (sc.fast || !(amax > 0.0f))) {          // an all-zero block gives +0 whatever its (clamped) scale is
             // For large blocks every vector is finished before the next begins (register barriers): otherwise the
             // compiler hoists work from all of them, and sinks the whole chain of error terms below the last store
             // with every magnitude and quotient alive, which doubles the registers.
@@ -1720,7 +1737,8 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
             if (phase == 1) q = bs_vec_fast<E8, true, false>(v[k], sc, e);          // in place: decision pass,
             else if (phase == 2) q = bs_vec_fast<E8, false, true>(v[k], sc, e);     // write pass
             else q = bs_vec_fast<E8, true, true>(v[k], sc, e);
-            if (sc.fast || !(amax > 0.0f)) {      // an all-zero block gives +0 whatever its (clamped) scale is
+            const bool has_nan = group_umax(vec_has_nan(v[k]) ? 1u : 0u, G) != 0u;          // exact arithmetic for such a block
+            if (!has_nan && (sc.fast || !(amax > 0.0f))) {      // an all-zero block gives +0 whatever its (clamped) scale is
                 err += e;
                 if (c < nchunks && write) store16_rt(out + c, q, nt);
             } else if (c < nchunks) slow |= 1u << k;

@@ -71,6 +71,40 @@ def test_scaling_inplace_and_flavour(G, shape, thr):
         check_scaling(G, a, br, bc, thr, ss, channel, flags=1)
 
 
+# in place with a block-local scale: a decision pass and a gated write pass of the single-pass kernel, for blocks of
+# 2, 4 and 8 vectors per lane, whole and ragged, and a width that is not a power of two (general path)
+@pytest.mark.parametrize("ss", [2, 3])
+@pytest.mark.parametrize("shape", [(64, 4096, 1, 4096, True), (128, 256, 64, 128, False), (256, 384, 128, 128, False),
+                                   (96, 2048, 1, 2048, True), (64, 3072, 1, 3072, True), (200, 256, 100, 128, False)])
+def test_scaling_single_pass_in_place(G, ss, shape):
+    rows, cols, br, bc, channel = shape
+    a = uniform_bits(rows + cols + ss, rows, cols, -300.0, 300.0)
+    a[1, :8] = 0
+    a[3, 5] = 0x8000
+    assert check_scaling(G, a, br, bc, 0.045, ss, channel, inplace=True) == 1
+    assert check_scaling(G, a, br, bc, 0.02, ss, channel, inplace=True) == 3      # fallback: the input stays as it is
+
+
+@pytest.mark.parametrize("ss", [1, 2, 3, 4])
+@pytest.mark.parametrize("shape", [(256, 256, 128, 128, False), (64, 4096, 1, 4096, True), (64, 512, 1, 32, True),
+                                   (512, 64, 128, 1, True), (96, 80, 32, 16, False)])
+def test_scaling_blocks_with_nan_and_inf(G, ss, shape):
+    """A NaN does not become the block's amax (the reference's float maximum skips it), an infinity does; the error sum
+    is NaN either way, which is not above any threshold."""
+    rows, cols, br, bc, channel = shape
+    a = uniform_bits(7 + ss, rows, cols, -100.0, 100.0)
+    a[5, 7] = 0x7FC0
+    a[rows - 3, cols - 2] = 0xFF80
+    print("scaling nan/inf", shape, ss, flush=True)
+    out, meta, gamax, gnnz, gerr = G.block_scaling(a, br, bc, 0.045, ss, channel=channel)
+    want, wmeta, wamax, wnnz, werr = O.block_scaling(a, br, bc, 0.045, ss, channel=channel)
+    assert gnnz[0] == wnnz[0] and meta[0] == wmeta[0]
+    assert (np.isnan(gamax[0]) and np.isnan(wamax[0])) or gamax[0] == wamax[0]
+    assert (np.isnan(gerr[0]) and np.isnan(werr[0])) or np.isclose(gerr[0], werr[0], rtol=1e-6)
+    bad = np.argwhere(out != want)
+    assert len(bad) == 0, f"{len(bad)} differ, first {bad[0]} got {out[tuple(bad[0])]:#06x} want {want[tuple(bad[0])]:#06x}"
+
+
 def test_scaling_reference_bf16_fallback_known_answer(G):
     """test_fake_quantize_block_scaling.py:138-175: the 1.46e11 outlier gives meta 3 and output == input."""
     a = E.fixture_words(256, 256, [(0, 70, 21000, 53768)])
