@@ -7,5 +7,6 @@ operators on top of it and mirrors the reference's `mor.ops` Python API.  `impor
 from . import _cabi  # noqa: F401
 from . import ops  # noqa: F401
 from . import wire  # noqa: F401
+from . import stats  # noqa: F401
 
-__all__ = ["ops", "wire"]
+__all__ = ["ops", "wire", "stats"]
