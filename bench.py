@@ -241,6 +241,11 @@ def other_configs(torch, run, cabi, K, W):
         i = turn[0] = (turn[0] + 1) % 6
         run.fake_quantize(xs6[i], os6[i], mx_meta, 1, 32, 0.0, 2, 2)
     add("mx_e4m3_8192x8192_rotating_buffers_cold_cache", rotating, n * 4 + (n // 32) * 4, n)
+
+    def rotating_copy():          # the floor of that run: the library's plain copy over the same rotation
+        i = turn[0] = (turn[0] + 1) % 6
+        run.fake_quantize(xs6[i], os6[i], meta, 128, 128, 0.0, 7, 1)
+    add("copy_mode7_8192x8192_rotating_buffers_cold_cache", rotating_copy, n * 4 + meta.numel() * 4, n)
     del xs6, os6, mx_meta
     # C1: per-tensor E4M3, 4096x4096, scale from the tensor amax (the quantize pass only: 4 B/element)
     x1 = x[:4096, :4096].contiguous()
@@ -283,6 +288,17 @@ def other_configs(torch, run, cabi, K, W):
     ms_ = torch.empty((1, 1), dtype=torch.int32, device="cuda")
     ms, wall = time_launches(torch, lambda: run.fake_quantize(xs, os_, ms_, 1, 32, 0.0, 2, 2), 200, 20)
     res["tiny_1x32"] = {"us_per_call_events": round(ms * 1e3, 2), "us_per_call_wall": round(wall * 1e3, 2)}
+    # 100 such calls captured in a HIP graph (the C ABI allocates nothing and clears with kernels): per call on replay
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        run.fake_quantize(xs, os_, ms_, 1, 32, 0.0, 2, 2)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(100):
+            run.fake_quantize(xs, os_, ms_, 1, 32, 0.0, 2, 2)
+    ms, wall = time_launches(torch, graph.replay, 20, 3)
+    res["tiny_1x32"]["graph_replay_us_per_call"] = round(ms * 1e3 / 100, 2)
     # the same call through the operator layer a user of the reference calls (allocations of out and meta included)
     import mor
     xg = xs.clone().requires_grad_(True)
