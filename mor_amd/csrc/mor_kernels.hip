@@ -790,15 +790,20 @@ static void launch_rowgroup_f(const uint4* i4, uint4* o4, int32_t* meta, int64_t
         else k_rowgroup<F, E8, NV, 256, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
         return;
     }
-    if (nchunks >= 8ll * WG * 2048) {
-        constexpr int NV = 8;
-        const int grid = (int)cdiv(nchunks, (int64_t)NV * WG);
-        const bool full = nchunks % ((int64_t)NV * WG) == 0;
-        if (G == 4 && full) k_rowgroup<F, E8, NV, 4, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
-        else if (G == 16 && full) k_rowgroup<F, E8, NV, 16, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
-        else k_rowgroup<F, E8, NV, 0, false, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
-    } else {
-        constexpr int NV = 2;
+    // Two vectors per lane: many small workgroups interleave their loads and stores more finely than few large ones
+    // (measured at 8192^2 with 8 / 4 / 2 / 1 vectors per lane: E4M3 41.3 / 40.6 / 39.3 / 42.4 us, E2M3 41.8 / 40.1 /
+    // 37.9 / 38.6 us).
+    constexpr int NV = 2;
+    if (nchunks * 16 >= ((int64_t)4 << 20) && nchunks % ((int64_t)NV * WG) == 0 && (G == 4 || G == 16)) {
+        const int64_t grid64 = nchunks / ((int64_t)NV * WG);
+        if (grid64 <= 0x7FFFFFFFll) {
+            const int grid = (int)grid64;
+            if (G == 4) k_rowgroup<F, E8, NV, 4, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+            else k_rowgroup<F, E8, NV, 16, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
+            return;
+        }
+    }
+    {
         const int grid = (int)cdiv(nchunks, (int64_t)NV * WG);
         if (nchunks * 16 >= ((int64_t)4 << 20)) k_rowgroup<F, E8, NV, 0, false, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
         else k_rowgroup<F, E8, NV, 0, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
