@@ -881,11 +881,7 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
         const int e8v = (int)((sbits >> 23) & 0xFF) - 127;
         if (fast_ok && e8v >= -100 && e8v <= 100) {
             int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
-            if (nvec >= 8ll * WG * 2048) {
-                int grid = (int)cdiv(nvec, 8ll * WG);
-                if (e8) k_elementwise_fast<true, 8><<<grid, WG, 0, st>>>(in16, out16, meta, n, nvec, nblocks, qa.fmt, qa.clamp, qa.meta_val);
-                else k_elementwise_fast<false, 8><<<grid, WG, 0, st>>>(in16, out16, meta, n, nvec, nblocks, qa.fmt, qa.clamp, qa.meta_val);
-            } else {
+            {       // two vectors per lane at every size (as k_rowgroup)
                 int grid = nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16);
                 if (e8) k_elementwise_fast<true, 2><<<grid, WG, 0, st>>>(in16, out16, meta, n, nvec, nblocks, qa.fmt, qa.clamp, qa.meta_val);
                 else k_elementwise_fast<false, 2><<<grid, WG, 0, st>>>(in16, out16, meta, n, nvec, nblocks, qa.fmt, qa.clamp, qa.meta_val);
@@ -946,8 +942,7 @@ extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
             if (output != input) {
                 const int64_t n = rows * cols;
                 const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
-                if (nvec >= 8ll * WG * 2048) k_copy<8><<<(int)cdiv(nvec, 8ll * WG), WG, 0, st>>>(static_cast<const uint16_t*>(input), static_cast<uint16_t*>(output), n, nvec);
-                else k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(static_cast<const uint16_t*>(input), static_cast<uint16_t*>(output), n, nvec);
+                k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(static_cast<const uint16_t*>(input), static_cast<uint16_t*>(output), n, nvec);
             }
             k_fill_i32<<<grid_for(nblocks), WG, 0, st>>>(meta, nblocks, 3);
             return mor_check_launch("k_copy / k_fill_i32");
@@ -1707,6 +1702,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
 // The same single pass for row blocks of 1 x 8G elements, G <= 64 lanes (MX 1 x 32 through the channel op is G = 4):
 // the flat chunk array in tiles of 4 * 256 chunks, a block is G consecutive lanes (amax by DPP), as in k_rowgroup.
 // Groups whose scale is outside the fast range are redone from memory by a second, non-unrolled loop.
+constexpr int BS_ROWS_NV = 4;         // vectors per lane and tile (2 is not faster here: 55.9 against 54.5 us)
 template <bool E8>
 __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* out, uint32_t* ws, int64_t nchunks, int G, int ss_mode,
                                                       const int32_t* meta, int phase) {
@@ -1714,7 +1710,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
     __shared__ int s_i[WAVES];
     if (phase == 2 && meta[0] != 1) return;          // phases as in k_bs_fused
     const bool write = phase != 1;
-    constexpr int NV = 4;
+    constexpr int NV = BS_ROWS_NV;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool nt = streams_out(nchunks * 8);
     float gmax = 0.0f, err = 0.0f;
@@ -1863,7 +1859,7 @@ __global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, 
     const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
     const uint4* in4 = reinterpret_cast<const uint4*>(in);
     uint4* out4 = reinterpret_cast<uint4*>(out);
-    constexpr int NV = 4;                       // a workgroup takes tiles of NV * 256 consecutive 16-byte chunks
+    constexpr int NV = 2;                       // a workgroup takes tiles of NV * 256 consecutive 16-byte chunks
     const int64_t ntiles = (nvec + NV * WG - 1) / (NV * WG);
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int64_t c0 = tile * (NV * WG) + threadIdx.x;
@@ -1983,7 +1979,7 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
     if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && brows == 1 && bcols % 8 == 0 && is_pow2(bcols / 8)
         && bcols / 8 <= 64) {
         const int64_t nchunks = rows * cols / 8;
-        const int grid = (int)std::min<int64_t>(cdiv(nchunks, 4 * WG), MAX_PARTIALS);
+        const int grid = (int)std::min<int64_t>(cdiv(nchunks, BS_ROWS_NV * WG), MAX_PARTIALS);
         const uint4* i4 = static_cast<const uint4*>(input);
         uint4* o4 = static_cast<uint4*>(output);
         const int G = (int)(bcols / 8);
@@ -2066,7 +2062,7 @@ extern "C" int mor_e8mx(const void* input, void* output, int64_t rows, int64_t c
     uint16_t* out16 = static_cast<uint16_t*>(output);
     const int64_t n = rows * cols;
     const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
-    const int grid = nvec > 0 ? (int)std::min<int64_t>(cdiv(nvec, 4 * WG), 1 << 20) : grid_for(n, 16);
+    const int grid = nvec > 0 ? (int)std::min<int64_t>(cdiv(nvec, 2 * WG), 1 << 20) : grid_for(n, 16);
     const int strategy = (int)scaling_strategy;
     int npart = 0;
     if (strategy == 1) {

@@ -605,7 +605,7 @@ extern "C" int mor_mx_quantize(const void* input, void* payload, void* scales, i
     if (int rc = validate_wire(input, payload, scales, rows, cols, fmt, 1)) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t nchunks = rows * cols / 8;
-    constexpr int NV = 4;
+    constexpr int NV = 2;
     const unsigned grid = (unsigned)((nchunks + NV * WWG - 1) / (NV * WWG));
     const uint4* in = static_cast<const uint4*>(input);
     uint8_t* p = static_cast<uint8_t*>(payload);
@@ -643,7 +643,8 @@ extern "C" int mor_mx_dequantize(const void* payload, const void* scales, void* 
     if (int rc = validate_wire(output, payload, scales, rows, cols, fmt, 1)) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t nchunks = rows * cols / 8;
-    const unsigned grid = (unsigned)std::min<int64_t>((nchunks + WWG - 1) / WWG, 256 * 16);
+    // two chunks per lane (grid-stride): 8192^2 E4M3 31.0 us with a grid of 4096 workgroups, 29.4 us with 16384
+    const unsigned grid = (unsigned)std::min<int64_t>((nchunks + 2 * WWG - 1) / (2 * WWG), 0x7FFFFFFFll);
     const uint8_t* p = static_cast<const uint8_t*>(payload);
     const uint8_t* s = static_cast<const uint8_t*>(scales);
     uint4* out = static_cast<uint4*>(output);
