@@ -184,9 +184,35 @@ __device__ __forceinline__ uint16_t fq_one_fast(uint16_t h, int fmt, bool e8, co
 // Walks the elements tid, tid + 256, ... of a bh x bw block in row-major order and calls f(offset of the element
 // from the block's first element) without a division per element: (r, c) advance by (256 / bw, 256 % bw) with one
 // carry.
-template <class F>
+// per-wave partial results in LDS -> the workgroup's result, for NW = 4 or 8 waves (sums in a fixed pairwise order)
+template <int NW> __device__ __forceinline__ float lds_fmax(const float* s) {
+    float m = s[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) m = fmaxf(m, s[w]);
+    return m;
+}
+template <int NW> __device__ __forceinline__ float lds_umaxf(const float* s) {      // maximum of the bit patterns (NaN wins)
+    uint32_t m = f2u(s[0]);
+#pragma unroll
+    for (int w = 1; w < NW; ++w) m = max(m, f2u(s[w]));
+    return u2f(m);
+}
+template <int NW> __device__ __forceinline__ uint32_t lds_umin(const uint32_t* s) {
+    uint32_t m = s[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) m = min(m, s[w]);
+    return m;
+}
+template <int NW> __device__ __forceinline__ float lds_sum(const float* s) {
+    static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+    const float a = (s[0] + s[1]) + (s[2] + s[3]);
+    if constexpr (NW == 8) return a + ((s[4] + s[5]) + (s[6] + s[7]));
+    else return a;
+}
+
+template <int WGS = WG, class F>
 __device__ __forceinline__ void for_block_elements(int64_t bh, int64_t bw, int64_t row_pitch, int tid, F&& f) {
-    const int64_t step_r = WG / bw, step_c = WG % bw;
+    const int64_t step_r = WGS / bw, step_c = WGS % bw;
     int64_t r = tid / bw, c = tid % bw;
 #pragma unroll 1
     while (r < bh) {
@@ -201,10 +227,11 @@ __device__ __forceinline__ void for_block_elements(int64_t bh, int64_t bw, int64
 // It is the body of k_generic and the fallback of k_wgblock for blocks outside the fast range.  FAST (k_generic, default
 // flavour): blocks whose scale is in the fast range use the few-instruction arithmetic, with the same safeguard on
 // close MoR decisions as k_wgblock.
-template <bool EMU, bool FAST = false>
+template <bool EMU, bool FAST = false, int WGS = WG>
 __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out, int32_t* meta, float* stats,
                                               const Shape& sh, const QuantArgs& qa, bool e8, int64_t bid,
-                                              float (*s_f)[WAVES], uint32_t* s_u, bool allow_fast = false) {
+                                              float (*s_f)[WGS / 64], uint32_t* s_u, bool allow_fast = false) {
+    constexpr int NW = WGS / 64;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
     const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
@@ -212,7 +239,7 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
     float amax = 0.0f;
     uint32_t amin_m1 = AMIN_INIT_M1;
     const uint16_t* bin = in + r0 * sh.cols + c0;
-    for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) {
+    for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) {
         uint32_t a = ((uint32_t)bin[at] << 16) & 0x7FFFFFFFu;
         amax = fmaxf(amax, u2f(a));
         amin_m1 = min(amin_m1, a - 1u);
@@ -222,8 +249,8 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
     __syncthreads();
     if (lane == 0) { s_f[0][wave] = amax; s_u[wave] = amin_m1; }
     __syncthreads();
-    amax = fmaxf(fmaxf(s_f[0][0], s_f[0][1]), fmaxf(s_f[0][2], s_f[0][3]));
-    amin_m1 = min(min(s_u[0], s_u[1]), min(s_u[2], s_u[3]));
+    amax = lds_fmax<NW>(s_f[0]);
+    amin_m1 = lds_umin<NW>(s_u);
     const float amin = u2f(amin_m1 + 1u);
 
     int fmt = qa.fmt;
@@ -237,28 +264,28 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
             if constexpr (FAST && !EMU) {
                 if (allow_fast && s4.fast && s4.e8 >= -90 && s4.e8 <= 90) {
                     uint32_t codes = 0;
-                    if (e8) for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<true>((uint32_t)bin[at], s4, e4, e5, codes); });
-                    else for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<false>((uint32_t)bin[at], s4, e4, e5, codes); });
+                    if (e8) for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<true>((uint32_t)bin[at], s4, e4, e5, codes); });
+                    else for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<false>((uint32_t)bin[at], s4, e4, e5, codes); });
                     e4 = wave_sum(e4);
                     e5 = wave_sum(e5);
                     __syncthreads();
                     if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
                     __syncthreads();
-                    e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
-                    e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+                    e4 = lds_sum<NW>(s_f[0]);
+                    e5 = lds_sum<NW>(s_f[1]);
                     exact = !(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5));       // too close: repeat with the reference's divisions
                     if (exact) { e4 = 0.0f; e5 = 0.0f; }
                 }
             }
             if (exact) {
-                for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { err_terms_exact<EMU>(bf16_one(bin[at]), e8, s4, s5, e4, e5); });
+                for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { err_terms_exact<EMU>(bf16_one(bin[at]), e8, s4, s5, e4, e5); });
                 e4 = wave_sum(e4);
                 e5 = wave_sum(e5);
                 __syncthreads();
                 if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
                 __syncthreads();
-                e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
-                e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+                e4 = lds_sum<NW>(s_f[0]);
+                e5 = lds_sum<NW>(s_f[1]);
             }
             qt = mor_decide_error(amax, qa.clamp, e4, e5);
         }
@@ -277,9 +304,9 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
     bool fast = false;
     if constexpr (FAST && !EMU) fast = allow_fast && !copy && sc.fast && sc.e8 >= -90 && sc.e8 <= 90;
     if (fast) {
-        for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) { bout[at] = fq_one_fast(bin[at], fmt, e8, sc); });
+        for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { bout[at] = fq_one_fast(bin[at], fmt, e8, sc); });
     } else {
-        for_block_elements(bh, bw, sh.cols, tid, [&](int64_t at) {
+        for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) {
             uint16_t h = bin[at];
             if (!copy) h = fq_one_exact<EMU>(h, fmt, e8, sc);
             bout[at] = h;
@@ -461,14 +488,24 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
 // Chunk ch = k * 256 + tid of the block sits at block row ch / cpr, chunk column ch % cpr.
 // MOR: per-block format selection (FQ:610-682), else one forced format.  FULL: every block is complete and has
 // exactly NV * 256 chunks, so no predicates.  NT: streaming loads and stores.  Blocks outside the fast range go
-// through generic_block.
-template <bool MOR, bool E8, int NV, bool FULL, int NT>
-__global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
-                                                float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
-    __shared__ float s_f[2][WAVES];
-    __shared__ uint32_t s_u[WAVES];
+// through generic_block.  WGS threads per workgroup (256 everywhere: 512 threads with half the vectors per lane were
+// measured no faster).
+template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG>
+__global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
+                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
+    constexpr int NW = WGS / 64;
+    __shared__ float s_f[2][NW];
+    __shared__ uint32_t s_u[NW];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t bid = blockIdx.x;
+    // Workgroup -> block.  cpr_shift bit 8 (large tensors whose block grid is a multiple of 8 wide): consecutive
+    // workgroup ids go round the 8 XCDs, and each XCD takes a band of gx / 8 block columns, walking it row by row.
+    int64_t bid = blockIdx.x;
+    if (cpr_shift >= 256) {            // (a negative cpr_shift means a chunk count per row that is not a power of two)
+        const int64_t xcd = bid & 7, j = bid >> 3, per = sh.gx >> 3, byb = j / per;
+        bid = byb * sh.gx + xcd * per + (j - byb * per);
+        cpr_shift &= 255;
+        if (cpr_shift == 255) cpr_shift = -1;
+    }
     const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
     const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
     const uint32_t row_stride = (uint32_t)(sh.cols >> 3);          // chunks per tensor row
@@ -483,7 +520,7 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
     bool ok[NV];
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
-        int ch = k * WG + tid;
+        int ch = k * WGS + tid;
         int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
         int cc = ch - r * cpr;
         ok[k] = FULL || ((ch < nch) && (r < rows_valid) && (cc < cols_valid));
@@ -506,8 +543,8 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
     if constexpr (MOR) amin_m1 = group_umin(amin_m1_of(amin2_m1), 64);
     if (lane == 0) { s_f[0][wave] = u2f(amax_b); s_u[wave] = amin_m1; }
     __syncthreads();
-    amax_b = max(max(f2u(s_f[0][0]), f2u(s_f[0][1])), max(f2u(s_f[0][2]), f2u(s_f[0][3])));
-    amin_m1 = min(min(s_u[0], s_u[1]), min(s_u[2], s_u[3]));
+    amax_b = f2u(lds_umaxf<NW>(s_f[0]));
+    amin_m1 = lds_umin<NW>(s_u);
     const float amax = u2f(amax_b);
     const float amin = u2f(amin_m1 + 1u);
 
@@ -515,7 +552,7 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
     const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
     // (a NaN in the block shows as amax_b above the bits of infinity: the exact path takes its maximum as the reference does)
     if (amax_b > 0x7F800000u || (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast))) {           // uniform over the workgroup
-        generic_block<false>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
+        generic_block<false, false, WGS>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
                              sh, qa, E8, bid, s_f, s_u);
         return;
     }
@@ -543,8 +580,8 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
             e5 = wave_sum(e5);
             if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
             __syncthreads();
-            e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
-            e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+            e4 = lds_sum<NW>(s_f[0]);
+            e5 = lds_sum<NW>(s_f[1]);
             if (!(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) {
                 // The sums above divide with a Newton step.  When they are too close for that to be trusted with
                 // the decision, repeat them with IEEE divisions (from memory, non-unrolled: this is rare).
@@ -552,7 +589,7 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
                 const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
                 e4 = 0.0f; e5 = 0.0f;
 #pragma unroll 1
-                for (int64_t i = tid; i < bh * bw; i += WG) {
+                for (int64_t i = tid; i < bh * bw; i += WGS) {
                     int64_t r = i / bw, c = i - r * bw;
                     err_terms_exact<false>(bf16_one(in16[(r0 + r) * sh.cols + c0 + c]), E8, s4, s5, e4, e5);
                 }
@@ -561,8 +598,8 @@ __global__ __launch_bounds__(WG) void k_wgblock(const uint4* in, uint4* out, int
                 __syncthreads();
                 if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
                 __syncthreads();
-                e4 = (s_f[0][0] + s_f[0][1]) + (s_f[0][2] + s_f[0][3]);
-                e5 = (s_f[1][0] + s_f[1][1]) + (s_f[1][2] + s_f[1][3]);
+                e4 = lds_sum<NW>(s_f[0]);
+                e5 = lds_sum<NW>(s_f[1]);
             }
             qt = mor_decide_error(amax, qa.clamp, e4, e5);
         }
@@ -822,7 +859,7 @@ static void launch_rowgroup(int fmt, const void* in, void* out, int32_t* meta, i
     }
 }
 
-template <bool MOR, bool E8, int NV>
+template <bool MOR, bool E8, int NV, int WGS = WG>
 static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, int32_t* meta, float* stats,
                               const Shape& sh, const QuantArgs& qa, int cpr, int shift, hipStream_t st) {
     // Streaming stores for outputs that do not fit an L2 anyway (>= 4 MiB): the quantized tensor then does not evict
@@ -835,7 +872,11 @@ static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, i
     // 8192^2 block E4M3: 41.4 -> 40.1 us), while a grid that fits the chip at once wants every slot (4096^2: 9.2
     // against 10.8 us).
     const size_t dyn_lds = (NV == 8 && grid >= 4096) ? 53000 : 0;
-#define MOR_WGBLOCK(FULL, NT) k_wgblock<MOR, E8, NV, FULL, NT><<<grid, WG, dyn_lds, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift)
+    // Tensors beyond the last-level cache: each XCD takes a band of gx / 8 block columns and walks it row by row, so
+    // that the blocks sharing a DRAM page are in flight on one XCD at about the same time (16384 x 14336, 128 x 128
+    // blocks: MoR 170 -> 157 us, block E4M3 166.6 -> 153.8 us; no difference at 8192^2 and below).
+    const int shift_arg = (ntm == 1 && sh.gx % 8 == 0) ? ((shift & 255) | 256) : shift;
+#define MOR_WGBLOCK(FULL, NT) k_wgblock<MOR, E8, NV, FULL, NT, WGS><<<grid, WGS, dyn_lds, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift_arg)
     if (full) {
         if (ntm == 1) MOR_WGBLOCK(true, 1); else if (ntm == 2) MOR_WGBLOCK(true, 2); else MOR_WGBLOCK(true, 0);
     } else {
@@ -1570,6 +1611,8 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
     const uint32_t row_stride = (uint32_t)(sh.cols >> 3);
     const int nch = (int)sh.brows * cpr;
     const bool nt = streams_out(sh.rows * sh.cols);
+    const bool bands = (cpr_shift & 256) != 0;      // XCD bands of block columns, as in k_wgblock (gx and the grid multiples of 8)
+    cpr_shift &= 255;
     // chunk k * 256 + tid of a block is at off_k(k) + off_tid; cpr is a power of two, so off_k is uniform (no per-lane
     // index arithmetic is carried through the loop over blocks)
     const uint32_t off_tid = cpr_shift <= 8 ? (uint32_t)(tid >> cpr_shift) * row_stride + (uint32_t)(tid & (cpr - 1)) : (uint32_t)tid;
@@ -1579,7 +1622,12 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
     };
     float gmax = 0.0f, err = 0.0f;
     int nnz_total = 0;
-    for (int64_t bid = blockIdx.x; bid < nblocks; bid += gridDim.x) {
+    for (int64_t t = blockIdx.x; t < nblocks; t += gridDim.x) {
+        int64_t bid = t;
+        if (bands) {
+            const int64_t xcd = t & 7, j = t >> 3, per = sh.gx >> 3, byb = j / per;
+            bid = byb * sh.gx + xcd * per + (j - byb * per);
+        }
         const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
         const int64_t base = by * sh.brows * row_stride + ((bx * sh.bcols) >> 3);
         uint4 v[NV];
@@ -1951,11 +1999,13 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
     if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG && blk_chunks <= 8 * WG
         && brows * (cols / 8) < 0x7FFFFFFFll && is_pow2(bcols / 8)) {
         const int cpr = (int)(bcols / 8);
-        const int shift = ilog2(cpr);
         const int nv = (int)cdiv(blk_chunks, WG);
         const int NVc = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
         const bool full = blk_chunks == (int64_t)NVc * WG;
         const int grid = (int)std::min<int64_t>(nb, 4096);      // partials: one per workgroup (the finalize kernel reads them all)
+        // tensors beyond the last-level cache: XCD bands of block columns (16384 x 14336, 128 x 128 blocks: 193 -> 185 us)
+        const bool bands = rows * cols > ((int64_t)128 << 20) && sh.gx % 8 == 0 && grid % 8 == 0 && nb % 8 == 0;
+        const int shift = ilog2(cpr) | (bands ? 256 : 0);
         const uint4* i4 = static_cast<const uint4*>(input);
         uint4* o4 = static_cast<uint4*>(output);
 #define MOR_BS_FUSED(E8, NV, PHASE) do { \
