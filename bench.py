@@ -217,8 +217,8 @@ def other_configs(torch, run, cabi, K, W):
 
     def add(name, fn, nbytes, nelem):
         ms, wall = time_launches(torch, fn, K, W)
-        if ms * K < 3.0:        # short bursts end before the clocks have left their idle state: time about 3 ms of launches
-            ms, wall = time_launches(torch, fn, min(400, int(3.0 / ms) + 1), W)
+        if ms * K < 10.0:       # short bursts are noisy (clock ramp, refresh): time about 10 ms of back-to-back launches
+            ms, wall = time_launches(torch, fn, min(1000, int(10.0 / ms) + 1), W)
         res[name] = {"ms": round(ms, 5), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "elements_per_s": round(nelem / (ms * 1e-3), 0)}
 
@@ -357,12 +357,12 @@ def c5_sweep(torch, run, K, W):
     cache = {}
 
     def timed(key, fn):
-        # short kernels are timed over about 3 ms of back-to-back launches: a burst of a few hundred microseconds
-        # ends before the clocks have left their idle state
+        # every shape is timed over about 10 ms of back-to-back launches: a burst of a few hundred microseconds ends
+        # before the clocks have left their idle state, and a millisecond is still noisy
         if key not in cache:
             ms = time_launches(torch, fn, K, W)[0]
-            if ms * K < 3.0:
-                ms = time_launches(torch, fn, min(400, int(3.0 / ms) + 1), W)[0]
+            if ms * K < 10.0:
+                ms = time_launches(torch, fn, min(1000, int(10.0 / ms) + 1), W)[0]
             cache[key] = ms
         return cache[key]
 

@@ -204,10 +204,11 @@ template <int NW> __device__ __forceinline__ uint32_t lds_umin(const uint32_t* s
     return m;
 }
 template <int NW> __device__ __forceinline__ float lds_sum(const float* s) {
-    static_assert(NW == 4 || NW == 8, "4 or 8 waves");
-    const float a = (s[0] + s[1]) + (s[2] + s[3]);
-    if constexpr (NW == 8) return a + ((s[4] + s[5]) + (s[6] + s[7]));
-    else return a;
+    static_assert(NW == 4 || NW == 8 || NW == 16, "4, 8 or 16 waves");
+    float a = (s[0] + s[1]) + (s[2] + s[3]);
+    if constexpr (NW >= 8) a += (s[4] + s[5]) + (s[6] + s[7]);
+    if constexpr (NW == 16) a += ((s[8] + s[9]) + (s[10] + s[11])) + ((s[12] + s[13]) + (s[14] + s[15]));
+    return a;
 }
 
 template <int WGS = WG, class F>
@@ -488,8 +489,7 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
 // Chunk ch = k * 256 + tid of the block sits at block row ch / cpr, chunk column ch % cpr.
 // MOR: per-block format selection (FQ:610-682), else one forced format.  FULL: every block is complete and has
 // exactly NV * 256 chunks, so no predicates.  NT: streaming loads and stores.  Blocks outside the fast range go
-// through generic_block.  WGS threads per workgroup (256 everywhere: 512 threads with half the vectors per lane were
-// measured no faster).
+// through generic_block.  WGS threads per workgroup: 256, or 512 for one-row blocks of more than 8192 elements.
 template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG>
 __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                  float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
@@ -900,7 +900,12 @@ static void launch_wgblock(const void* in, void* out, int32_t* meta, float* stat
         case 1: launch_wgblock_nv<MOR, E8, 1>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
         case 2: launch_wgblock_nv<MOR, E8, 2>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
         case 4: launch_wgblock_nv<MOR, E8, 4>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
-        default: launch_wgblock_nv<MOR, E8, 8>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
+        default:
+            // a contiguous block (one long row) is faster with 512 threads and 4 vectors per lane (rows of 14336 elements:
+            // 167 -> 157 us at 16384 rows, 38.7 -> 36.2 us at 4096 rows); a 128 x 128 tile is not
+            if (sh.brows == 1) launch_wgblock_nv<MOR, E8, 4, 512>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st);
+            else launch_wgblock_nv<MOR, E8, 8>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st);
+            break;
     }
 }
 

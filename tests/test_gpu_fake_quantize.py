@@ -98,6 +98,9 @@ SHAPES = [
     (37, 45, 16, 32),                 # odd columns: generic kernel
     (1, 32, 1, 32),
     (130, 260, 128, 128),             # ragged, cols not a multiple of 8
+    (12, 14336, 1, 14336),            # one long row per workgroup of 512 threads, last vector partly filled
+    (6, 16384, 1, 16384),             # the same, every vector full
+    (9, 10000, 1, 10000),             # ... and a chunk count per row that is not a power of two
     (16, 40000, 1, 40000),            # block larger than the register-resident limit
 ]
 
