@@ -56,6 +56,12 @@ __device__ __forceinline__ void store16_rt(uint4* p, uint4 v, bool nt) {
     else store16<false>(p, v);
 }
 
+// Inputs stream too once a kernel's traffic (2 bytes read + 2 written per element) exceeds twice the 256 MB last-level
+// cache: nothing of such a tensor is found there again (MX 1 x 32 on 16384 x 14336: 160 -> 150 us; at 8192^2 streaming
+// loads cost 39 -> 44 us).
+__device__ __forceinline__ bool streams_in(int64_t bf16_elements) { return bf16_elements > ((int64_t)128 << 20); }
+__device__ __forceinline__ uint4 load16_rt(const uint4* p, bool nt) { return nt ? load16<true>(p) : load16<false>(p); }
+
 // ---------------------------------------------------------------- bf16 <-> fp32
 // FQ:38-44: a bf16 is the upper half of an fp32.
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }

@@ -339,7 +339,7 @@ __global__ __launch_bounds__(WG) void k_elementwise_fast(const uint16_t* in, uin
     const int64_t base = (int64_t)blockIdx.x * (EW_NV * WG) + threadIdx.x;
     uint4 v[EW_NV];
 #pragma unroll
-    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = in4[c]; }
+    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = load16_rt(in4 + c, streams_in(n)); }
     const bool nt = streams_out(n);
     if (fmt == FMT_E4M3) {
 #pragma unroll
@@ -377,7 +377,7 @@ __global__ __launch_bounds__(WG) void k_copy(const uint16_t* in, uint16_t* out, 
     const int64_t base = (int64_t)blockIdx.x * (EW_NV * WG) + threadIdx.x;
     uint4 v[EW_NV];
 #pragma unroll
-    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = in4[c]; }
+    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = load16_rt(in4 + c, streams_in(n)); }
 #pragma unroll
     for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) store16_rt(out4 + c, v[k], streams_out(n)); }
     for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = in[i];
@@ -395,12 +395,13 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
                                                  int64_t nchunks, int G, int logG, int meta_val) {
     if constexpr (GT > 0) { G = GT; }
     const int64_t base = (int64_t)blockIdx.x * (NV * WG) + threadIdx.x;
+    const bool lnt = streams_in(nchunks * 8);
     uint4 v[NV];
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         int64_t c = base + k * WG;
         v[k] = make_uint4(0, 0, 0, 0);
-        if (FULL || c < nchunks) v[k] = in[c];
+        if (FULL || c < nchunks) v[k] = load16_rt(in + c, lnt);
     }
     // groups wider than a wave (GT = 128 / 256 lanes): the waves' maxima meet in LDS, once for all NV chunks
     float wide_amax[NV];
@@ -1918,7 +1919,7 @@ __global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, 
         const int64_t c0 = tile * (NV * WG) + threadIdx.x;
         uint4 v[NV];
 #pragma unroll
-        for (int k = 0; k < NV; ++k) { v[k] = make_uint4(0, 0, 0, 0); if (c0 + k * WG < nvec) v[k] = in4[c0 + k * WG]; }
+        for (int k = 0; k < NV; ++k) { v[k] = make_uint4(0, 0, 0, 0); if (c0 + k * WG < nvec) v[k] = load16_rt(in4 + c0 + k * WG, streams_in(n)); }
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};

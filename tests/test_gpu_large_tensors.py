@@ -112,3 +112,33 @@ def test_fake_quantize_dual_whole_equals_single_orientation(x):
     _cabi.check(L.mor_fake_quantize(xt.data_ptr(), reft.data_ptr(), mref.data_ptr(), COLS, ROWS, 1, 32, 0.0, 2, 2, 0, stream()))
     torch.cuda.synchronize()
     assert torch.equal(ot.view(torch.int16), reft.view(torch.int16)) and torch.equal(mt, mref)
+
+
+def test_linear_kernels_whole_equals_halves(x):
+    """MX 1 x 32, per-tensor scale and the wire quantizer read such a tensor with streaming loads."""
+    print("large linear kernels", flush=True)
+    L = _cabi.lib()
+    h = ROWS // 2
+
+    def mx(t, mode, sf, br, bc, clamp=0.0):
+        r, c = t.shape
+        out = torch.empty_like(t)
+        meta = torch.full(((r + br - 1) // br, c // bc), -9, dtype=torch.int32, device="cuda")
+        _cabi.check(L.mor_fake_quantize(t.data_ptr(), out.data_ptr(), meta.data_ptr(), r, c, br, bc, clamp, mode, sf, 0, stream()))
+        return out, meta
+
+    for args in ((2, 2, 1, 32), (3, 2, 1, 32), (4, 1, 128, 128, 37.5), (2, 1, 1, 1024)):
+        out, meta = mx(x, *args)
+        for part in (slice(0, h), slice(h, ROWS)):
+            o2, _ = mx(x[part].contiguous(), *args)
+            assert torch.equal(out[part].view(torch.int16), o2.view(torch.int16)), args
+        assert int((meta == -9).sum()) == 0
+    n = ROWS * COLS
+    p, s_ = torch.empty(n, dtype=torch.uint8, device="cuda"), torch.empty(n // 32, dtype=torch.uint8, device="cuda")
+    p2, s2 = torch.empty(n // 2, dtype=torch.uint8, device="cuda"), torch.empty(n // 64, dtype=torch.uint8, device="cuda")
+    _cabi.check(L.mor_mx_quantize(x.data_ptr(), p.data_ptr(), s_.data_ptr(), ROWS, COLS, _cabi.FMT_E4M3, stream()))
+    for k, part in enumerate((slice(0, h), slice(h, ROWS))):
+        xp = x[part].contiguous()
+        _cabi.check(L.mor_mx_quantize(xp.data_ptr(), p2.data_ptr(), s2.data_ptr(), h, COLS, _cabi.FMT_E4M3, stream()))
+        torch.cuda.synchronize()
+        assert torch.equal(p[k * (n // 2):(k + 1) * (n // 2)], p2) and torch.equal(s_[k * (n // 64):(k + 1) * (n // 64)], s2)
