@@ -1146,7 +1146,7 @@ __global__ __launch_bounds__(WG) void k_bs_amax_flat(const uint4* in, uint32_t* 
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             v[k] = make_uint4(0, 0, 0, 0);
-            if (base + k * WG < nchunks) v[k] = in[base + k * WG];
+            if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_in(nchunks * 8));
         }
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
@@ -1195,7 +1195,7 @@ __global__ __launch_bounds__(WG) void k_bs_amax_block(const uint16_t* in, uint32
 #pragma unroll 4
             for (uint32_t i = threadIdx.x; i < nch; i += WG) {
                 const uint32_t r = div_u32(i, d_cpr), cc = i - r * cpr;
-                acc_amax_nnz(amax, nnz, bin[r * row_stride + cc]);
+                acc_amax_nnz(amax, nnz, load16_rt(bin + r * row_stride + cc, streams_in(sh.rows * sh.cols)));
             }
         } else {
             for (int64_t i = threadIdx.x; i < sh.brows * sh.bcols; i += WG) {
@@ -1240,7 +1240,7 @@ __global__ __launch_bounds__(WG) void k_bs_amax_col(const uint16_t* in, uint32_t
             const uint4* in4 = reinterpret_cast<const uint4*>(in);
 #pragma unroll 8
             for (int64_t r = r_begin + rl; r < r_end; r += 8) {
-                const uint4 v = in4[(r * sh.cols + col0) >> 3];
+                const uint4 v = load16_rt(in4 + ((r * sh.cols + col0) >> 3), streams_in(sh.rows * sh.cols));
                 const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -1394,7 +1394,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
         for (uint32_t c = blockIdx.x * WG + threadIdx.x; c < nchunks; c += gridDim.x * WG) {
             const uint32_t row = div_u32(c, d_rowchunks), cc = c - row * row_chunks;
             const uint32_t by = div_u32(row, d_brows);
-            uint4 v = in4[c];
+            uint4 v = load16_rt(in4 + c, streams_in(sh.rows * sh.cols));
             uint32_t w[4] = {v.x, v.y, v.z, v.w};
             if constexpr (COL) {
                 const float* sp = scales + (int64_t)by * sh.cols + (int64_t)cc * 8;
@@ -1477,7 +1477,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         v[k] = make_uint4(0, 0, 0, 0);
-                        if (r + k < r_end) v[k] = in4[(r + k) * row_stride + (col0 >> 3)];
+                        if (r + k < r_end) v[k] = load16_rt(in4 + (r + k) * row_stride + (col0 >> 3), streams_in(sh.rows * sh.cols));
                     }
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
@@ -1776,7 +1776,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             v[k] = make_uint4(0, 0, 0, 0);
-            if (base + k * WG < nchunks) v[k] = in[base + k * WG];
+            if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_in(nchunks * 8));
         }
         uint32_t slow = 0;
 #pragma unroll
