@@ -1493,18 +1493,19 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
                         } else
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
+                            // as bs_pair_fast, with a scale of its own for each of the two columns of the word
                             const float a = fabsf(bf16_lo(w[j])), b = fabsf(bf16_hi(w[j]));
-                            const uint32_t p = hw_pack2<FMT_E4M3>(a * sc[2 * j].s, b * sc[2 * j + 1].s);
-                            const float ca = hw_unpack<FMT_E4M3, 0>(p), cb = hw_unpack<FMT_E4M3, 1>(p);
-                            const float ta = ca * rs[2 * j], tb = cb * rs[2 * j + 1];
-                            const float qa = fmaf(fmaf(-ta, sc[2 * j].s, ca), rs[2 * j], ta);
-                            const float qb = fmaf(fmaf(-tb, sc[2 * j + 1].s, cb), rs[2 * j + 1], tb);
-                            const bool za = (a == 0.0f), zb = (b == 0.0f);
-                            row_err = fmaf(fabsf(qa - a), za ? 0.0f : __builtin_amdgcn_rcpf(a), row_err);
-                            row_err = fmaf(fabsf(qb - b), zb ? 0.0f : __builtin_amdgcn_rcpf(b), row_err);
-                            const uint32_t lo = za ? 0u : ((rhu_bits(qa) >> 16) | (w[j] & 0x8000u));
-                            const uint32_t hi = zb ? 0u : ((rhu_bits(qb) & 0xFFFF0000u) | (w[j] & 0x80000000u));
-                            w[j] = lo | hi;
+                            const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc[2 * j].s, b * sc[2 * j + 1].s));
+                            const float qa = div_by_scale(c.x, sc[2 * j].s, rs[2 * j]);
+                            const float qb = div_by_scale(c.y, sc[2 * j + 1].s, rs[2 * j + 1]);
+                            if constexpr (ERR) {
+                                row_err = fmaf(fabsf(qa - a), fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), row_err);
+                                row_err = fmaf(fabsf(qb - b), fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f), row_err);
+                            }
+                            if constexpr (WRITE) {
+                                const uint32_t nonzero = pk_min_u16(w[j] & 0x7FFF7FFFu, 0x00010001u);
+                                w[j] = store_pair<false>(qa, qb) | (w[j] & (nonzero << 15));
+                            }
                         }
                         err += row_err;
                         if constexpr (WRITE) {
