@@ -128,8 +128,10 @@ MOR_API int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t
  * Exhaustive on-device comparison of the gfx950 FP8 convert instructions with the software
  * cast over all 2^32 fp32 inputs whose magnitude does not exceed the format maximum.
  * mismatches[0] = E4M3 count, mismatches[1] = E5M2 count, mismatches[2] = count of inputs for which
- * the scaled pair converts (codes of both formats in one register, two values decoded at once)
- * differ from the plain converts (device pointer, 3 x uint64).
+ * the scaled converts differ from the plain ones: the fp32 pair converts (codes of both formats in
+ * one register, two values decoded at once) on the same inputs, and the power-of-two quantize step
+ * through the scaled bf16 converts against its ldexp / exponent-arithmetic form for every finite bf16
+ * value and every scale exponent in [-100, 100] (device pointer, 3 x uint64).
  */
 MOR_API int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
 

@@ -239,7 +239,10 @@ template <int F> __device__ __forceinline__ Scale make_scale_e8(float amax) {
 //   |x| * 2^e8 (exact), hardware convert and back, then integer exponent subtraction clamped at 0,
 //   which also yields the reference's 2^(-e8-127) for a zero cast result when e8 < 0.  The sign
 //   comes from the input word (the hardware cast keeps the sign, including on zeros).
-template <int F, bool CLAMP> __device__ __forceinline__ uint32_t e8_pair_fast(uint32_t w, int e8) {
+// (E4M3 / E5M2: this is the reference form of the arithmetic; kernels run e8_pair_fast_scaled below, which the
+// library's selftest compares with it for every finite bf16 value and every e8 of the fast range)
+template <int F, bool CLAMP> __device__ __forceinline__ uint32_t e8_pair_fast_scaled(uint32_t w, int e8);
+template <int F, bool CLAMP> __device__ __forceinline__ uint32_t e8_pair_fast_ref(uint32_t w, int e8) {
     const int e8s = e8 << 23;
     if constexpr (Fmt<F>::hw) {
         float a = ldexpf(fabsf(bf16_lo(w)), e8);
@@ -261,6 +264,10 @@ template <int F, bool CLAMP> __device__ __forceinline__ uint32_t e8_pair_fast(ui
         uint32_t mb = (uint32_t)max((int)rb - e8s, 0) | sb;
         return __builtin_amdgcn_perm(mb, ma, 0x07060302u);
     }
+}
+template <int F, bool CLAMP> __device__ __forceinline__ uint32_t e8_pair_fast(uint32_t w, int e8) {
+    if constexpr (Fmt<F>::hw) return e8_pair_fast_scaled<F, CLAMP>(w, e8);
+    else return e8_pair_fast_ref<F, CLAMP>(w, e8);
 }
 
 // Division by the block scale without a divide per element: with r = RN(1 / s) (one IEEE division per block),
@@ -434,6 +441,35 @@ __device__ __forceinline__ bool vec_has_nan(uint4 v) {
     acc_amax_pk(m, v.x); acc_amax_pk(m, v.y); acc_amax_pk(m, v.z); acc_amax_pk(m, v.w);
     return amax_bits_of(m) > 0x7F800000u;
 }
+// The same pair function for E4M3 / E5M2 through the gfx950 scaled converts, straight from the packed bf16 word:
+// v_cvt_scalef32_pk_fp8/bf8_bf16 gives the codes of |x| / 2^-e8 and v_cvt_scalef32_pk_bf16_fp8/bf8 the packed bf16
+// values of code * 2^-e8 (exact: a code has at most 4 significant bits), 5 instructions for the pair instead of 18.
+// A zero code comes back as 0, where the reference's exponent subtraction leaves 2^(-e8-127) for e8 < 0: the packed
+// maximum with that value puts it back (every non-zero result is far above it).  |e8| <= 126 (callers: |e8| <= 100).
+// mor_selftest_hw_cast compares it with e8_pair_fast_ref for every finite bf16 value and every e8 in [-100, 100].
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+template <int F, bool CLAMP> __device__ __forceinline__ uint32_t e8_pair_fast_scaled(uint32_t w, int e8) {
+    static_assert(Fmt<F>::hw, "E4M3 / E5M2 only");
+    const float scale = u2f((uint32_t)(127 - e8) << 23);                      // 2^-e8
+    uint32_t mag = w & 0x7FFF7FFFu;
+    if constexpr (CLAMP) {          // the reference's hardware cast saturates; the scaled convert returns NaN above fmax
+        const uint32_t lim = (F == FMT_E4M3 ? 0x43E0u : 0x4760u) - ((uint32_t)e8 << 7);      // bf16 bits of fmax * 2^-e8
+        mag = pk_min_u16(mag, lim | (lim << 16));
+    }
+    const s16x2 z = {0, 0};
+    uint32_t res;
+    if constexpr (F == FMT_E4M3) {
+        const s16x2 codes = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(z, __builtin_bit_cast(bf16x2v, mag), scale, false);
+        res = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(__builtin_bit_cast(uint32_t, codes), scale, false));
+    } else {
+        const s16x2 codes = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(z, __builtin_bit_cast(bf16x2v, mag), scale, false);
+        res = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(__builtin_bit_cast(uint32_t, codes), scale, false));
+    }
+    const uint32_t art = e8 < 0 ? (uint32_t)(-e8) << 7 : 0u;                  // bf16 bits of 2^(-e8-127)
+    res = pk_max_u16(res, art | (art << 16));
+    return res | (w & 0x80008000u);
+}
+
 // keeps the compiler from carrying unpacked copies of a data register from one pass over the block to the next
 __device__ __forceinline__ void opaque(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
 

@@ -722,6 +722,22 @@ __global__ __launch_bounds__(WG) void k_selftest_hw_cast(unsigned long long* mis
             bad_scaled += !(((l5 & 0xFFFFu) == (p5 & 0xFFFFu)) && f2u(d5.x) == f2u(hw_unpack<FMT_E5M2, 0>(p5)) && f2u(d5.y) == f2u(hw_unpack<FMT_E5M2, 1>(p5)));
         }
     }
+    // the power-of-two pair function through the scaled converts against the one through ldexp and exponent
+    // arithmetic: every bf16 pattern (finite or not counted alike: only finite ones reach it) and every e8 in [-100, 100]
+    for (uint64_t i = (uint64_t)blockIdx.x * WG + threadIdx.x; i < 65536ull * 201ull; i += stride) {
+        const uint32_t h = (uint32_t)(i & 0xFFFFu);
+        const int e8 = (int)(i >> 16) - 100;
+        if ((h & 0x7F80u) == 0x7F80u) continue;                    // Inf / NaN: such blocks do not take the fast path
+        const uint32_t w = h | ((h ^ 0x8055u) << 16);               // the other half: another finite value or the same class
+        if ((w & 0x7F800000u) == 0x7F800000u) continue;
+        // (without the clamp the pair function is only used on blocks scaled by their own amax: nothing above fmax)
+        const float big = ldexpf(fmaxf(fabsf(bf16_lo(w)), fabsf(bf16_hi(w))), e8);
+        bool ok = big > 448.0f || e8_pair_fast_scaled<FMT_E4M3, false>(w, e8) == e8_pair_fast_ref<FMT_E4M3, false>(w, e8);
+        ok = ok && (big > 57344.0f || e8_pair_fast_scaled<FMT_E5M2, false>(w, e8) == e8_pair_fast_ref<FMT_E5M2, false>(w, e8));
+        ok = ok && e8_pair_fast_scaled<FMT_E4M3, true>(w, e8) == e8_pair_fast_ref<FMT_E4M3, true>(w, e8);
+        ok = ok && e8_pair_fast_scaled<FMT_E5M2, true>(w, e8) == e8_pair_fast_ref<FMT_E5M2, true>(w, e8);
+        bad_scaled += !ok;
+    }
     if (bad4) atomicAdd(&mism[0], bad4);
     if (bad5) atomicAdd(&mism[1], bad5);
     if (bad_scaled) atomicAdd(&mism[2], bad_scaled);
