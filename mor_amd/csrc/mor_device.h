@@ -470,6 +470,20 @@ template <int F, bool CLAMP> __device__ __forceinline__ uint32_t e8_pair_fast_sc
     return res | (w & 0x80008000u);
 }
 
+// E4M3 / E5M2 values of both halves of a packed bf16 word under a power-of-two scale, as two floats: |x| * 2^e8 to
+// codes and code * 2^-e8 back, both by the scaled converts (true arithmetic: a zero code gives 0).  |e8| <= 126.
+template <int F> __device__ __forceinline__ f32x2 e8_pair_values(uint32_t mag2, int e8) {
+    const float scale = u2f((uint32_t)(127 - e8) << 23);
+    const s16x2 z = {0, 0};
+    if constexpr (F == FMT_E4M3) {
+        const s16x2 codes = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(z, __builtin_bit_cast(bf16x2v, mag2), scale, false);
+        return __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(__builtin_bit_cast(uint32_t, codes), scale, false);
+    } else {
+        const s16x2 codes = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(z, __builtin_bit_cast(bf16x2v, mag2), scale, false);
+        return __builtin_amdgcn_cvt_scalef32_pk_f32_bf8(__builtin_bit_cast(uint32_t, codes), scale, false);
+    }
+}
+
 // keeps the compiler from carrying unpacked copies of a data register from one pass over the block to the next
 __device__ __forceinline__ void opaque(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
 

@@ -132,19 +132,16 @@ template <bool E8>
 __device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float& e4, float& e5, uint32_t& codes) {
     float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
     if constexpr (E8) {
-        const int e84 = s4.e8, e85 = s4.e8 + 7;
-        uint32_t p4 = hw_pack2<FMT_E4M3>(ldexpf(a, e84), ldexpf(b, e84));
-        uint32_t p5 = hw_pack2<FMT_E5M2>(ldexpf(a, e85), ldexpf(b, e85));
-        float qa4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p4)) - (e84 << 23), 0));
-        float qb4 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p4)) - (e84 << 23), 0));
-        float qa5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 0>(p5)) - (e85 << 23), 0));
-        float qb5 = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E5M2, 1>(p5)) - (e85 << 23), 0));
-        float ya = (a != 0.0f) ? __builtin_amdgcn_rcpf(a) : 0.0f;
-        float yb = (b != 0.0f) ? __builtin_amdgcn_rcpf(b) : 0.0f;
-        e4 = fmaf(fabsf(qa4 - a), ya, e4);
-        e5 = fmaf(fabsf(qa5 - a), ya, e5);
-        e4 = fmaf(fabsf(qb4 - b), yb, e4);
-        e5 = fmaf(fabsf(qb5 - b), yb, e5);
+        // q = cast(x 2^e8) 2^-e8 by the scaled converts from the packed word (a zero code gives 0 where the reference's
+        // exponent arithmetic leaves 2^(-e8-127): a difference far below the terms' rounding errors); a zero element has
+        // q = 0, so its term is 0 * min(1 / 0, FLT_MAX) = 0
+        const uint32_t mag2 = w & 0x7FFF7FFFu;
+        const f32x2 q4 = e8_pair_values<FMT_E4M3>(mag2, s4.e8), q5 = e8_pair_values<FMT_E5M2>(mag2, s4.e8 + 7);
+        const float ya = fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), yb = fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f);
+        e4 = fmaf(fabsf(q4.x - a), ya, e4);
+        e5 = fmaf(fabsf(q5.x - a), ya, e5);
+        e4 = fmaf(fabsf(q4.y - b), yb, e4);
+        e5 = fmaf(fabsf(q5.y - b), yb, e5);
     } else {
         // y + 2^-100 is y for every non-zero element of such a block and keeps the reciprocal of a zero element
         // finite: its codes are 0 and c - x s = 0 (one fma, x s not rounded), so its term is 0 without a select
@@ -1362,12 +1359,12 @@ __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, fl
     const float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
     float qa, qb;
     if constexpr (E8) {
-        const int e8s = sc.e8 << 23;
-        uint32_t p = hw_pack2<FMT_E4M3>(ldexpf(a, sc.e8), ldexpf(b, sc.e8));
-        qa = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 0>(p)) - e8s, 0));
-        qb = u2f((uint32_t)max((int)f2u(hw_unpack<FMT_E4M3, 1>(p)) - e8s, 0));
-        qa = (a == 0.0f) ? 0.0f : qa;                // the exponent arithmetic turns a zero code into 2^-e8 (e8 < 0), and
-        qb = (b == 0.0f) ? 0.0f : qb;                // zero inputs are skipped by the reference (FQ:1133)
+        // scaled converts from the packed word; a zero code of a non-zero element is the reference's 2^(-e8-127) for
+        // e8 < 0 (its exponent subtraction, FQ:296-303), zero inputs are skipped by the reference (FQ:1133) and stay 0
+        const f32x2 q = e8_pair_values<FMT_E4M3>(w & 0x7FFF7FFFu, sc.e8);
+        const float art = u2f(sc.e8 < 0 ? (uint32_t)(-sc.e8) << 23 : 0u);
+        qa = (a == 0.0f) ? 0.0f : fmaxf(q.x, art);
+        qb = (b == 0.0f) ? 0.0f : fmaxf(q.y, art);
     } else {
         const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc.s, b * sc.s));
         qa = div_by_scale(c.x, sc.s, rs);
