@@ -370,6 +370,11 @@ def c5_sweep(torch, run, K, W):
         return src[: r * c].view(r, c)
 
     fam = {}
+    # the buffers are fresh: the first tens of milliseconds on them run slower (first touch), so they are not timed
+    xw, ow = view(big, T, D), view(obuf, T, D)
+    for _ in range(300):
+        run.fake_quantize(xw, ow, mbuf, 128, 128, 1e-15, 1, 1)
+    torch.cuda.synchronize()
 
     def family(name, entries):
         tot_b = tot_ms = 0.0
