@@ -488,7 +488,10 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
 // MOR: per-block format selection (FQ:610-682), else one forced format.  FULL: every block is complete and has
 // exactly NV * 256 chunks, so no predicates.  NT: streaming loads and stores.  Blocks outside the fast range go
 // through generic_block.  WGS threads per workgroup: 256, or 512 for one-row blocks of more than 8192 elements.
-template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG>
+// GATHER: the block's elements are read and written one by one (odd column counts, pointers or block widths that are
+// not multiples of 16 bytes): element s * WGS + tid of the block, counted row by row over its valid part, is half s % 2
+// of word s / 2; every later step is elementwise, so nothing else changes.
+template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false>
 __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                  float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
     constexpr int NW = WGS / 64;
@@ -516,6 +519,32 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     uint4 v[NV];
     uint32_t off[NV];
     bool ok[NV];
+    // GATHER: the walk over the block's valid elements advances by WGS elements per slot (no division per element)
+    const int g_bw = (int)min(sh.bcols, sh.cols - c0);
+    const int g_step_r = WGS / g_bw, g_step_c = WGS % g_bw;
+    const uint32_t g_cols = (uint32_t)sh.cols;
+    if constexpr (GATHER) {
+        const uint16_t* src = reinterpret_cast<const uint16_t*>(in) + (r0 * sh.cols + c0);
+        int r = tid / g_bw, c = tid - r * g_bw;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            ok[k] = true;
+            off[k] = 0;
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                uint32_t e[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    e[h] = (r < rows_valid) ? (uint32_t)src[(uint32_t)r * g_cols + (uint32_t)c] : 0u;
+                    r += g_step_r; c += g_step_c;
+                    if (c >= g_bw) { c -= g_bw; ++r; }
+                }
+                w[j] = e[0] | (e[1] << 16);
+            }
+            v[k] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    } else {
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         int ch = k * WGS + tid;
@@ -525,6 +554,25 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
         off[k] = (uint32_t)r * row_stride + (uint32_t)cc;
         if (ok[k]) v[k] = load16<(NT == 1)>(bin + off[k]);
     }
+    }
+    // the store of one result vector (GATHER: element by element along the same walk, which `put` is called in order of)
+    int g_r = tid / g_bw, g_c = tid - g_r * g_bw;
+    auto put = [&](int k, uint4 q) {
+        if constexpr (GATHER) {
+            uint16_t* dst = reinterpret_cast<uint16_t*>(out) + (r0 * sh.cols + c0);
+            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    if (g_r < rows_valid) dst[(uint32_t)g_r * g_cols + (uint32_t)g_c] = (uint16_t)(w[j] >> (16 * h));
+                    g_r += g_step_r; g_c += g_step_c;
+                    if (g_c >= g_bw) { g_c -= g_bw; ++g_r; }
+                }
+        } else {
+            store16<(NT != 0)>(bout + off[k], q);
+        }
+    };
 
     // pass 1 (registers): amax and min over non-zero magnitudes, FQ:407-485
     // (packed 16-bit integer maxima / minima of both halves of a word; the data stays packed in its registers)
@@ -614,7 +662,7 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     if ((fmt < 0) || !(amax > 0.0f)) {
         if (out != in) {
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], v[k]);
+            for (int k = 0; k < NV; ++k) if (ok[k]) put(k, v[k]);
         }
         return;
     }
@@ -623,10 +671,10 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
             const float r4 = 1.0f / s4.s;            // 1 / s5 = r4 / 128 exactly
             if (fmt == FMT_E4M3) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_div<FMT_E4M3>(v[k], s4.s, r4));
+                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_div<FMT_E4M3>(v[k], s4.s, r4));
             } else {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f));
+                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f));
             }
             return;
         }
@@ -635,21 +683,21 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     switch (fmt) {
         case FMT_E4M3:
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_fast<FMT_E4M3, E8>(v[k], sc));
+            for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_fast<FMT_E4M3, E8>(v[k], sc));
             break;
         case FMT_E5M2:
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_fast<FMT_E5M2, E8>(v[k], sc));
+            for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_fast<FMT_E5M2, E8>(v[k], sc));
             break;
         case FMT_E3M2:
             if constexpr (!MOR) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_fast<FMT_E3M2, E8>(v[k], sc));
+                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_fast<FMT_E3M2, E8>(v[k], sc));
             }
             break;
         default:
 #pragma unroll
-            for (int k = 0; k < NV; ++k) if (ok[k]) store16<(NT != 0)>(bout + off[k], fq_vec_fast<FMT_E2M3, E8>(v[k], sc));
+            for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_fast<FMT_E2M3, E8>(v[k], sc));
             break;
     }
 }
@@ -923,6 +971,19 @@ static void launch_wgblock(const void* in, void* out, int32_t* meta, float* stat
     }
 }
 
+// Blocks of up to 16384 elements whose rows cannot be read as 16-byte vectors: the same kernel with element-wise
+// loads and stores (4097 x 4095 MoR 128 x 128: 84 us through k_generic).
+template <bool MOR, bool E8>
+static void launch_wgblock_gather(const void* in, void* out, int32_t* meta, float* stats, const Shape& sh, const QuantArgs& qa, hipStream_t st) {
+    const int grid = (int)(sh.gy * sh.gx);
+    const int nv = (int)cdiv(sh.brows * sh.bcols, 8 * WG);
+    const uint4* i4 = static_cast<const uint4*>(in);
+    uint4* o4 = static_cast<uint4*>(out);
+#define MOR_GATHER(NV) k_wgblock<MOR, E8, NV, false, 0, WG, true><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, 1, 0)
+    if (nv <= 1) MOR_GATHER(1); else if (nv <= 2) MOR_GATHER(2); else if (nv <= 4) MOR_GATHER(4); else MOR_GATHER(8);
+#undef MOR_GATHER
+}
+
 // Common driver of mor_fake_quantize / mor_block_format / mor_mor_stats.
 static int run_quantize(const void* input, void* output, int32_t* meta, float* stats,
                         int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
@@ -970,6 +1031,16 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
             else launch_wgblock<false, false>(input, output, meta, stats, sh, qa, st);
         }
         return mor_check_launch("k_wgblock");
+    }
+    if (fast_ok && brows * bcols <= 64 * WG && brows * cols < 0x7FFFFFFFll && nblocks <= 0x7FFFFFFFll) {
+        if (qa.qmode == 1) {
+            if (e8) launch_wgblock_gather<true, true>(input, output, meta, stats, sh, qa, st);
+            else launch_wgblock_gather<true, false>(input, output, meta, stats, sh, qa, st);
+        } else {
+            if (e8) launch_wgblock_gather<false, true>(input, output, meta, stats, sh, qa, st);
+            else launch_wgblock_gather<false, false>(input, output, meta, stats, sh, qa, st);
+        }
+        return mor_check_launch("k_wgblock (element-wise)");
     }
     // bit 0: power-of-two scale; bit 1: the few-instruction arithmetic (hardware converts) is allowed
     const int gflags = (e8 ? 1 : 0) | (fast_ok ? 2 : 0);
