@@ -488,9 +488,9 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
 // MOR: per-block format selection (FQ:610-682), else one forced format.  FULL: every block is complete and has
 // exactly NV * 256 chunks, so no predicates.  NT: streaming loads and stores.  Blocks outside the fast range go
 // through generic_block.  WGS threads per workgroup: 256, or 512 for one-row blocks of more than 8192 elements.
-// GATHER: the block's elements are read and written one by one (odd column counts, pointers or block widths that are
-// not multiples of 16 bytes): element s * WGS + tid of the block, counted row by row over its valid part, is half s % 2
-// of word s / 2; every later step is elementwise, so nothing else changes.
+// GATHER: the block's elements are read and written pair by pair (odd column counts, pointers or block widths that are
+// not multiples of 16 bytes): a lane's words are pairs of neighbouring elements of a row; every later step is
+// elementwise, so nothing else changes.
 template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false>
 __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                  float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
@@ -519,13 +519,17 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     uint4 v[NV];
     uint32_t off[NV];
     bool ok[NV];
-    // GATHER: the walk over the block's valid elements advances by WGS elements per slot (no division per element)
+    // GATHER: word s of a lane is pair s * WGS + tid of the block's valid part, pairs counted row by row (the last pair of
+    // a row of odd width has one element); the walk advances by WGS pairs per word, without a division per word.  A pair
+    // is one 4-byte access at a 2-byte-aligned address.
+    typedef uint32_t u32_a2 __attribute__((aligned(2)));
     const int g_bw = (int)min(sh.bcols, sh.cols - c0);
-    const int g_step_r = WGS / g_bw, g_step_c = WGS % g_bw;
+    const int g_pr = (g_bw + 1) >> 1;                                   // pairs per row
+    const int g_step_r = WGS / g_pr, g_step_c = WGS % g_pr;
     const uint32_t g_cols = (uint32_t)sh.cols;
     if constexpr (GATHER) {
         const uint16_t* src = reinterpret_cast<const uint16_t*>(in) + (r0 * sh.cols + c0);
-        int r = tid / g_bw, c = tid - r * g_bw;
+        int r = tid / g_pr, cp = tid - r * g_pr;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             ok[k] = true;
@@ -533,14 +537,13 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
             uint32_t w[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                uint32_t e[2];
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    e[h] = (r < rows_valid) ? (uint32_t)src[(uint32_t)r * g_cols + (uint32_t)c] : 0u;
-                    r += g_step_r; c += g_step_c;
-                    if (c >= g_bw) { c -= g_bw; ++r; }
+                w[j] = 0;
+                if (r < rows_valid) {
+                    const uint16_t* p = src + ((uint32_t)r * g_cols + 2u * (uint32_t)cp);
+                    w[j] = (2 * cp + 1 < g_bw) ? *reinterpret_cast<const u32_a2*>(p) : (uint32_t)*p;
                 }
-                w[j] = e[0] | (e[1] << 16);
+                r += g_step_r; cp += g_step_c;
+                if (cp >= g_pr) { cp -= g_pr; ++r; }
             }
             v[k] = make_uint4(w[0], w[1], w[2], w[3]);
         }
@@ -555,20 +558,22 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
         if (ok[k]) v[k] = load16<(NT == 1)>(bin + off[k]);
     }
     }
-    // the store of one result vector (GATHER: element by element along the same walk, which `put` is called in order of)
-    int g_r = tid / g_bw, g_c = tid - g_r * g_bw;
+    // the store of one result vector (GATHER: pair by pair along the same walk, which `put` is called in order of)
+    int g_r = tid / g_pr, g_cp = tid - g_r * g_pr;
     auto put = [&](int k, uint4 q) {
         if constexpr (GATHER) {
             uint16_t* dst = reinterpret_cast<uint16_t*>(out) + (r0 * sh.cols + c0);
             const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    if (g_r < rows_valid) dst[(uint32_t)g_r * g_cols + (uint32_t)g_c] = (uint16_t)(w[j] >> (16 * h));
-                    g_r += g_step_r; g_c += g_step_c;
-                    if (g_c >= g_bw) { g_c -= g_bw; ++g_r; }
+            for (int j = 0; j < 4; ++j) {
+                if (g_r < rows_valid) {
+                    uint16_t* p = dst + ((uint32_t)g_r * g_cols + 2u * (uint32_t)g_cp);
+                    if (2 * g_cp + 1 < g_bw) *reinterpret_cast<u32_a2*>(p) = w[j];
+                    else *p = (uint16_t)w[j];
                 }
+                g_r += g_step_r; g_cp += g_step_c;
+                if (g_cp >= g_pr) { g_cp -= g_pr; ++g_r; }
+            }
         } else {
             store16<(NT != 0)>(bout + off[k], q);
         }
@@ -976,7 +981,7 @@ static void launch_wgblock(const void* in, void* out, int32_t* meta, float* stat
 template <bool MOR, bool E8>
 static void launch_wgblock_gather(const void* in, void* out, int32_t* meta, float* stats, const Shape& sh, const QuantArgs& qa, hipStream_t st) {
     const int grid = (int)(sh.gy * sh.gx);
-    const int nv = (int)cdiv(sh.brows * sh.bcols, 8 * WG);
+    const int nv = (int)cdiv(sh.brows * ((sh.bcols + 1) / 2), 4 * WG);        // a lane's word is one pair of a row
     const uint4* i4 = static_cast<const uint4*>(in);
     uint4* o4 = static_cast<uint4*>(out);
 #define MOR_GATHER(NV) k_wgblock<MOR, E8, NV, false, 0, WG, true><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, 1, 0)
@@ -1032,7 +1037,7 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
         }
         return mor_check_launch("k_wgblock");
     }
-    if (fast_ok && brows * bcols <= 64 * WG && brows * cols < 0x7FFFFFFFll && nblocks <= 0x7FFFFFFFll) {
+    if (fast_ok && brows * ((bcols + 1) / 2) <= 32 * WG && brows * cols < 0x7FFFFFFFll && nblocks <= 0x7FFFFFFFll) {
         if (qa.qmode == 1) {
             if (e8) launch_wgblock_gather<true, true>(input, output, meta, stats, sh, qa, st);
             else launch_wgblock_gather<true, false>(input, output, meta, stats, sh, qa, st);

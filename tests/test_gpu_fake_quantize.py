@@ -102,6 +102,11 @@ SHAPES = [
     (6, 16384, 1, 16384),             # the same, every vector full
     (9, 10000, 1, 10000),             # ... and a chunk count per row that is not a power of two
     (16, 40000, 1, 40000),            # block larger than the register-resident limit
+    (300, 7, 64, 1),                  # blocks one column wide: every pair of the element-wise kernel is half empty
+    (257, 33, 128, 3),                # odd block width, partial last block row and column
+    (500, 129, 100, 127),             # odd width close to the pair capacity of a workgroup
+    (9000, 5, 8192, 1),               # 8192 single-element pairs: the capacity itself
+    (9000, 5, 8193, 1),               # ... and one more: the generic kernel
 ]
 
 
