@@ -30,6 +30,10 @@ extern "C" {
 #define MOR_ERR_WORKSPACE (-2)          /* workspace missing or too small */
 #define MOR_ERR_LAUNCH (-3)             /* hipGetLastError() after a launch */
 
+/* The largest tensor an entry point takes: 2^35 elements (64 GiB of bf16).  Larger ones are refused with
+ * MOR_ERR_INVALID_ARGUMENT (the scaling ops, whose element counts are 32-bit as in the reference, stop at 2^34). */
+#define MOR_MAX_ELEMENTS (1ll << 35)
+
 /* flags */
 #define MOR_FLAG_DEFAULT 0u
 /* Return what the reference's torch emulation returns instead of what its CUDA

@@ -314,10 +314,10 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
 
 template <bool EMU>
 __global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* out, int32_t* __restrict__ meta,
-                                                float* __restrict__ stats, Shape sh, QuantArgs qa, int e8) {
+                                                float* __restrict__ stats, Shape sh, QuantArgs qa, int e8, int64_t first) {
     __shared__ float s_f[2][WAVES];
     __shared__ uint32_t s_u[WAVES];
-    generic_block<EMU, true>(in, out, meta, stats, sh, qa, (e8 & 1) != 0, blockIdx.x, s_f, s_u, (e8 & 2) != 0);
+    generic_block<EMU, true>(in, out, meta, stats, sh, qa, (e8 & 1) != 0, first + blockIdx.x, s_f, s_u, (e8 & 2) != 0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -493,14 +493,15 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
 // elementwise, so nothing else changes.
 template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false>
 __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
-                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift) {
+                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift,
+                                                 int64_t first) {
     constexpr int NW = WGS / 64;
     __shared__ float s_f[2][NW];
     __shared__ uint32_t s_u[NW];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // Workgroup -> block.  cpr_shift bit 8 (large tensors whose block grid is a multiple of 8 wide): consecutive
     // workgroup ids go round the 8 XCDs, and each XCD takes a band of gx / 8 block columns, walking it row by row.
-    int64_t bid = blockIdx.x;
+    int64_t bid = first + blockIdx.x;       // (a launch holds a slice of the blocks, see for_slices)
     if (cpr_shift >= 256) {            // (a negative cpr_shift means a chunk count per row that is not a power of two)
         const int64_t xcd = bid & 7, j = bid >> 3, per = sh.gx >> 3, byb = j / per;
         bid = byb * sh.gx + xcd * per + (j - byb * per);
@@ -711,10 +712,10 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
 // Debug view: per block amax, fp32 scale, biased exponent of the scale.
 __global__ __launch_bounds__(WG) void k_block_stats(const uint16_t* __restrict__ in, Shape sh, float fmax,
                                                     float* __restrict__ amax_o, float* __restrict__ scale_o,
-                                                    int32_t* __restrict__ e8m0_o) {
+                                                    int32_t* __restrict__ e8m0_o, int64_t first) {
     __shared__ float s_f[WAVES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t bid = blockIdx.x;
+    const int64_t bid = first + blockIdx.x;
     const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
     const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
     const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
@@ -870,6 +871,13 @@ static int grid_for(int64_t work_items, int per_cu = 8) {
     return (int)(want < cap ? want : cap);
 }
 
+// A launch holds fewer than 2^32 threads per dimension (a larger grid wraps without an error): kernels that take one
+// workgroup per block are launched slice by slice, f(first block, blocks of the slice).
+constexpr int64_t LAUNCH_SLICE = (int64_t)1 << 22;
+template <class Fn> static void for_slices(int64_t nblocks, Fn&& f) {
+    for (int64_t first = 0; first < nblocks; first += LAUNCH_SLICE) f(first, (int)std::min(LAUNCH_SLICE, nblocks - first));
+}
+
 extern "C" const char* mor_last_error(void) { return g_err; }
 extern "C" const char* mor_version(void) { return "mor_hip 0.1 (gfx950)"; }
 
@@ -878,6 +886,8 @@ static int validate_shape(const void* input, int64_t rows, int64_t cols, int64_t
     if (rows <= 0 || cols <= 0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "rows and cols must be positive (got %lld x %lld)", (long long)rows, (long long)cols);
     if (brows <= 0 || bcols <= 0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "block dims must be positive (got %lld x %lld)", (long long)brows, (long long)bcols);
     if (cdiv(rows, brows) * cdiv(cols, bcols) > 0x7FFFFFFFll) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many blocks");
+    // 2^35 elements (64 GiB of bf16): the flat kernels' grids, one workgroup per 512 vectors, stay below 2^24 workgroups
+    if (rows > MOR_MAX_ELEMENTS / cols) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor too large (more than 2^35 elements)");
     return MOR_OK;
 }
 
@@ -943,7 +953,8 @@ static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, i
     // that the blocks sharing a DRAM page are in flight on one XCD at about the same time (16384 x 14336, 128 x 128
     // blocks: MoR 170 -> 157 us, block E4M3 166.6 -> 153.8 us; no difference at 8192^2 and below).
     const int shift_arg = (ntm == 1 && sh.gx % 8 == 0) ? ((shift & 255) | 256) : shift;
-#define MOR_WGBLOCK(FULL, NT) k_wgblock<MOR, E8, NV, FULL, NT, WGS><<<grid, WGS, dyn_lds, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift_arg)
+#define MOR_WGBLOCK(FULL, NT) for_slices(grid, [&](int64_t first, int count) { \
+        k_wgblock<MOR, E8, NV, FULL, NT, WGS><<<count, WGS, dyn_lds, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift_arg, first); })
     if (full) {
         if (ntm == 1) MOR_WGBLOCK(true, 1); else if (ntm == 2) MOR_WGBLOCK(true, 2); else MOR_WGBLOCK(true, 0);
     } else {
@@ -984,7 +995,8 @@ static void launch_wgblock_gather(const void* in, void* out, int32_t* meta, floa
     const int nv = (int)cdiv(sh.brows * ((sh.bcols + 1) / 2), 4 * WG);        // a lane's word is one pair of a row
     const uint4* i4 = static_cast<const uint4*>(in);
     uint4* o4 = static_cast<uint4*>(out);
-#define MOR_GATHER(NV) k_wgblock<MOR, E8, NV, false, 0, WG, true><<<grid, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, 1, 0)
+#define MOR_GATHER(NV) for_slices(grid, [&](int64_t first, int count) { \
+        k_wgblock<MOR, E8, NV, false, 0, WG, true><<<count, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, 1, 0, first); })
     if (nv <= 1) MOR_GATHER(1); else if (nv <= 2) MOR_GATHER(2); else if (nv <= 4) MOR_GATHER(4); else MOR_GATHER(8);
 #undef MOR_GATHER
 }
@@ -1049,8 +1061,10 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
     }
     // bit 0: power-of-two scale; bit 1: the few-instruction arithmetic (hardware converts) is allowed
     const int gflags = (e8 ? 1 : 0) | (fast_ok ? 2 : 0);
-    if (emu) k_generic<true><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags);
-    else k_generic<false><<<(int)nblocks, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags);
+    for_slices(nblocks, [&](int64_t first, int count) {
+        if (emu) k_generic<true><<<count, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags, first);
+        else k_generic<false><<<count, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags, first);
+    });
     return mor_check_launch("k_generic");
 }
 
@@ -1114,7 +1128,9 @@ extern "C" int mor_block_stats(const void* input, int64_t rows, int64_t cols, in
     if (int rc = validate_shape(input, rows, cols, brows, bcols)) return rc;
     if (!amax || !scale || !e8m0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
     Shape sh{rows, cols, brows, bcols, cdiv(rows, brows), cdiv(cols, bcols)};
-    k_block_stats<<<(int)(sh.gy * sh.gx), WG, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const uint16_t*>(input), sh, fmax, amax, scale, e8m0);
+    for_slices(sh.gy * sh.gx, [&](int64_t first, int count) {
+        k_block_stats<<<count, WG, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const uint16_t*>(input), sh, fmax, amax, scale, e8m0, first);
+    });
     return mor_check_launch("k_block_stats");
 }
 

@@ -598,6 +598,7 @@ static int validate_wire(const void* a, const void* b, const void* c, int64_t ro
     if (cols % 32 || rows % row_multiple)
         return mor_fail(MOR_ERR_INVALID_ARGUMENT, "MX blocks need cols %% 32 == 0 and rows %% %lld == 0 (got %lld x %lld)", (long long)row_multiple, (long long)rows, (long long)cols);
     if (fmt < MOR_FMT_E4M3 || fmt > MOR_FMT_E2M3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "unknown element format %d", fmt);
+    if (rows > MOR_MAX_ELEMENTS / cols) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor too large (more than 2^35 elements)");
     if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor and payload must be 16-byte aligned");
     if (reinterpret_cast<uintptr_t>(c) & 3u) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "scales must be 4-byte aligned");
     return MOR_OK;
@@ -678,7 +679,7 @@ extern "C" int mor_fake_quantize_dual(const void* input, void* output_rows, int3
     if (qmode != 2 && qmode != 3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mode must be 2 (E4M3) or 3 (E5M2), got %lld", (long long)mode);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t tiles = ((rows + 127) / 128) * ((cols + TILE_C - 1) / TILE_C);
-    if (tiles > 0x7FFFFFFFll) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many tiles");
+    if (rows > MOR_MAX_ELEMENTS / cols) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor too large (more than 2^35 elements)");
     const uint4* in = static_cast<const uint4*>(input);
     uint4* orow = static_cast<uint4*>(output_rows);
     uint16_t* ocol = static_cast<uint16_t*>(output_cols);
