@@ -3,12 +3,15 @@
 // One pass over HBM wherever a quantization block fits in registers:
 //   k_rowgroup   blocks 1 x 8G elements (G = 1..256 lanes, 16-byte loads; the MX 1x32 case is G = 4):
 //                amax by DPP inside the lane group, quantize from registers, 16-byte stores.
-//   k_wgblock    one 256-thread workgroup per block of up to 16384 elements (128x128 tiles, 1x4096 rows):
-//                the block lives in registers as 16-byte vectors; amax / min-nonzero / MoR error sums by
-//                DPP + LDS; the MoR decision and the quantization reuse the registers.
+//   k_wgblock    one workgroup per block of up to 65536 elements (128x128 tiles, 1x4096 rows: 256 threads; up to
+//                32768 / 65536 elements: 512 / 1024 threads): the block lives in registers as 16-byte vectors;
+//                amax / min-nonzero / MoR error sums by DPP + LDS; the MoR decision and the quantization reuse the
+//                registers.  A variant reads and writes pairs of elements where rows cannot be read as vectors.
+//   k_bigblock   larger blocks of whole vectors: one 512-thread workgroup per block, a pass over the block per step
+//                (the repeated reads come from cache).
 //   k_elementwise  current-scaling modes (the scale is an argument): flat 16-byte vectors + scalar tail.
-//   k_generic    any block shape and alignment (odd columns, partial blocks, huge blocks): scalar loads,
-//                exact arithmetic only, the block is re-read from cache for each pass.
+//   k_generic    any block shape and alignment (odd columns, partial blocks, huge blocks) and the other flavours:
+//                scalar loads, the block is re-read from cache for each pass.
 // "FQ" below is the reference file mor/csrc/cuda/fake_quantize.cu.
 
 #include <hip/hip_runtime.h>
@@ -709,6 +712,149 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
 }
 
 // ------------------------------------------------------------------------------------------------
+// k_bigblock: blocks of more than 16384 elements whose rows can be read as 16-byte vectors (rows of 28672 or 131072
+// elements, 256 x 256 tiles, ...).  One 512-thread workgroup per block, as the reference's one thread block per block
+// (FQ:1782-1790).  The block does not fit the registers, so every pass reads it again, four vectors in flight per
+// lane; the second and third read come from L2 / the last-level cache, HBM still sees one read and one write.
+// The steps are those of k_wgblock.
+constexpr int BIG_WG = 512;
+template <bool MOR, bool E8>
+__global__ __launch_bounds__(BIG_WG) void k_bigblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
+                                                     float* __restrict__ stats, Shape sh, QuantArgs qa, int64_t first) {
+    constexpr int WGS = BIG_WG, NW = WGS / 64, UN = 4;
+    __shared__ float s_f[2][NW];
+    __shared__ uint32_t s_u[NW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t bid = first + blockIdx.x;
+    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3);          // chunks per tensor row
+    const uint4* bin = in + (r0 * row_stride + (c0 >> 3));
+    uint4* bout = out ? out + (r0 * row_stride + (c0 >> 3)) : nullptr;
+    const int rows_valid = (int)min(sh.brows, sh.rows - r0);
+    const int cpr = (int)(min(sh.bcols, sh.cols - c0) >> 3);       // chunks per row of the block's valid part
+    const int nch = rows_valid * cpr;                              // (the host checks brows * cols / 8 < 2^31)
+    const int step_r = WGS / cpr, step_c = WGS % cpr;
+    // chunk tid + j * WGS of the valid part, j = 0, 1, ...: the walk advances by WGS chunks without a division
+    auto sweep = [&](bool nt, auto&& f) {
+        int r = tid / cpr, cc = tid - r * cpr;
+        for (int64_t i = tid; i < nch; i += UN * WGS) {        // (64-bit: i + u * WGS may pass 2^31)
+            uint4 v[UN];
+            uint32_t off[UN];
+            bool ok[UN];
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                ok[u] = i + u * WGS < nch;
+                off[u] = (uint32_t)r * row_stride + (uint32_t)cc;
+                r += step_r; cc += step_c;
+                if (cc >= cpr) { cc -= cpr; ++r; }
+                if (ok[u]) v[u] = load16_rt(bin + off[u], nt);
+            }
+#pragma unroll
+            for (int u = 0; u < UN; ++u) if (ok[u]) f(v[u], off[u]);
+        }
+    };
+
+    // pass 1: amax and min over non-zero magnitudes, FQ:407-485 (packed 16-bit integer maxima / minima)
+    uint32_t amax2 = 0, amin2_m1 = AMIN2_INIT_M1;
+    sweep(false, [&](uint4 v, uint32_t) {
+        acc_amax_pk(amax2, v.x); acc_amax_pk(amax2, v.y); acc_amax_pk(amax2, v.z); acc_amax_pk(amax2, v.w);
+        if constexpr (MOR) { acc_amin_pk(amin2_m1, v.x); acc_amin_pk(amin2_m1, v.y); acc_amin_pk(amin2_m1, v.z); acc_amin_pk(amin2_m1, v.w); }
+    });
+    uint32_t amax_b = group_umax(amax_bits_of(amax2), 64);
+    uint32_t amin_m1 = AMIN_INIT_M1;
+    if constexpr (MOR) amin_m1 = group_umin(amin_m1_of(amin2_m1), 64);
+    if (lane == 0) { s_f[0][wave] = u2f(amax_b); s_u[wave] = amin_m1; }
+    __syncthreads();
+    amax_b = f2u(lds_umaxf<NW>(s_f[0]));
+    amin_m1 = lds_umin<NW>(s_u);
+    const float amax = u2f(amax_b);
+    const float amin = u2f(amin_m1 + 1u);
+
+    const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
+    // a NaN in the block, or a scale outside the range of the few-instruction arithmetic: the exact path
+    if (amax_b > 0x7F800000u || (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast))) {           // uniform over the workgroup
+        generic_block<false, false, WGS>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
+                                         sh, qa, E8, bid, s_f, s_u);
+        return;
+    }
+
+    int fmt = qa.fmt;
+    int meta_val = qa.meta_val;
+    float e4 = 0.0f, e5 = 0.0f;
+    if constexpr (MOR) {
+        int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
+        if (qt == Q_UNKNOWN) {
+            // pass 2: the two error sums, FQ:487-584.  amax > 0 here.
+            __syncthreads();                     // s_f[0] has been read by every wave
+            uint32_t codes = 0;
+            sweep(false, [&](uint4 v, uint32_t) {
+                err_pair_fast<E8>(v.x, s4, e4, e5, codes);
+                err_pair_fast<E8>(v.y, s4, e4, e5, codes);
+                err_pair_fast<E8>(v.z, s4, e4, e5, codes);
+                err_pair_fast<E8>(v.w, s4, e4, e5, codes);
+            });
+            e4 = wave_sum(e4);
+            e5 = wave_sum(e5);
+            if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+            __syncthreads();
+            e4 = lds_sum<NW>(s_f[0]);
+            e5 = lds_sum<NW>(s_f[1]);
+            if (!(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) {
+                // too close for the reciprocal-based sums to be trusted with the decision: IEEE divisions (rare)
+                const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in);
+                const int64_t bh = rows_valid, bw = min(sh.bcols, sh.cols - c0);
+                e4 = 0.0f; e5 = 0.0f;
+#pragma unroll 1
+                for (int64_t i = tid; i < bh * bw; i += WGS) {
+                    int64_t r = i / bw, c = i - r * bw;
+                    err_terms_exact<false>(bf16_one(in16[(r0 + r) * sh.cols + c0 + c]), E8, s4, s5, e4, e5);
+                }
+                e4 = wave_sum(e4);
+                e5 = wave_sum(e5);
+                __syncthreads();
+                if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+                __syncthreads();
+                e4 = lds_sum<NW>(s_f[0]);
+                e5 = lds_sum<NW>(s_f[1]);
+            }
+            qt = mor_decide_error(amax, qa.clamp, e4, e5);
+        }
+        meta_val = qt;
+        fmt = mor_fmt_of(qt);
+    }
+    if (tid == 0) {
+        if (meta && meta_val >= 0) meta[bid] = meta_val;
+        if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+    }
+    if (!out) return;
+
+    // pass 3: quantize and store, FQ:733-851 (the last read of the block: streamed when the tensor streams)
+    const bool nt_in = streams_in(sh.rows * sh.cols), nt_out = streams_out(sh.rows * sh.cols);
+    if ((fmt < 0) || !(amax > 0.0f)) {
+        if (out != in) sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, v, nt_out); });
+        return;
+    }
+    if constexpr (!E8) {
+        if (fmt == FMT_E4M3 || fmt == FMT_E5M2) {
+            const float r4 = 1.0f / s4.s;            // 1 / s5 = r4 / 128 exactly
+            if (fmt == FMT_E4M3) sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_div<FMT_E4M3>(v, s4.s, r4), nt_out); });
+            else sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_div<FMT_E5M2>(v, s5.s, r4 * 0.0078125f), nt_out); });
+            return;
+        }
+    }
+    const Scale sc = make_scale(fmax_of(fmt) / amax);
+    switch (fmt) {
+        case FMT_E4M3: sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_fast<FMT_E4M3, E8>(v, sc), nt_out); }); break;
+        case FMT_E5M2: sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_fast<FMT_E5M2, E8>(v, sc), nt_out); }); break;
+        case FMT_E3M2:
+            if constexpr (!MOR) sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_fast<FMT_E3M2, E8>(v, sc), nt_out); });
+            break;
+        default: sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_fast<FMT_E2M3, E8>(v, sc), nt_out); }); break;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Debug view: per block amax, fp32 scale, biased exponent of the scale.
 __global__ __launch_bounds__(WG) void k_block_stats(const uint16_t* __restrict__ in, Shape sh, float fmax,
                                                     float* __restrict__ amax_o, float* __restrict__ scale_o,
@@ -948,7 +1094,7 @@ static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, i
     // fewer tiles in flight keep the memory system on fewer DRAM pages at a time (16384 x 14336 MoR: 176.8 -> 170.8 us,
     // 8192^2 block E4M3: 41.4 -> 40.1 us), while a grid that fits the chip at once wants every slot (4096^2: 9.2
     // against 10.8 us).
-    const size_t dyn_lds = (NV == 8 && grid >= 4096) ? 53000 : 0;
+    const size_t dyn_lds = (NV == 8 && WGS == WG && grid >= 4096) ? 53000 : 0;
     // Tensors beyond the last-level cache: each XCD takes a band of gx / 8 block columns and walks it row by row, so
     // that the blocks sharing a DRAM page are in flight on one XCD at about the same time (16384 x 14336, 128 x 128
     // blocks: MoR 170 -> 157 us, block E4M3 166.6 -> 153.8 us; no difference at 8192^2 and below).
@@ -974,6 +1120,15 @@ static void launch_wgblock(const void* in, void* out, int32_t* meta, float* stat
     uint4* o4 = static_cast<uint4*>(out);
     int NVc = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
     bool full = (sh.rows % sh.brows == 0) && (sh.cols % sh.bcols == 0) && (nch == NVc * WG);
+    if (nch > 8 * WG) {
+        // up to 32768 / 65536 elements (rows of 28672 elements, 256 x 256 tiles): still in registers, 8 vectors per lane
+        // of 512 / 1024 threads (8192^2 in 256 x 256 tiles: block E4M3 59.5 us with a pass over the block per step)
+        const bool w512 = nch <= 8 * 512;
+        full = (sh.rows % sh.brows == 0) && (sh.cols % sh.bcols == 0) && (nch == 8 * (w512 ? 512 : 1024));
+        if (w512) launch_wgblock_nv<MOR, E8, 8, 512>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st);
+        else launch_wgblock_nv<MOR, E8, 8, 1024>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st);
+        return;
+    }
     switch (NVc) {
         case 1: launch_wgblock_nv<MOR, E8, 1>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
         case 2: launch_wgblock_nv<MOR, E8, 2>(full, grid, i4, o4, meta, stats, sh, qa, cpr, shift, st); break;
@@ -1039,7 +1194,7 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
         else launch_rowgroup<false>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
         return mor_check_launch("k_rowgroup");
     }
-    if (vec_ok && brows * (bcols / 8) <= 8 * WG) {
+    if (vec_ok && brows * (bcols / 8) <= 8 * 1024) {
         if (qa.qmode == 1) {
             if (e8) launch_wgblock<true, true>(input, output, meta, stats, sh, qa, st);
             else launch_wgblock<true, false>(input, output, meta, stats, sh, qa, st);
@@ -1048,6 +1203,20 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
             else launch_wgblock<false, false>(input, output, meta, stats, sh, qa, st);
         }
         return mor_check_launch("k_wgblock");
+    }
+    if (vec_ok) {                                   // larger blocks of whole vectors
+        const uint4* i4 = static_cast<const uint4*>(input);
+        uint4* o4 = static_cast<uint4*>(output);
+        for_slices(nblocks, [&](int64_t first, int count) {
+            if (qa.qmode == 1) {
+                if (e8) k_bigblock<true, true><<<count, BIG_WG, 0, st>>>(i4, o4, meta, stats, sh, qa, first);
+                else k_bigblock<true, false><<<count, BIG_WG, 0, st>>>(i4, o4, meta, stats, sh, qa, first);
+            } else {
+                if (e8) k_bigblock<false, true><<<count, BIG_WG, 0, st>>>(i4, o4, meta, stats, sh, qa, first);
+                else k_bigblock<false, false><<<count, BIG_WG, 0, st>>>(i4, o4, meta, stats, sh, qa, first);
+            }
+        });
+        return mor_check_launch("k_bigblock");
     }
     if (fast_ok && brows * ((bcols + 1) / 2) <= 32 * WG && brows * cols < 0x7FFFFFFFll && nblocks <= 0x7FFFFFFFll) {
         if (qa.qmode == 1) {

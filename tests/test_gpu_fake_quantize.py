@@ -107,6 +107,13 @@ SHAPES = [
     (500, 129, 100, 127),             # odd width close to the pair capacity of a workgroup
     (9000, 5, 8192, 1),               # 8192 single-element pairs: the capacity itself
     (9000, 5, 8193, 1),               # ... and one more: the generic kernel
+    (6, 32768, 1, 32768),             # 32768 elements: in the registers of 512 threads
+    (512, 768, 256, 256),             # blocks of 65536 elements: in the registers of 1024 threads
+    (300, 1032, 256, 1024),           # larger blocks: the large-block kernel (a pass over the block per step)
+    (300, 520, 256, 512),             # ... with partial last block rows and a last block column 8 elements wide
+    (5, 28672, 1, 28672),             # ... one long row per block
+    (3, 131072, 1, 131072),
+    (131, 2056, 129, 2048),           # ... an odd row count per block
 ]
 
 
@@ -187,6 +194,20 @@ def test_inplace_and_stats(G):
     assert np.array_equal(amax, wa) and np.array_equal(scale.view(np.uint32), ws.view(np.uint32)) and np.array_equal(e8, we)
 
 
+def test_large_blocks_inplace_and_stats(G):
+    a = data_gen.c4_mixture(512, 1024, seed=78)
+    x = G.to_dev_u16(a)
+    out, meta = G.fake_quantize(a, 256, 256, 1e-15, 1, 1)
+    want, wmeta, wstats = O.fake_quantize(a, 256, 256, 1e-15, 1, 1, want_stats=True)
+    assert np.array_equal(meta, wmeta)
+    assert_same(out, want, "large blocks")
+    out2, meta2 = G.fake_quantize(a, 256, 256, 1e-15, 1, 1, inplace=True, x_dev=x)
+    assert np.array_equal(meta, meta2) and np.array_equal(out, out2)
+    st = G.mor_stats(a, 256, 256, 1e-15, 1, 1)
+    assert np.array_equal(st[..., 0], wstats[..., 0]) and np.array_equal(st[..., 1], wstats[..., 1])
+    np.testing.assert_allclose(st[..., 2:], wstats[..., 2:], rtol=1e-6, atol=0)
+
+
 def test_extreme_exponents(G):
     """Blocks whose scale exponent is outside the fast-path range, bf16 denormals and the largest finite values."""
     rng = np.random.default_rng(5)
@@ -209,6 +230,16 @@ def test_extreme_exponents(G):
             want, wmeta = O.fake_quantize(wide, br, bc, 1e-15, mode, sf)
             assert np.array_equal(meta, wmeta), (br, bc, mode, sf)
             assert_same(out, want, f"extreme wide {br}x{bc} mode {mode} sf {sf}")
+    huge = np.zeros((16, 32768), np.uint16)              # rows of 32768 elements, and two of them per block
+    for r in range(16):
+        huge[r] = np.tile(a[r % 8], 128)
+    for (br, bc) in ((1, 32768), (2, 32768)):
+        for mode, sf in ((2, 1), (2, 2), (3, 1), (3, 2), (1, 1), (1, 2), (101, 2)):
+            print("extreme huge", br, bc, mode, sf, flush=True)
+            out, meta = G.fake_quantize(huge, br, bc, 1e-15, mode, sf)
+            want, wmeta = O.fake_quantize(huge, br, bc, 1e-15, mode, sf)
+            assert np.array_equal(meta, wmeta), (br, bc, mode, sf)
+            assert_same(out, want, f"extreme huge {br}x{bc} mode {mode} sf {sf}")
     for (br, bc) in ((1, 32), (1, 256), (8, 256)):
         for mode, sf in ((2, 1), (2, 2), (3, 1), (3, 2), (1, 1), (1, 2), (101, 2)):
             print("extreme", br, bc, mode, sf, flush=True)
@@ -218,7 +249,7 @@ def test_extreme_exponents(G):
             assert_same(out, want, f"extreme {br}x{bc} mode {mode} sf {sf}")
 
 
-@pytest.mark.parametrize("br,bc", [(1, 32), (128, 128), (1, 512)])
+@pytest.mark.parametrize("br,bc", [(1, 32), (128, 128), (1, 512), (128, 256)])
 @pytest.mark.parametrize("mode,sf", [(1, 1), (2, 2), (3, 1)])
 def test_nan_and_inf_elements_stay_inside_their_block(G, br, bc, mode, sf):
     """NaN / Inf inputs have no pinned reference result; what is asserted: the call completes and every block without
