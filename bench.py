@@ -231,6 +231,12 @@ def other_configs(torch, run, cabi, K, W):
     add("mor_128x128_8192x8192_normal", lambda: run.fake_quantize(x, out, meta, 128, 128, 1e-15, 1, 1), n * 4 + meta.numel() * 4, n)
     add("copy_mode7_8192x8192", lambda: run.fake_quantize(x, out, meta, 128, 128, 0.0, 7, 1), n * 4 + meta.numel() * 4, n)
     add("block_e4m3_128x128_8192x8192_fp32scale", lambda: run.fake_quantize(x, out, meta, 128, 128, 0.0, 2, 1), n * 4 + meta.numel() * 4, n)
+    # blocks beyond the 16384 elements a 256-thread workgroup keeps in registers (same 67.1 M elements)
+    add("block_e4m3_128x256_8192x8192", lambda: run.fake_quantize(x, out, meta, 128, 256, 0.0, 2, 1), n * 4, n)
+    add("block_e4m3_256x256_8192x8192", lambda: run.fake_quantize(x, out, meta, 256, 256, 0.0, 2, 1), n * 4, n)
+    add("mor_256x256_8192x8192_normal", lambda: run.fake_quantize(x, out, meta, 256, 256, 1e-15, 1, 1), n * 4, n)
+    add("per_row_e4m3_2048x32768", lambda: run.fake_quantize(x.view(2048, 32768), out.view(2048, 32768), meta, 1, 32768, 0.0, 2, 1), n * 4, n)
+    add("per_row_e4m3_512x131072", lambda: run.fake_quantize(x.view(512, 131072), out.view(512, 131072), meta, 1, 131072, 0.0, 2, 1), n * 4, n)
     # the benchmark kernel with nothing left in the 256 MB last-level cache: 6 input / output pairs (1.6 GB) in rotation
     xs6 = [x] + [x.clone() for _ in range(5)]
     os6 = [torch.empty_like(x) for _ in range(6)]
