@@ -1879,11 +1879,15 @@ __global__ __launch_bounds__(WG) void k_bs_finalize(const uint32_t* ws, int npar
 // instead of two reads.  Workgroups walk the blocks grid-stride and publish one partial each of the tensor amax, the
 // non-zero count and the error sum.  A block whose scale is outside the fast range is redone from memory with the
 // exact arithmetic.
-template <bool E8, int NV, bool FULL>
-__global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, uint32_t* ws, Shape sh, int ss_mode,
+template <bool E8, int NV, bool FULL, int WGS = WG>
+__global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, uint32_t* ws, Shape sh, int ss_mode,
                                                  int cpr, int cpr_shift, int64_t nblocks, const int32_t* meta, int phase) {
-    __shared__ float s_f[WAVES];
-    __shared__ int s_i[WAVES];
+    constexpr int NW = WGS / 64, LG = WGS == 256 ? 8 : WGS == 512 ? 9 : 10;       // waves; log2 of the workgroup size
+    __shared__ float s_f[NW];
+    __shared__ int s_i[NW];
+    // sums and maxima over the waves' LDS slots (four waves: pairwise, the order the sums have always had)
+    auto red_fsum = [&]() { if constexpr (NW == 4) return (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]); else return lds_sum<NW>(s_f); };
+    auto red_fmax = [&]() { if constexpr (NW == 4) return fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3])); else return lds_fmax<NW>(s_f); };
     // phase 0: out of place (write and publish the partials); in place the input must survive until the decision:
     // phase 1 publishes the partials without writing, phase 2 writes if the decision was E4M3 (meta[0] == 1)
     if (phase == 2 && meta[0] != 1) return;
@@ -1896,10 +1900,10 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
     cpr_shift &= 255;
     // chunk k * 256 + tid of a block is at off_k(k) + off_tid; cpr is a power of two, so off_k is uniform (no per-lane
     // index arithmetic is carried through the loop over blocks)
-    const uint32_t off_tid = cpr_shift <= 8 ? (uint32_t)(tid >> cpr_shift) * row_stride + (uint32_t)(tid & (cpr - 1)) : (uint32_t)tid;
+    const uint32_t off_tid = cpr_shift <= LG ? (uint32_t)(tid >> cpr_shift) * row_stride + (uint32_t)(tid & (cpr - 1)) : (uint32_t)tid;
     auto off_k = [&](int k) -> uint32_t {
-        return cpr_shift <= 8 ? (uint32_t)(k << (8 - cpr_shift)) * row_stride
-                              : (uint32_t)(k >> (cpr_shift - 8)) * row_stride + (uint32_t)((k & ((1 << (cpr_shift - 8)) - 1)) << 8);
+        return cpr_shift <= LG ? (uint32_t)(k << (LG - cpr_shift)) * row_stride
+                               : (uint32_t)(k >> (cpr_shift - LG)) * row_stride + (uint32_t)((k & ((1 << (cpr_shift - LG)) - 1)) << LG);
     };
     float gmax = 0.0f, err = 0.0f;
     int nnz_total = 0;
@@ -1915,7 +1919,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
         bool ok[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            ok[k] = FULL || (k * WG + tid < nch);
+            ok[k] = FULL || (k * WGS + tid < nch);
             v[k] = make_uint4(0, 0, 0, 0);
             if (ok[k]) v[k] = in[base + off_k(k) + off_tid];
         }
@@ -1947,14 +1951,14 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
         __syncthreads();                          // the previous block's readers of s_f are done
         if (lane == 0) s_f[wave] = u2f(amax_b);
         __syncthreads();
-        amax_b = max(max(f2u(s_f[0]), f2u(s_f[1])), max(f2u(s_f[2]), f2u(s_f[3])));
+        amax_b = f2u(lds_umaxf<NW>(s_f));
         float amax = u2f(amax_b);
         const bool has_nan = amax_b > 0x7F800000u;
         if (has_nan) {                            // the float maximum and the count of the reference skip a NaN (rare)
             amax = 0.0f;
             int nans = 0;
 #pragma unroll 1
-            for (int ch = tid; ch < nch; ch += WG) {              // from memory again: no second use of the registers
+            for (int ch = tid; ch < nch; ch += WGS) {              // from memory again: no second use of the registers
                 const int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
                 const uint4 x = in[base + (uint32_t)r * row_stride + (uint32_t)(ch - r * cpr)];
                 acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
@@ -1965,7 +1969,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
             __syncthreads();
             if (lane == 0) s_f[wave] = amax;
             __syncthreads();
-            amax = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+            amax = red_fmax();
         }
         gmax = fmaxf(gmax, amax);
         nnz_total += (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
@@ -2003,7 +2007,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
             uint16_t* out16 = reinterpret_cast<uint16_t*>(out);
             const int64_t e0 = by * sh.brows * sh.cols + bx * sh.bcols;
 #pragma unroll 1
-            for (int64_t i = tid; i < sh.brows * sh.bcols; i += WG) {
+            for (int64_t i = tid; i < sh.brows * sh.bcols; i += WGS) {
                 const int64_t r = i / sh.bcols, c = i - r * sh.bcols;
                 const float q = bs_element<E8, false>(bf16_one(in16[e0 + r * sh.cols + c]), sc, err);
                 if (write) out16[e0 + r * sh.cols + c] = store_bf16<false>(q);
@@ -2016,15 +2020,17 @@ __global__ __launch_bounds__(WG) void k_bs_fused(const uint4* in, uint4* out, ui
     __syncthreads();
     if (lane == 0) { s_f[wave] = err; s_i[wave] = nnz_total; }
     __syncthreads();
-    const float e = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
-    const int n = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    const float e = red_fsum();
+    int n = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) n += s_i[w];
     __syncthreads();
     if (lane == 0) s_f[wave] = gmax;
     __syncthreads();
     if (tid == 0 && phase != 2) {
         reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = e;
         reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
-        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = red_fmax();
     }
 }
 
@@ -2277,23 +2283,31 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
     // (a decision pass that computes no output words and a write pass that computes no error terms; 128 x 128 blocks
     // in place at 8192^2: 83 us against 99 through the general three-pass path; blocks that fill less than a workgroup
     // take the general path)
-    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG && blk_chunks <= 8 * WG
-        && brows * (cols / 8) < 0x7FFFFFFFll && is_pow2(bcols / 8)) {
+    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG && blk_chunks <= 8 * 1024
+        && brows * (cols / 8) < 0x7FFFFFFFll && (is_pow2(bcols / 8) || brows == 1)) {
         const int cpr = (int)(bcols / 8);
         const int nv = (int)cdiv(blk_chunks, WG);
         const int NVc = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
-        const bool full = blk_chunks == (int64_t)NVc * WG;
+        // up to 8 * 256 chunks: 256 threads; up to 32768 / 65536 elements: 8 vectors per lane of 512 / 1024 threads
+        const int wgs = blk_chunks <= 8 * WG ? WG : blk_chunks <= 8 * 512 ? 512 : 1024;
+        const bool full = blk_chunks == (int64_t)(wgs == WG ? NVc : 8) * wgs;
         const int grid = (int)std::min<int64_t>(nb, 4096);      // partials: one per workgroup (the finalize kernel reads them all)
         // tensors beyond the last-level cache: XCD bands of block columns (16384 x 14336, 128 x 128 blocks: 193 -> 185 us)
         const bool bands = rows * cols > ((int64_t)128 << 20) && sh.gx % 8 == 0 && grid % 8 == 0 && nb % 8 == 0;
-        const int shift = ilog2(cpr) | (bands ? 256 : 0);
+        // a one-row block is contiguous whatever its width: chunk k * 256 + tid is at that offset (shift 20: row 0 always)
+        const int shift = (brows == 1 ? 20 : ilog2(cpr)) | (bands ? 256 : 0);
         const uint4* i4 = static_cast<const uint4*>(input);
         uint4* o4 = static_cast<uint4*>(output);
 #define MOR_BS_FUSED(E8, NV, PHASE) do { \
         if (full) k_bs_fused<E8, NV, true><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); \
         else k_bs_fused<E8, NV, false><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); } while (0)
+#define MOR_BS_FUSED_W(E8, WGS_, PHASE) do { \
+        if (full) k_bs_fused<E8, 8, true, WGS_><<<grid, WGS_, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); \
+        else k_bs_fused<E8, 8, false, WGS_><<<grid, WGS_, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); } while (0)
 #define MOR_BS_FUSED_ALL(PHASE) do { \
-        if (ss_mode == 2) { switch (NVc) { case 1: MOR_BS_FUSED(true, 1, PHASE); break; case 2: MOR_BS_FUSED(true, 2, PHASE); break; case 4: MOR_BS_FUSED(true, 4, PHASE); break; default: MOR_BS_FUSED(true, 8, PHASE); break; } } \
+        if (wgs == 512) { if (ss_mode == 2) MOR_BS_FUSED_W(true, 512, PHASE); else MOR_BS_FUSED_W(false, 512, PHASE); } \
+        else if (wgs == 1024) { if (ss_mode == 2) MOR_BS_FUSED_W(true, 1024, PHASE); else MOR_BS_FUSED_W(false, 1024, PHASE); } \
+        else if (ss_mode == 2) { switch (NVc) { case 1: MOR_BS_FUSED(true, 1, PHASE); break; case 2: MOR_BS_FUSED(true, 2, PHASE); break; case 4: MOR_BS_FUSED(true, 4, PHASE); break; default: MOR_BS_FUSED(true, 8, PHASE); break; } } \
         else { switch (NVc) { case 1: MOR_BS_FUSED(false, 1, PHASE); break; case 2: MOR_BS_FUSED(false, 2, PHASE); break; case 4: MOR_BS_FUSED(false, 4, PHASE); break; default: MOR_BS_FUSED(false, 8, PHASE); break; } } } while (0)
         MOR_BS_FUSED_ALL(inplace ? 1 : 0);
         k_bs_finalize<<<1, WG, 0, st>>>(ws, grid, grid, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
@@ -2303,6 +2317,7 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
             k_copy_if<<<grid_for(n_all / 8, 4), WG, 0, st>>>(in16, out16, meta, 3, n_all, n_all / 8);
         }
 #undef MOR_BS_FUSED_ALL
+#undef MOR_BS_FUSED_W
 #undef MOR_BS_FUSED
         return mor_check_launch("mor_block_scaling (single pass)");
     }

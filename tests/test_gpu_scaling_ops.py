@@ -44,7 +44,14 @@ def check_scaling(G, a, br, bc, thr, ss, channel, flags=0, inplace=False):
                                    # single-pass kernel (ss_mode 2 / 3): whole rows, 128 lanes, odd chunks per row,
                                    # more blocks than partial slots
                                    (64, 4096, 1, 4096, True), (32, 2048, 1, 1024, True), (64, 240, 16, 120, False),
-                                   (9000, 1024, 1, 1024, True)])
+                                   (9000, 1024, 1, 1024, True),
+                                   # ... rows whose chunk count is no power of two (1792, 257, 384 chunks)
+                                   (24, 14336, 1, 14336, True), (40, 2056, 1, 2056, True), (64, 3072, 1, 3072, True),
+                                   # ... blocks of up to 32768 / 65536 elements (512 / 1024 threads)
+                                   (12, 28672, 1, 28672, True), (256, 512, 128, 256, False), (512, 512, 256, 256, False),
+                                   (6, 65536, 1, 65536, True), (5, 40000, 1, 40000, True),
+                                   # ... and larger ones (two reads)
+                                   (4, 131072, 1, 131072, True), (512, 1024, 512, 256, False)])
 def test_scaling_fixture_and_random(G, ss, shape):
     rows, cols, br, bc, channel = shape
     if rows == 256 and cols == 256:
@@ -75,7 +82,9 @@ def test_scaling_inplace_and_flavour(G, shape, thr):
 # 2, 4 and 8 vectors per lane, whole and ragged, and a width that is not a power of two (general path)
 @pytest.mark.parametrize("ss", [2, 3])
 @pytest.mark.parametrize("shape", [(64, 4096, 1, 4096, True), (128, 256, 64, 128, False), (256, 384, 128, 128, False),
-                                   (96, 2048, 1, 2048, True), (64, 3072, 1, 3072, True), (200, 256, 100, 128, False)])
+                                   (96, 2048, 1, 2048, True), (64, 3072, 1, 3072, True), (200, 256, 100, 128, False),
+                                   (24, 14336, 1, 14336, True), (40, 2056, 1, 2056, True),
+                                   (12, 28672, 1, 28672, True), (512, 512, 256, 256, False), (5, 40000, 1, 40000, True)])
 def test_scaling_single_pass_in_place(G, ss, shape):
     rows, cols, br, bc, channel = shape
     a = uniform_bits(rows + cols + ss, rows, cols, -300.0, 300.0)
@@ -87,7 +96,8 @@ def test_scaling_single_pass_in_place(G, ss, shape):
 
 @pytest.mark.parametrize("ss", [1, 2, 3, 4])
 @pytest.mark.parametrize("shape", [(256, 256, 128, 128, False), (64, 4096, 1, 4096, True), (64, 512, 1, 32, True),
-                                   (512, 64, 128, 1, True), (96, 80, 32, 16, False)])
+                                   (512, 64, 128, 1, True), (96, 80, 32, 16, False), (24, 14336, 1, 14336, True),
+                                   (12, 28672, 1, 28672, True), (512, 512, 256, 256, False)])
 def test_scaling_blocks_with_nan_and_inf(G, ss, shape):
     """A NaN does not become the block's amax (the reference's float maximum skips it), an infinity does; the error sum
     is NaN either way, which is not above any threshold."""
