@@ -377,6 +377,16 @@ __device__ __forceinline__ uint32_t group_umin(uint32_t v, int G) {
     if (G >= 64) v = min(v, (uint32_t)__shfl_xor((int)v, 32));
     return v;
 }
+// Sum over groups of G = 1, 2, 4, ... 64 consecutive lanes (every lane of a group gets the group's sum).
+__device__ __forceinline__ float group_sum(float v, int G) {
+    if (G >= 2) v += dpp_f<DPP_XOR1>(v);
+    if (G >= 4) v += dpp_f<DPP_XOR2>(v);
+    if (G >= 8) v += dpp_f<DPP_HALF_MIRROR>(v);
+    if (G >= 16) v += dpp_f<DPP_MIRROR>(v);
+    if (G >= 32) v += __shfl_xor(v, 16);
+    if (G >= 64) v += __shfl_xor(v, 32);
+    return v;
+}
 __device__ __forceinline__ float wave_sum(float v) {
     v += dpp_f<DPP_XOR1>(v);
     v += dpp_f<DPP_XOR2>(v);

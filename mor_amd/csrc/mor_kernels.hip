@@ -7,6 +7,8 @@
 //                32768 / 65536 elements: 512 / 1024 threads): the block lives in registers as 16-byte vectors;
 //                amax / min-nonzero / MoR error sums by DPP + LDS; the MoR decision and the quantization reuse the
 //                registers.  A variant reads and writes pairs of elements where rows cannot be read as vectors.
+//   k_subblock   blocks of fewer than 256 vectors (8x8 ... 32x32 tiles, short rows): a group of 1 ... 64 lanes per
+//                block, several blocks per wave, reductions inside the lane group.
 //   k_bigblock   larger blocks of whole vectors: one 512-thread workgroup per block, a pass over the block per step
 //                (the repeated reads come from cache).
 //   k_elementwise  current-scaling modes (the scale is an argument): flat 16-byte vectors + scalar tail.
@@ -711,6 +713,159 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     }
 }
 
+struct DivU32 {   // x / d for 32-bit x by multiply-shift (d >= 1)
+    uint32_t d, mul, shift;
+};
+static DivU32 make_div(uint32_t d) {
+    DivU32 r{d, 0, 0};
+    if (d <= 1) { r.mul = 0; r.shift = 0; return r; }
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;                       // ceil(log2 d)
+    r.mul = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    r.shift = l;
+    return r;
+}
+__device__ __forceinline__ uint32_t div_u32(uint32_t x, const DivU32& d) {
+    if (d.d <= 1) return x;
+    uint32_t t = __umulhi(x, d.mul);
+    return (t + ((x - t) >> 1)) >> (d.shift - 1);
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_subblock: blocks of fewer than 256 vectors (8 x 8 ... 32 x 32 tiles, rows of 24 ... 1536 elements, MoR on 1 x 32):
+// a group of L = 1, 2, 4 ... 64 consecutive lanes holds one block, NV <= 4 vectors per lane, so a wave works on 64 / L
+// blocks at once and a workgroup on 256 / L (one workgroup per such block would leave most of its lanes idle: 8 x 8
+// tiles of a 4096 x 6144 tensor took 354 us).  Reductions stay inside the group (DPP and shuffles, no LDS); the steps
+// are those of k_wgblock, lane groups of a wave diverging where their blocks choose different formats.  Blocks that
+// need the exact arithmetic (a NaN, a scale outside the fast range, MoR error sums too close to call) are flagged and
+// done afterwards by the whole workgroup through generic_block.
+template <bool MOR, bool E8, int NV>
+__global__ __launch_bounds__(WG) void k_subblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
+                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int L, int logL,
+                                                 int64_t first, DivU32 d_gx, DivU32 d_cpr) {
+    __shared__ float s_f[2][WAVES];
+    __shared__ uint32_t s_u[WAVES];
+    __shared__ uint32_t s_hard[WG];
+    const int tid = threadIdx.x;
+    const int g = tid >> logL, l = tid & (L - 1), groups = WG >> logL;
+    const int64_t nblocks = sh.gy * sh.gx;
+    const int64_t bid0 = (first + blockIdx.x) * groups;
+    const int64_t bid = bid0 + g;
+    const bool valid = bid < nblocks;
+    s_hard[tid] = 0;
+    __syncthreads();
+
+    const int64_t by = valid ? (int64_t)div_u32((uint32_t)bid, d_gx) : 0, bx = valid ? bid - by * sh.gx : 0;   // (fewer than 2^31 blocks)
+    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3);
+    const uint4* bin = in + (r0 * row_stride + (c0 >> 3));
+    uint4* bout = out ? out + (r0 * row_stride + (c0 >> 3)) : nullptr;
+    const int rows_valid = (int)min(sh.brows, sh.rows - r0);
+    const int cols_valid = (int)min((int64_t)cpr, (sh.cols - c0) >> 3);
+    const int nchb = (int)sh.brows * cpr;
+    const bool nt_in = streams_in(sh.rows * sh.cols), nt_out = streams_out(sh.rows * sh.cols);
+
+    uint4 v[NV];
+    uint32_t off[NV];
+    bool ok[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int j = l + k * L, r = (int)div_u32((uint32_t)j, d_cpr), cc = j - r * cpr;
+        ok[k] = valid && j < nchb && r < rows_valid && cc < cols_valid;
+        off[k] = (uint32_t)r * row_stride + (uint32_t)cc;
+        v[k] = make_uint4(0, 0, 0, 0);
+        if (ok[k]) v[k] = load16_rt(bin + off[k], nt_in);
+    }
+    // pass 1: amax and min over non-zero magnitudes, FQ:407-485 (zeros of idle lanes change neither)
+    uint32_t amax2 = 0, amin2_m1 = AMIN2_INIT_M1;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+        if constexpr (MOR) { acc_amin_pk(amin2_m1, v[k].x); acc_amin_pk(amin2_m1, v[k].y); acc_amin_pk(amin2_m1, v[k].z); acc_amin_pk(amin2_m1, v[k].w); }
+    }
+    const uint32_t amax_b = group_umax(amax_bits_of(amax2), L);
+    uint32_t amin_m1 = AMIN_INIT_M1;
+    if constexpr (MOR) amin_m1 = group_umin(amin_m1_of(amin2_m1), L);
+    const float amax = u2f(amax_b);
+    const float amin = u2f(amin_m1 + 1u);
+    const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
+    bool hard = amax_b > 0x7F800000u || (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast));
+
+    int fmt = qa.fmt;
+    int meta_val = qa.meta_val;
+    float e4 = 0.0f, e5 = 0.0f;
+    if constexpr (MOR) {
+        int qt = Q_UNKNOWN;
+        if (!hard) qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
+        // (the group sums use shuffles: every lane of the wave takes part, with zeros where its block needs no sums)
+        const bool want = valid && !hard && qt == Q_UNKNOWN;
+        uint32_t codes = 0;
+        if (want) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k)
+                if (ok[k]) {
+                    err_pair_fast<E8>(v[k].x, s4, e4, e5, codes);
+                    err_pair_fast<E8>(v[k].y, s4, e4, e5, codes);
+                    err_pair_fast<E8>(v[k].z, s4, e4, e5, codes);
+                    err_pair_fast<E8>(v[k].w, s4, e4, e5, codes);
+                }
+        }
+        e4 = group_sum(e4, L);
+        e5 = group_sum(e5, L);
+        if (want) {
+            if (!(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) hard = true;        // too close for the reciprocal-based sums
+            else qt = mor_decide_error(amax, qa.clamp, e4, e5);
+        }
+        meta_val = qt;
+        fmt = mor_fmt_of(qt);
+    }
+    if (valid && hard && l == 0) s_hard[g] = 1;
+    if (valid && !hard) {
+        if (l == 0) {
+            if (meta && meta_val >= 0) meta[bid] = meta_val;
+            if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+        }
+        // pass 3: quantize and store, FQ:733-851
+        if (out) {
+            if ((fmt < 0) || !(amax > 0.0f)) {
+                if (out != in) {
+#pragma unroll
+                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], v[k], nt_out);
+                }
+            } else if (!E8 && (fmt == FMT_E4M3 || fmt == FMT_E5M2)) {
+                const float r4 = 1.0f / s4.s;            // 1 / s5 = r4 / 128 exactly
+#pragma unroll
+                for (int k = 0; k < NV; ++k)
+                    if (ok[k]) store16_rt(bout + off[k], fmt == FMT_E4M3 ? fq_vec_div<FMT_E4M3>(v[k], s4.s, r4)
+                                                                          : fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f), nt_out);
+            } else {
+                const Scale sc = make_scale(fmax_of(fmt) / amax);
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    if (!ok[k]) continue;
+                    uint4 q;
+                    switch (fmt) {
+                        case FMT_E4M3: q = fq_vec_fast<FMT_E4M3, E8>(v[k], sc); break;
+                        case FMT_E5M2: q = fq_vec_fast<FMT_E5M2, E8>(v[k], sc); break;
+                        case FMT_E3M2: q = fq_vec_fast<FMT_E3M2, E8>(v[k], sc); break;
+                        default:       q = fq_vec_fast<FMT_E2M3, E8>(v[k], sc); break;
+                    }
+                    store16_rt(bout + off[k], q, nt_out);
+                }
+            }
+        }
+    }
+    // the flagged blocks, one after the other, by the whole workgroup (their inputs are untouched: blocks are disjoint)
+    __syncthreads();
+#pragma unroll 1
+    for (int g2 = 0; g2 < groups; ++g2) {
+        if (!s_hard[g2]) continue;                 // uniform over the workgroup
+        __syncthreads();
+        generic_block<false, false, WG>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
+                                        sh, qa, E8, bid0 + g2, s_f, s_u);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // k_bigblock: blocks of more than 16384 elements whose rows can be read as 16-byte vectors (rows of 28672 or 131072
 // elements, 256 x 256 tiles, ...).  One 512-thread workgroup per block, as the reference's one thread block per block
@@ -1156,6 +1311,27 @@ static void launch_wgblock_gather(const void* in, void* out, int32_t* meta, floa
 #undef MOR_GATHER
 }
 
+// Blocks of fewer than 256 vectors: lane groups (k_subblock).
+template <bool MOR, bool E8>
+static void launch_subblock(const void* in, void* out, int32_t* meta, float* stats, const Shape& sh, const QuantArgs& qa, hipStream_t st) {
+    const int cpr = (int)(sh.bcols / 8);
+    const int nchb = (int)sh.brows * cpr;
+    int logL = 0;
+    // vectors per lane: 4 where the group still has 8 lanes or so, else 2 (a 4096 x 6144 tensor in rows of 192 elements:
+    // 31 / 22 / 18 us with 1 / 2 / 4 vectors per lane, in 8 x 8 tiles 33 / 27 / 28 us, the plain copy 17 us)
+    const int pref = nchb >= 24 ? 4 : 2;
+    while ((1 << logL) * pref < nchb && logL < 6) ++logL;
+    const int L = 1 << logL, nv = (int)cdiv(nchb, L), groups = WG >> logL;
+    const uint4* i4 = static_cast<const uint4*>(in);
+    uint4* o4 = static_cast<uint4*>(out);
+    const DivU32 d_gx = make_div((uint32_t)sh.gx), d_cpr = make_div((uint32_t)cpr);
+    for_slices(cdiv(sh.gy * sh.gx, groups), [&](int64_t first, int count) {
+        if (nv <= 1) k_subblock<MOR, E8, 1><<<count, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, L, logL, first, d_gx, d_cpr);
+        else if (nv <= 2) k_subblock<MOR, E8, 2><<<count, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, L, logL, first, d_gx, d_cpr);
+        else k_subblock<MOR, E8, 4><<<count, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, cpr, L, logL, first, d_gx, d_cpr);
+    });
+}
+
 // Common driver of mor_fake_quantize / mor_block_format / mor_mor_stats.
 static int run_quantize(const void* input, void* output, int32_t* meta, float* stats,
                         int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
@@ -1193,6 +1369,16 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
         if (e8) launch_rowgroup<true>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
         else launch_rowgroup<false>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
         return mor_check_launch("k_rowgroup");
+    }
+    if (vec_ok && brows * (bcols / 8) < WG) {
+        if (qa.qmode == 1) {
+            if (e8) launch_subblock<true, true>(input, output, meta, stats, sh, qa, st);
+            else launch_subblock<true, false>(input, output, meta, stats, sh, qa, st);
+        } else {
+            if (e8) launch_subblock<false, true>(input, output, meta, stats, sh, qa, st);
+            else launch_subblock<false, false>(input, output, meta, stats, sh, qa, st);
+        }
+        return mor_check_launch("k_subblock");
     }
     if (vec_ok && brows * (bcols / 8) <= 8 * 1024) {
         if (qa.qmode == 1) {
@@ -1342,24 +1528,6 @@ constexpr int WS_ERR = WS_HEADER;
 constexpr int WS_PAMAX = WS_HEADER + MAX_PARTIALS;
 constexpr int WS_PNNZ = WS_HEADER + 2 * MAX_PARTIALS;
 constexpr int WS_BLOCKS = WS_HEADER + 3 * MAX_PARTIALS;
-
-struct DivU32 {   // x / d for 32-bit x by multiply-shift (d >= 1)
-    uint32_t d, mul, shift;
-};
-static DivU32 make_div(uint32_t d) {
-    DivU32 r{d, 0, 0};
-    if (d <= 1) { r.mul = 0; r.shift = 0; return r; }
-    uint32_t l = 0;
-    while ((1ull << l) < d) ++l;                       // ceil(log2 d)
-    r.mul = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
-    r.shift = l;
-    return r;
-}
-__device__ __forceinline__ uint32_t div_u32(uint32_t x, const DivU32& d) {
-    if (d.d <= 1) return x;
-    uint32_t t = __umulhi(x, d.mul);
-    return (t + ((x - t) >> 1)) >> (d.shift - 1);
-}
 
 __global__ void k_zero_f32(float* p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) p[i] = 0.0f;

@@ -107,6 +107,12 @@ SHAPES = [
     (500, 129, 100, 127),             # odd width close to the pair capacity of a workgroup
     (9000, 5, 8192, 1),               # 8192 single-element pairs: the capacity itself
     (9000, 5, 8193, 1),               # ... and one more: the generic kernel
+    (40, 96, 8, 8),                   # lane groups: 8 lanes per tile, 32 tiles per workgroup
+    (50, 200, 16, 16),                # ... 32 lanes, partial last tile row and column
+    (96, 160, 32, 32),                # ... a wave per tile, two vectors per lane
+    (30, 192, 1, 24),                 # ... 3 vectors per block in groups of 4 lanes
+    (20, 1536, 1, 1536),              # ... 192 vectors per block: 3 of 4 vector slots per lane
+    (70, 120, 2, 40),                 # ... 10 vectors per block in groups of 16 lanes
     (6, 32768, 1, 32768),             # 32768 elements: in the registers of 512 threads
     (512, 768, 256, 256),             # blocks of 65536 elements: in the registers of 1024 threads
     (300, 1032, 256, 1024),           # larger blocks: the large-block kernel (a pass over the block per step)
