@@ -1658,6 +1658,40 @@ __global__ __launch_bounds__(WG) void k_bs_amax_block(const uint16_t* in, uint32
     publish_partial(ws, gmax, nnz, s_f, s_i);
 }
 
+// The same for blocks of fewer than 256 vectors (8 x 8 ... 32 x 32 tiles, rows of 96 or 768 elements): a group of
+// L = 1 ... 64 consecutive lanes per block, as in k_subblock, 256 / L blocks per workgroup and step; the block maximum
+// by DPP / shuffles inside the group.  (One workgroup per block: 4096 x 6144 in 8 x 8 tiles 242 us for the whole op.)
+__global__ __launch_bounds__(WG) void k_bs_amax_sub(const uint4* in, uint32_t* ws, float* block_amax, Shape sh, int L, int logL,
+                                                    DivU32 d_gx, DivU32 d_cpr) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const int tid = threadIdx.x;
+    const uint32_t g = (uint32_t)(tid >> logL), l = (uint32_t)(tid & (L - 1)), groups = (uint32_t)(WG >> logL);
+    const uint32_t nb = (uint32_t)(sh.gy * sh.gx);                       // (fewer than 2^31 blocks)
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3), cpr = (uint32_t)(sh.bcols >> 3), nchb = (uint32_t)sh.brows * cpr;
+    const bool nt = streams_in(sh.rows * sh.cols);
+    float gmax = 0.0f;
+    int nnz = 0;
+    for (uint32_t b0 = blockIdx.x * groups; b0 < nb; b0 += gridDim.x * groups) {
+        const uint32_t bid = b0 + g;
+        float amax = 0.0f;
+        if (bid < nb) {
+            const uint32_t by = div_u32(bid, d_gx), bx = bid - by * (uint32_t)sh.gx;
+            const uint4* bin = in + ((int64_t)by * sh.brows * row_stride + (((int64_t)bx * sh.bcols) >> 3));
+#pragma unroll 4
+            for (uint32_t j = l; j < nchb; j += (uint32_t)L) {
+                const uint32_t r = div_u32(j, d_cpr), cc = j - r * cpr;
+                acc_amax_nnz(amax, nnz, load16_rt(bin + r * row_stride + cc, nt));
+            }
+        }
+        amax = group_max(amax, L);                   // (shuffles: every lane of the wave takes part)
+        if (bid < nb && l == 0) block_amax[bid] = amax;
+        gmax = fmaxf(gmax, amax);
+    }
+    publish_partial(ws, gmax, nnz, s_f, s_i);
+}
+
+
 // pass 1, column blocks N x 1 (FQ:1538-1610): a workgroup covers 256 adjacent columns (32 groups of 8) with 8 row
 // lanes; a thread takes every 8th row of a row segment, the 8 row lanes meet in LDS and one thread per column merges
 // into the (zero-initialised) per-block maxima with atomicMax on the bit patterns of non-negative floats.
@@ -2522,6 +2556,14 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
         const int64_t nchunks = rows * cols / 8;
         npart = (int)std::min<int64_t>(cdiv(nchunks, 8 * WG), MAX_PARTIALS);
         k_bs_amax_flat<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, blocks, nchunks, (int)G, ilog2(G));
+    } else if (vec && bcols % 8 == 0 && brows * (bcols / 8) < WG && brows * (cols / 8) < 0x7FFFFFFFll) {
+        const int nchb = (int)(brows * (bcols / 8));
+        int logL = 0;
+        while ((4 << logL) < nchb && logL < 6) ++logL;               // about four vectors per lane
+        const int groups = WG >> logL;
+        npart = (int)std::min<int64_t>(cdiv(nb, groups), MAX_PARTIALS);
+        k_bs_amax_sub<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, blocks, sh, 1 << logL, logL, make_div((uint32_t)sh.gx),
+                                            make_div((uint32_t)(bcols / 8)));
     } else {
         const int v1 = (vec && bcols % 8 == 0 && brows * (cols / 8) < 0x7FFFFFFFll) ? 1 : 0;
         npart = (int)std::min<int64_t>(nb, MAX_PARTIALS);

@@ -50,6 +50,8 @@ def check_scaling(G, a, br, bc, thr, ss, channel, flags=0, inplace=False):
                                    # ... blocks of up to 32768 / 65536 elements (512 / 1024 threads)
                                    (12, 28672, 1, 28672, True), (256, 512, 128, 256, False), (512, 512, 256, 256, False),
                                    (6, 65536, 1, 65536, True), (5, 40000, 1, 40000, True),
+                                   # ... small blocks: lane groups in the amax pass
+                                   (64, 96, 8, 8, False), (48, 192, 16, 16, False), (40, 192, 1, 96, True), (64, 160, 32, 32, False),
                                    # ... and larger ones (two reads)
                                    (4, 131072, 1, 131072, True), (512, 1024, 512, 256, False)])
 def test_scaling_fixture_and_random(G, ss, shape):
