@@ -735,7 +735,7 @@ __device__ __forceinline__ uint32_t div_u32(uint32_t x, const DivU32& d) {
 // k_subblock: blocks of fewer than 256 vectors (8 x 8 ... 32 x 32 tiles, rows of 24 ... 1536 elements, MoR on 1 x 32):
 // a group of L = 1, 2, 4 ... 64 consecutive lanes holds one block, NV <= 4 vectors per lane, so a wave works on 64 / L
 // blocks at once and a workgroup on 256 / L (one workgroup per such block would leave most of its lanes idle: 8 x 8
-// tiles of a 4096 x 6144 tensor took 354 us).  Reductions stay inside the group (DPP and shuffles, no LDS); the steps
+// tiles of a 4096 x 6144 tensor took 354 us, now 17.4 us, the time of a copy).  Reductions stay inside the group (DPP and shuffles, no LDS); the steps
 // are those of k_wgblock, lane groups of a wave diverging where their blocks choose different formats.  Blocks that
 // need the exact arithmetic (a NaN, a scale outside the fast range, MoR error sums too close to call) are flagged and
 // done afterwards by the whole workgroup through generic_block.
@@ -856,7 +856,8 @@ __global__ __launch_bounds__(WG) void k_subblock(const uint4* in, uint4* out, in
         }
     }
     // the flagged blocks, one after the other, by the whole workgroup (their inputs are untouched: blocks are disjoint)
-    __syncthreads();
+    // (most workgroups have none: one vote instead of a walk over up to 256 flags, each an LDS round trip)
+    if (!__syncthreads_or(valid && hard ? 1 : 0)) return;
 #pragma unroll 1
     for (int g2 = 0; g2 < groups; ++g2) {
         if (!s_hard[g2]) continue;                 // uniform over the workgroup
@@ -1318,7 +1319,7 @@ static void launch_subblock(const void* in, void* out, int32_t* meta, float* sta
     const int nchb = (int)sh.brows * cpr;
     int logL = 0;
     // vectors per lane: 4 where the group still has 8 lanes or so, else 2 (a 4096 x 6144 tensor in rows of 192 elements:
-    // 31 / 22 / 18 us with 1 / 2 / 4 vectors per lane, in 8 x 8 tiles 33 / 27 / 28 us, the plain copy 17 us)
+    // 29.8 / 18.9 / 17.2 us with 1 / 2 / 4 vectors per lane, in 8 x 8 tiles 21.9 / 17.4 / 18.8 us, the plain copy 17 us)
     const int pref = nchb >= 24 ? 4 : 2;
     while ((1 << logL) * pref < nchb && logL < 6) ++logL;
     const int L = 1 << logL, nv = (int)cdiv(nchb, L), groups = WG >> logL;
