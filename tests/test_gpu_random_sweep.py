@@ -32,6 +32,25 @@ def make_data(rng, rows, cols, kind):
     return t.view(torch.int16).numpy().view(np.uint16).copy()
 
 
+def fq_cases_lane_groups_and_large_blocks():
+    """Small blocks (a group of lanes per block) and blocks beyond what 256 threads hold in registers."""
+    rng = np.random.default_rng(20253)
+    blocks = [(1, 48), (1, 96), (1, 192), (1, 384), (1, 768), (1, 1536), (2, 40), (8, 16), (32, 8), (128, 8), (16, 128), (32, 64),
+              (24, 24), (128, 256), (256, 256), (1, 28672), (1, 40000), (1, 131072), (129, 2048), (512, 64), (64, 1024), (300, 512)]
+    cases = []
+    for i in range(60):
+        br, bc = blocks[rng.integers(len(blocks))]
+        exact = rng.random() < 0.5
+        ny, nx = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        rows = br * ny if exact else br * ny - int(rng.integers(0, br))
+        cols = bc * nx if exact else bc * nx - 8 * int(rng.integers(0, max(bc // 8, 1)))     # whole vectors: the vector kernels
+        rows, cols = max(rows, 1), max(cols, 8)
+        mode = int(rng.choice([1, 101, 2, 3]))
+        sf = int(rng.choice([1, 2]))
+        cases.append((100 + i, rows, cols, br, bc, mode, sf, int(rng.integers(4))))
+    return cases
+
+
 def fq_cases():
     rng = np.random.default_rng(20251)
     blocks = [(1, 8), (1, 16), (1, 32), (1, 64), (1, 128), (1, 256), (1, 512), (1, 1024), (1, 2048), (2, 64), (4, 32),
@@ -50,7 +69,7 @@ def fq_cases():
     return cases
 
 
-@pytest.mark.parametrize("case", fq_cases(), ids=lambda c: "fq%d_%dx%d_b%dx%d_m%d_s%d_k%d" % c)
+@pytest.mark.parametrize("case", fq_cases() + fq_cases_lane_groups_and_large_blocks(), ids=lambda c: "fq%d_%dx%d_b%dx%d_m%d_s%d_k%d" % c)
 def test_fake_quantize_sweep(G, case):
     i, rows, cols, br, bc, mode, sf, kind = case
     rng = np.random.default_rng(1000 + i)
@@ -87,7 +106,19 @@ def scaling_cases():
     return cases
 
 
-@pytest.mark.parametrize("case", scaling_cases(), ids=lambda c: "bs%d_%dx%d_b%dx%d_ss%d_k%d_%s_%g" % c)
+def scaling_cases_small_and_large_blocks():
+    rng = np.random.default_rng(20254)
+    blocks = [(1, 96), (1, 768), (8, 8), (16, 16), (32, 32), (1, 14336), (1, 28672), (1, 40000), (128, 256), (256, 256), (512, 256)]
+    cases = []
+    for i in range(40):
+        br, bc = blocks[rng.integers(len(blocks))]
+        ny, nx = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        cases.append((100 + i, br * ny, bc * nx, br, bc, int(rng.choice([1, 2, 3, 4])), int(rng.integers(3)), bool(rng.integers(2)),
+                      float(rng.choice([0.02, 0.045, 0.2]))))
+    return cases
+
+
+@pytest.mark.parametrize("case", scaling_cases() + scaling_cases_small_and_large_blocks(), ids=lambda c: "bs%d_%dx%d_b%dx%d_ss%d_k%d_%s_%g" % c)
 def test_scaling_sweep(G, case):
     i, rows, cols, br, bc, ss, kind, inplace, thr = case
     rng = np.random.default_rng(2000 + i)
