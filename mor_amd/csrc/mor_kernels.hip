@@ -834,23 +834,28 @@ __global__ __launch_bounds__(WG) void k_subblock(const uint4* in, uint4* out, in
                 }
             } else if (!E8 && (fmt == FMT_E4M3 || fmt == FMT_E5M2)) {
                 const float r4 = 1.0f / s4.s;            // 1 / s5 = r4 / 128 exactly
+                if (fmt == FMT_E4M3) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k)
-                    if (ok[k]) store16_rt(bout + off[k], fmt == FMT_E4M3 ? fq_vec_div<FMT_E4M3>(v[k], s4.s, r4)
-                                                                          : fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f), nt_out);
+                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_div<FMT_E4M3>(v[k], s4.s, r4), nt_out);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f), nt_out);
+                }
             } else {
                 const Scale sc = make_scale(fmax_of(fmt) / amax);
+                // (one branch per format around the loop over the vectors, not one per vector)
+                if (fmt == FMT_E4M3) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) {
-                    if (!ok[k]) continue;
-                    uint4 q;
-                    switch (fmt) {
-                        case FMT_E4M3: q = fq_vec_fast<FMT_E4M3, E8>(v[k], sc); break;
-                        case FMT_E5M2: q = fq_vec_fast<FMT_E5M2, E8>(v[k], sc); break;
-                        case FMT_E3M2: q = fq_vec_fast<FMT_E3M2, E8>(v[k], sc); break;
-                        default:       q = fq_vec_fast<FMT_E2M3, E8>(v[k], sc); break;
-                    }
-                    store16_rt(bout + off[k], q, nt_out);
+                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_fast<FMT_E4M3, E8>(v[k], sc), nt_out);
+                } else if (fmt == FMT_E5M2) {
+#pragma unroll
+                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_fast<FMT_E5M2, E8>(v[k], sc), nt_out);
+                } else if (!MOR && fmt == FMT_E3M2) {
+#pragma unroll
+                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_fast<FMT_E3M2, E8>(v[k], sc), nt_out);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_fast<FMT_E2M3, E8>(v[k], sc), nt_out);
                 }
             }
         }
