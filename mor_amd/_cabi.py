@@ -53,6 +53,13 @@ def lib():
             fn = getattr(L, name)
             fn.restype = res
             fn.argtypes = args
+        # a library built from other sources than the ones next to it must not be run silently
+        from . import build as _build
+        if os.path.exists(_build.VERSION_SRC):
+            want, have = _build.source_hash(), L.mor_version().decode()
+            if not have.endswith("src " + want):
+                raise ImportError(f"{LIB_PATH} reports '{have}' but the sources in {_build._CSRC} hash to {want}: "
+                                  "rebuild it (python -c 'import __graft_entry__ as g; g.build()')")
         _lib = L
     return _lib
 

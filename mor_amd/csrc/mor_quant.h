@@ -1,0 +1,286 @@
+// Device-side pieces shared by the fake-quantization kernels: the MoR decision, the error terms, the generic
+// one-workgroup-per-block path, and the declarations of the launchers each kernel file exports to the driver.
+// "FQ" below is the reference file mor/csrc/cuda/fake_quantize.cu.
+#pragma once
+
+#include <algorithm>
+
+#include "mor_common.h"
+
+namespace mor {
+
+
+
+// MorQuantType, FQ:600-608 (the values written to meta)
+enum : int { Q_UNKNOWN = 0, Q_E4M3 = 1, Q_E5M2 = 2, Q_BF16 = 3, Q_E2M3 = 4, Q_E4M3_SMALL = 11, Q_E5M2_SMALL = 12 };
+
+
+struct QuantArgs {
+    int qmode;        // 1 MoR, 2 fixed format (fmt), 4 current scaling (fmt, scale = clamp)
+    int fmt;          // forced format for qmode 2 / 4
+    int meta_val;     // value written to meta for qmode 2 / 4; < 0: leave meta alone
+    int dyn_range;    // MoR decision by dynamic range instead of quantization error
+    float clamp;      // clamp_threshold
+};
+
+// ------------------------------------------------------------------------------------------------
+// exact one-element quantization with run-time format / scale type (only used inside non-unrolled loops)
+template <bool EMU>
+__device__ __forceinline__ uint16_t fq_one_exact(uint16_t h, int fmt, bool e8, const Scale& sc) {
+    float x = bf16_one(h);
+    float r;
+    if (e8) {
+        switch (fmt) {
+            case FMT_E4M3: r = sqdd_exact<FMT_E4M3, true, EMU>(x, sc); break;
+            case FMT_E5M2: r = sqdd_exact<FMT_E5M2, true, EMU>(x, sc); break;
+            case FMT_E3M2: r = sqdd_exact<FMT_E3M2, true, EMU>(x, sc); break;
+            default:       r = sqdd_exact<FMT_E2M3, true, EMU>(x, sc); break;
+        }
+    } else {
+        switch (fmt) {
+            case FMT_E4M3: r = sqdd_exact<FMT_E4M3, false, EMU>(x, sc); break;
+            case FMT_E5M2: r = sqdd_exact<FMT_E5M2, false, EMU>(x, sc); break;
+            case FMT_E3M2: r = sqdd_exact<FMT_E3M2, false, EMU>(x, sc); break;
+            default:       r = sqdd_exact<FMT_E2M3, false, EMU>(x, sc); break;
+        }
+    }
+    return store_bf16<EMU>(r);
+}
+
+// FQ:610-682 without the error pass: returns Q_UNKNOWN when the error sums are needed.
+__device__ __forceinline__ int mor_decide_range(float amax, float amin, float clamp, int dyn_range) {
+    float range = 0.0f;
+    if (amax == 0.0f) { amax = clamp; range = 1.0f; }
+    if (range == 0.0f) range = amax / amin;
+    const float e4m3_range = dyn_range ? 28672.0f : 114688.0f;
+    if (range <= 7.5f) return Q_E2M3;
+    if (range <= e4m3_range) return (amax <= clamp) ? Q_E4M3_SMALL : Q_E4M3;
+    if (range <= 939524096.0f) {
+        if (dyn_range) return (amax <= clamp) ? Q_E5M2_SMALL : Q_E5M2;
+        return Q_UNKNOWN;
+    }
+    return Q_BF16;
+}
+__device__ __forceinline__ int mor_decide_error(float amax, float clamp, float e4, float e5) {
+    if (e4 <= e5) return (amax <= clamp) ? Q_E4M3_SMALL : Q_E4M3;
+    return Q_BF16;
+}
+__device__ __forceinline__ int mor_fmt_of(int qt) {
+    switch (qt) {
+        case Q_E2M3: return FMT_E2M3;
+        case Q_E4M3: case Q_E4M3_SMALL: return FMT_E4M3;
+        case Q_E5M2: case Q_E5M2_SMALL: return FMT_E5M2;
+        default: return -1;
+    }
+}
+
+// One element's two error terms with IEEE divisions, FQ:504-542.
+template <bool EMU>
+__device__ __forceinline__ void err_terms_exact(float x, bool e8, const Scale& s4, const Scale& s5, float& e4, float& e5) {
+    if (x != 0.0f) {
+        float q4 = e8 ? sqdd_exact<FMT_E4M3, true, EMU>(x, s4) : sqdd_exact<FMT_E4M3, false, EMU>(x, s4);
+        float q5 = e8 ? sqdd_exact<FMT_E5M2, true, EMU>(x, s5) : sqdd_exact<FMT_E5M2, false, EMU>(x, s5);
+        e4 += fabsf(q4 / x - 1.0f);
+        e5 += fabsf(q5 / x - 1.0f);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// quantize one packed word with an fp32 scale: |x| * s, hardware convert, divide by s, round-half-up store, sign
+template <int F> __device__ __forceinline__ uint32_t fq_pair_div(uint32_t w, float s, float r) {
+    const f32x2 c = hw_unpack2_low<F>(hw_pack2_low<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s));
+    return store_pair<false>(div_by_scale(c.x, s, r), div_by_scale(c.y, s, r)) | (w & 0x80008000u);
+}
+template <int F> __device__ __forceinline__ uint4 fq_vec_div(uint4 v, float s, float r) {
+    uint4 o;
+    o.x = fq_pair_div<F>(v.x, s, r);
+    o.y = fq_pair_div<F>(v.y, s, r);
+    o.z = fq_pair_div<F>(v.z, s, r);
+    o.w = fq_pair_div<F>(v.w, s, r);
+    return o;
+}
+
+// The two error terms of one packed word (FQ:504-542) on magnitudes; s5 = 128 * s4 exactly.
+// The reference computes |q / x - 1| with q = c / s.  E8 scale: |q - x| * (1 / x), q - x exact.  FP32 scale:
+// with y = x * s the same quantity is |c - y| / y (c - y is exact: c is within a factor 2 of y, or 0), which needs
+// neither q nor a division; for E5M2 c5 / 128 - y is one exact fma.  Each term differs from the reference's by
+// rounding errors of 1e-7 relative, of either sign, far inside the 1e-6 tolerance on the sums; decisions that would
+// depend on less than 1e-5 are recomputed with the reference's divisions by the caller.  The sums are only wanted
+// for blocks with amax / min non-zero |x| <= 939524096 (FQ:637), so a non-zero element scales to at least
+// 448 / 939524096 and no reciprocal overflows.
+// `codes` carries the register of the fp8 codes from one word to the next (the converts write half of it).
+template <bool E8>
+__device__ __forceinline__ void err_pair_fast(uint32_t w, const Scale& s4, float& e4, float& e5, uint32_t& codes) {
+    float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
+    if constexpr (E8) {
+        // q = cast(x 2^e8) 2^-e8 by the scaled converts from the packed word (a zero code gives 0 where the reference's
+        // exponent arithmetic leaves 2^(-e8-127): a difference far below the terms' rounding errors); a zero element has
+        // q = 0, so its term is 0 * min(1 / 0, FLT_MAX) = 0
+        const uint32_t mag2 = w & 0x7FFF7FFFu;
+        const f32x2 q4 = e8_pair_values<FMT_E4M3>(mag2, s4.e8), q5 = e8_pair_values<FMT_E5M2>(mag2, s4.e8 + 7);
+        const float ya = fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), yb = fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f);
+        e4 = fmaf(fabsf(q4.x - a), ya, e4);
+        e5 = fmaf(fabsf(q5.x - a), ya, e5);
+        e4 = fmaf(fabsf(q4.y - b), yb, e4);
+        e5 = fmaf(fabsf(q5.y - b), yb, e5);
+    } else {
+        // y + 2^-100 is y for every non-zero element of such a block and keeps the reciprocal of a zero element
+        // finite: its codes are 0 and c - x s = 0 (one fma, x s not rounded), so its term is 0 without a select
+        const float va = fmaf(a, s4.s, 0x1p-100f), vb = fmaf(b, s4.s, 0x1p-100f);
+        codes = hw_pack2_both(va, vb, codes);
+        const f32x2 c4 = hw_unpack2_e4m3_low(codes), c5 = hw_unpack2_e5m2_high_div128(codes);
+        const float ya = __builtin_amdgcn_rcpf(va), yb = __builtin_amdgcn_rcpf(vb);
+        e4 = fmaf(fabsf(fmaf(-a, s4.s, c4.x)), ya, e4);
+        e5 = fmaf(fabsf(fmaf(-a, s4.s, c5.x)), ya, e5);
+        e4 = fmaf(fabsf(fmaf(-b, s4.s, c4.y)), yb, e4);
+        e5 = fmaf(fabsf(fmaf(-b, s4.s, c5.y)), yb, e5);
+    }
+}
+
+// One element through the fast pair functions (the other half of the word is zero and contributes nothing).
+__device__ __forceinline__ uint16_t fq_one_fast(uint16_t h, int fmt, bool e8, const Scale& sc) {
+    const uint32_t w = h;
+    uint32_t r;
+    if (e8) {
+        switch (fmt) {
+            case FMT_E4M3: r = fq_pair_fast<FMT_E4M3, true>(w, sc); break;
+            case FMT_E5M2: r = fq_pair_fast<FMT_E5M2, true>(w, sc); break;
+            case FMT_E3M2: r = fq_pair_fast<FMT_E3M2, true>(w, sc); break;
+            default:       r = fq_pair_fast<FMT_E2M3, true>(w, sc); break;
+        }
+    } else {
+        switch (fmt) {
+            case FMT_E4M3: r = fq_pair_fast<FMT_E4M3, false>(w, sc); break;
+            case FMT_E5M2: r = fq_pair_fast<FMT_E5M2, false>(w, sc); break;
+            case FMT_E3M2: r = fq_pair_fast<FMT_E3M2, false>(w, sc); break;
+            default:       r = fq_pair_fast<FMT_E2M3, false>(w, sc); break;
+        }
+    }
+    return (uint16_t)r;
+}
+
+
+// Walks the elements tid, tid + 256, ... of a bh x bw block in row-major order and calls f(offset of the element
+// from the block's first element) without a division per element: (r, c) advance by (256 / bw, 256 % bw) with one
+// carry.
+template <int WGS = WG, class F>
+__device__ __forceinline__ void for_block_elements(int64_t bh, int64_t bw, int64_t row_pitch, int tid, F&& f) {
+    const int64_t step_r = WGS / bw, step_c = WGS % bw;
+    int64_t r = tid / bw, c = tid % bw;
+#pragma unroll 1
+    while (r < bh) {
+        f(r * row_pitch + c);
+        r += step_r;
+        c += step_c;
+        if (c >= bw) { c -= bw; ++r; }
+    }
+}
+
+// generic_block: one workgroup quantizes one block of any shape straight from memory with the exact arithmetic.
+// It is the body of k_generic and the fallback of k_wgblock for blocks outside the fast range.  FAST (k_generic, default
+// flavour): blocks whose scale is in the fast range use the few-instruction arithmetic, with the same safeguard on
+// close MoR decisions as k_wgblock.
+template <bool EMU, bool FAST = false, int WGS = WG>
+__device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out, int32_t* meta, float* stats,
+                                              const Shape& sh, const QuantArgs& qa, bool e8, int64_t bid,
+                                              float (*s_f)[WGS / 64], uint32_t* s_u, bool allow_fast = false) {
+    constexpr int NW = WGS / 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
+    const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
+    float amax = 0.0f;
+    uint32_t amin_m1 = AMIN_INIT_M1;
+    const uint16_t* bin = in + r0 * sh.cols + c0;
+    for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) {
+        uint32_t a = ((uint32_t)bin[at] << 16) & 0x7FFFFFFFu;
+        amax = fmaxf(amax, u2f(a));
+        amin_m1 = min(amin_m1, a - 1u);
+    });
+    amax = group_max(amax, 64);
+    amin_m1 = group_umin(amin_m1, 64);
+    __syncthreads();
+    if (lane == 0) { s_f[0][wave] = amax; s_u[wave] = amin_m1; }
+    __syncthreads();
+    amax = lds_fmax<NW>(s_f[0]);
+    amin_m1 = lds_umin<NW>(s_u);
+    const float amin = u2f(amin_m1 + 1u);
+
+    int fmt = qa.fmt;
+    int meta_val = qa.meta_val;
+    float e4 = 0.0f, e5 = 0.0f;
+    if (qa.qmode == 1) {
+        int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
+        if (qt == Q_UNKNOWN) {
+            const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
+            bool exact = true;
+            if constexpr (FAST && !EMU) {
+                if (allow_fast && s4.fast && s4.e8 >= -90 && s4.e8 <= 90) {
+                    uint32_t codes = 0;
+                    if (e8) for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<true>((uint32_t)bin[at], s4, e4, e5, codes); });
+                    else for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { err_pair_fast<false>((uint32_t)bin[at], s4, e4, e5, codes); });
+                    e4 = wave_sum(e4);
+                    e5 = wave_sum(e5);
+                    __syncthreads();
+                    if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+                    __syncthreads();
+                    e4 = lds_sum<NW>(s_f[0]);
+                    e5 = lds_sum<NW>(s_f[1]);
+                    exact = !(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5));       // too close: repeat with the reference's divisions
+                    if (exact) { e4 = 0.0f; e5 = 0.0f; }
+                }
+            }
+            if (exact) {
+                for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { err_terms_exact<EMU>(bf16_one(bin[at]), e8, s4, s5, e4, e5); });
+                e4 = wave_sum(e4);
+                e5 = wave_sum(e5);
+                __syncthreads();
+                if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
+                __syncthreads();
+                e4 = lds_sum<NW>(s_f[0]);
+                e5 = lds_sum<NW>(s_f[1]);
+            }
+            qt = mor_decide_error(amax, qa.clamp, e4, e5);
+        }
+        meta_val = qt;
+        fmt = mor_fmt_of(qt);
+    }
+    if (tid == 0) {
+        if (meta && meta_val >= 0) meta[bid] = meta_val;
+        if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+    }
+    if (!out) return;
+    const bool copy = (fmt < 0) || !(amax > 0.0f);
+    if (copy && out == in) return;
+    const Scale sc = make_scale(copy ? 1.0f : fmax_of(fmt) / amax);
+    uint16_t* bout = out + r0 * sh.cols + c0;
+    bool fast = false;
+    if constexpr (FAST && !EMU) fast = allow_fast && !copy && sc.fast && sc.e8 >= -90 && sc.e8 <= 90;
+    if (fast) {
+        for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { bout[at] = fq_one_fast(bin[at], fmt, e8, sc); });
+    } else {
+        for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) {
+            uint16_t h = bin[at];
+            if (!copy) h = fq_one_exact<EMU>(h, fmt, e8, sc);
+            bout[at] = h;
+        });
+    }
+}
+
+}  // namespace mor
+
+// A launch holds fewer than 2^32 threads per dimension (a larger grid wraps without an error): kernels that take one
+// workgroup per block are launched slice by slice, f(first block, blocks of the slice).
+constexpr int64_t LAUNCH_SLICE = (int64_t)1 << 22;
+template <class Fn> static void for_slices(int64_t nblocks, Fn&& f) {
+    for (int64_t first = 0; first < nblocks; first += LAUNCH_SLICE) f(first, (int)std::min(LAUNCH_SLICE, nblocks - first));
+}
+
+// Launchers of the kernels that live in files of their own (mor_wgblock.hip, mor_subblock.hip); `mor` selects the
+// per-block format decision, `e8` the power-of-two scale.
+__attribute__((visibility("hidden"))) void mor_launch_wgblock(bool mor, bool e8, bool gather, const void* in, void* out, int32_t* meta, float* stats,
+                                                              const mor::Shape& sh, const mor::QuantArgs& qa, hipStream_t st);
+__attribute__((visibility("hidden"))) void mor_launch_subblock(bool mor, bool e8, const void* in, void* out, int32_t* meta, float* stats,
+                                                               const mor::Shape& sh, const mor::QuantArgs& qa, hipStream_t st);
+__attribute__((visibility("hidden"))) void mor_launch_bigblock(bool mor, bool e8, const void* in, void* out, int32_t* meta, float* stats,
+                                                               const mor::Shape& sh, const mor::QuantArgs& qa, hipStream_t st);

@@ -1,0 +1,1139 @@
+// Block / channel scaling and e8mx kernels and their C ABI entry points for MI355X (gfx950, wave64).
+// "FQ" below is the reference file mor/csrc/cuda/fake_quantize.cu.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <algorithm>
+
+#include "mor_common.h"
+#include "mor_host.h"
+#include "../../include/mor_hip.h"
+
+// ================================================================================================
+// Block / channel scaling (FQ:951-1241, 1459-1752, host FQ:2013-2230, 2431-2660) and e8mx (FQ:1243-1428).
+//
+// Workspace layout (32-bit words): [0] tensor amax bits, [1] non-zero count, [2..3] spare, then three arrays of
+// MAX_PARTIALS per-workgroup partials (error sums of pass 2; amax and non-zero counts of pass 1), then one float
+// per block (amax, turned into the block's scale in place).  Nothing is accumulated with atomics except the
+// per-column maxima of the column kernel, so all results are independent of scheduling.
+namespace mor {
+
+constexpr int WS_HEADER = 4;
+constexpr int MAX_PARTIALS = 8192;
+constexpr int WS_ERR = WS_HEADER;
+constexpr int WS_PAMAX = WS_HEADER + MAX_PARTIALS;
+constexpr int WS_PNNZ = WS_HEADER + 2 * MAX_PARTIALS;
+constexpr int WS_BLOCKS = WS_HEADER + 3 * MAX_PARTIALS;
+
+__global__ void k_zero_f32(float* p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) p[i] = 0.0f;
+}
+
+// FQ:998-999: an element counts when |x| > 0 as floats, so a NaN does not
+__device__ __forceinline__ int nnz_word(uint32_t w) {
+    return (fabsf(bf16_lo(w)) > 0.0f) + (fabsf(bf16_hi(w)) > 0.0f);
+}
+__device__ __forceinline__ int nan_word(uint32_t w) { return ((w & 0x7FFFu) > 0x7F80u) + ((w & 0x7FFF0000u) > 0x7F800000u); }
+__device__ __forceinline__ void acc_amax_nnz(float& amax, int& nnz, uint4 v) {
+    acc_amax(amax, v.x); acc_amax(amax, v.y); acc_amax(amax, v.z); acc_amax(amax, v.w);
+    nnz += nnz_word(v.x) + nnz_word(v.y) + nnz_word(v.z) + nnz_word(v.w);
+}
+
+// one workgroup's amax / nnz -> its slot of the partial arrays; returns the workgroup amax to every thread
+__device__ __forceinline__ float publish_partial(uint32_t* ws, float amax, int nnz, float* s_f, int* s_i) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    amax = group_max(amax, 64);
+    nnz = wave_sum_i(nnz);
+    __syncthreads();
+    if (lane == 0) { s_f[wave] = amax; s_i[wave] = nnz; }
+    __syncthreads();
+    const float a = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+    if (threadIdx.x == 0) {
+        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = a;
+        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    }
+    return a;
+}
+
+// tensor amax from the pass-1 partials (every thread of the workgroup gets it)
+__device__ __forceinline__ float reduce_partial_amax(const uint32_t* ws, int npart, float* s_f) {
+    const float* pa = reinterpret_cast<const float*>(ws) + WS_PAMAX;
+    float a = 0.0f;
+#pragma unroll 8
+    for (int i = threadIdx.x; i < npart; i += WG) a = fmaxf(a, pa[i]);
+    a = group_max(a, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s_f[threadIdx.x >> 6] = a;
+    __syncthreads();
+    return fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+}
+
+// pass 1, blocks 1 x 8G as lane groups over the flat chunk array (FQ:1430-1457, 1611-1629).  A workgroup takes
+// tiles of 8 * 256 consecutive chunks, all loads of a tile in flight at once.  block_amax may be NULL (e8mx).
+__global__ __launch_bounds__(WG) void k_bs_amax_flat(const uint4* in, uint32_t* ws, float* block_amax,
+                                                     int64_t nchunks, int G, int logG) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    constexpr int NV = 8;
+    float gmax = 0.0f;
+    int nnz = 0;
+    const int64_t ntiles = (nchunks + NV * WG - 1) / (NV * WG);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t base = tile * (NV * WG) + threadIdx.x;
+        uint4 v[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            v[k] = make_uint4(0, 0, 0, 0);
+            if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_in(nchunks * 8));
+        }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int64_t c = base + k * WG;
+            float amax = 0.0f;
+            acc_amax_nnz(amax, nnz, v[k]);
+            gmax = fmaxf(gmax, amax);
+            if (block_amax) {
+                amax = group_max(amax, G);
+                if (c < nchunks && (c & (G - 1)) == 0) block_amax[c >> logG] = amax;
+            }
+        }
+    }
+    publish_partial(ws, gmax, nnz, s_f, s_i);
+}
+
+// tensor amax of an unaligned or odd-sized buffer, element by element (e8mx only needs the tensor amax)
+__global__ __launch_bounds__(WG) void k_amax_scalar(const uint16_t* in, uint32_t* ws, int64_t n) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    float amax = 0.0f;
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG)
+        amax = fmaxf(amax, fabsf(bf16_one(in[i])));
+    publish_partial(ws, amax, 0, s_f, s_i);
+}
+
+// pass 1, one workgroup per block of any shape (FQ:951-1015), blocks taken grid-stride;
+// vec: 16-byte loads (cols and bcols multiples of 8, aligned base)
+__global__ __launch_bounds__(WG) void k_bs_amax_block(const uint16_t* in, uint32_t* ws, float* block_amax, Shape sh, int vec,
+                                                      DivU32 d_gx, DivU32 d_cpr) {
+    __shared__ float s_f[WAVES];
+    __shared__ float s_b[WAVES];
+    __shared__ int s_i[WAVES];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t nb = (uint32_t)(sh.gy * sh.gx);
+    float gmax = 0.0f;
+    int nnz = 0;
+    for (uint32_t bid = blockIdx.x; bid < nb; bid += gridDim.x) {
+        const uint32_t by = div_u32(bid, d_gx), bx = bid - by * (uint32_t)sh.gx;
+        const int64_t r0 = (int64_t)by * sh.brows, c0 = (int64_t)bx * sh.bcols;
+        float amax = 0.0f;
+        if (vec) {
+            const uint32_t row_stride = (uint32_t)(sh.cols >> 3), cpr = (uint32_t)(sh.bcols >> 3);
+            const uint4* bin = reinterpret_cast<const uint4*>(in) + (r0 * row_stride + (c0 >> 3));
+            const uint32_t nch = (uint32_t)sh.brows * cpr;
+#pragma unroll 4
+            for (uint32_t i = threadIdx.x; i < nch; i += WG) {
+                const uint32_t r = div_u32(i, d_cpr), cc = i - r * cpr;
+                acc_amax_nnz(amax, nnz, load16_rt(bin + r * row_stride + cc, streams_in(sh.rows * sh.cols)));
+            }
+        } else {
+            for (int64_t i = threadIdx.x; i < sh.brows * sh.bcols; i += WG) {
+                int64_t r = i / sh.bcols, c = i - r * sh.bcols;
+                uint32_t a = ((uint32_t)in[(r0 + r) * sh.cols + c0 + c] << 16) & 0x7FFFFFFFu;
+                amax = fmaxf(amax, u2f(a));
+                nnz += (u2f(a) > 0.0f);
+            }
+        }
+        amax = group_max(amax, 64);
+        __syncthreads();
+        if (lane == 0) s_b[wave] = amax;
+        __syncthreads();
+        amax = fmaxf(fmaxf(s_b[0], s_b[1]), fmaxf(s_b[2], s_b[3]));
+        if (threadIdx.x == 0) block_amax[bid] = amax;
+        gmax = fmaxf(gmax, amax);
+    }
+    publish_partial(ws, gmax, nnz, s_f, s_i);
+}
+
+// The same for blocks of fewer than 256 vectors (8 x 8 ... 32 x 32 tiles, rows of 96 or 768 elements): a group of
+// L = 1 ... 64 consecutive lanes per block, as in k_subblock, 256 / L blocks per workgroup and step; the block maximum
+// by DPP / shuffles inside the group.  (One workgroup per block: 4096 x 6144 in 8 x 8 tiles 242 us for the whole op.)
+__global__ __launch_bounds__(WG) void k_bs_amax_sub(const uint4* in, uint32_t* ws, float* block_amax, Shape sh, int L, int logL,
+                                                    DivU32 d_gx, DivU32 d_cpr) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const int tid = threadIdx.x;
+    const uint32_t g = (uint32_t)(tid >> logL), l = (uint32_t)(tid & (L - 1)), groups = (uint32_t)(WG >> logL);
+    const uint32_t nb = (uint32_t)(sh.gy * sh.gx);                       // (fewer than 2^31 blocks)
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3), cpr = (uint32_t)(sh.bcols >> 3), nchb = (uint32_t)sh.brows * cpr;
+    const bool nt = streams_in(sh.rows * sh.cols);
+    float gmax = 0.0f;
+    int nnz = 0;
+    for (uint32_t b0 = blockIdx.x * groups; b0 < nb; b0 += gridDim.x * groups) {
+        const uint32_t bid = b0 + g;
+        float amax = 0.0f;
+        if (bid < nb) {
+            const uint32_t by = div_u32(bid, d_gx), bx = bid - by * (uint32_t)sh.gx;
+            const uint4* bin = in + ((int64_t)by * sh.brows * row_stride + (((int64_t)bx * sh.bcols) >> 3));
+#pragma unroll 4
+            for (uint32_t j = l; j < nchb; j += (uint32_t)L) {
+                const uint32_t r = div_u32(j, d_cpr), cc = j - r * cpr;
+                acc_amax_nnz(amax, nnz, load16_rt(bin + r * row_stride + cc, nt));
+            }
+        }
+        amax = group_max(amax, L);                   // (shuffles: every lane of the wave takes part)
+        if (bid < nb && l == 0) block_amax[bid] = amax;
+        gmax = fmaxf(gmax, amax);
+    }
+    publish_partial(ws, gmax, nnz, s_f, s_i);
+}
+
+
+// pass 1, column blocks N x 1 (FQ:1538-1610): a workgroup covers 256 adjacent columns (32 groups of 8) with 8 row
+// lanes; a thread takes every 8th row of a row segment, the 8 row lanes meet in LDS and one thread per column merges
+// into the (zero-initialised) per-block maxima with atomicMax on the bit patterns of non-negative floats.
+__global__ __launch_bounds__(WG) void k_bs_amax_col(const uint16_t* in, uint32_t* ws, float* block_amax, Shape sh,
+                                                    int rows_per_wg, int vec) {
+    __shared__ float s_m[8][32 * 8 + 8];
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const int cg = threadIdx.x & 31, rl = threadIdx.x >> 5;
+    const int64_t col0 = ((int64_t)blockIdx.x * 32 + cg) * 8;
+    const int64_t segs_per_block = (sh.brows + rows_per_wg - 1) / rows_per_wg;
+    const int ncol = (int)max((int64_t)0, min((int64_t)8, sh.cols - col0));
+    float gmax = 0.0f;
+    int nnz = 0;
+    // row segments of all block rows, taken grid-stride along y
+    for (int64_t seg = blockIdx.y; seg < sh.gy * segs_per_block; seg += gridDim.y) {
+        const int64_t by = seg / segs_per_block;
+        const int64_t r_begin = by * sh.brows + (seg - by * segs_per_block) * rows_per_wg;
+        const int64_t r_end = min(r_begin + rows_per_wg, (by + 1) * sh.brows);
+        float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (vec && ncol == 8) {
+            const uint4* in4 = reinterpret_cast<const uint4*>(in);
+#pragma unroll 8
+            for (int64_t r = r_begin + rl; r < r_end; r += 8) {
+                const uint4 v = load16_rt(in4 + ((r * sh.cols + col0) >> 3), streams_in(sh.rows * sh.cols));
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    m[2 * j] = fmaxf(m[2 * j], fabsf(bf16_lo(w[j])));
+                    m[2 * j + 1] = fmaxf(m[2 * j + 1], fabsf(bf16_hi(w[j])));
+                    nnz += nnz_word(w[j]);
+                }
+            }
+        } else {
+            for (int64_t r = r_begin + rl; r < r_end; r += 8)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (j < ncol) {
+                        const uint32_t a = ((uint32_t)in[r * sh.cols + col0 + j] << 16) & 0x7FFFFFFFu;
+                        m[j] = fmaxf(m[j], u2f(a));
+                        nnz += (a != 0);
+                    }
+        }
+        __syncthreads();                       // the previous segment's readers are done
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s_m[rl][cg * 8 + j] = m[j];
+        __syncthreads();
+        float cm = s_m[0][threadIdx.x];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) cm = fmaxf(cm, s_m[k][threadIdx.x]);
+        const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        if (c < sh.cols && cm > 0.0f) atomicMax(reinterpret_cast<uint32_t*>(&block_amax[by * sh.cols + c]), f2u(cm));
+        gmax = fmaxf(gmax, cm);
+    }
+    const uint32_t slot = blockIdx.x + gridDim.x * blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    gmax = group_max(gmax, 64);
+    nnz = wave_sum_i(nnz);
+    if (lane == 0) { s_f[wave] = gmax; s_i[wave] = nnz; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        reinterpret_cast<float*>(ws)[WS_PAMAX + slot] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        reinterpret_cast<int*>(ws)[WS_PNNZ + slot] = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    }
+}
+
+// FQ:1059-1093
+__device__ __forceinline__ float scaling_factor(float global_amax, float block_amax, int ss_mode) {
+    float sf = 1.0f;
+    const float fmax = 448.0f;
+    if (block_amax < 1e-35f) block_amax = 1e-35f;
+    switch (ss_mode) {
+        case 1: {
+            float ratio = fmax / global_amax;
+            uint32_t gman = f2u(ratio) & 0x007FFFFFu;
+            float bsf = fmax / block_amax;
+            uint32_t bb = f2u(bsf);
+            float adj = u2f((bb & 0xFF800000u) | gman);
+            sf = (gman <= (bb & 0x007FFFFFu)) ? adj : adj / 2.0f;
+            break;
+        }
+        case 2:
+        case 3: sf = fmax / block_amax; break;
+        case 4: if (global_amax > 0.0f) sf = fmax / global_amax; break;
+        default: break;
+    }
+    return sf;
+}
+
+// pass 1.5 (FQ:1017-1049 + the scale of every block): tensor amax and non-zero count from the partials into the
+// header, block amax -> block scale in place
+__global__ __launch_bounds__(WG) void k_bs_scales(uint32_t* ws, float* block_amax, int64_t nb, int ss_mode, int npart) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const float gamax = reduce_partial_amax(ws, npart, s_f);
+    if (blockIdx.x == 0) {
+        const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
+        int n = 0;
+#pragma unroll 8
+        for (int i = threadIdx.x; i < npart; i += WG) n += pn[i];
+        n = wave_sum_i(n);
+        if ((threadIdx.x & 63) == 0) s_i[threadIdx.x >> 6] = n;
+        __syncthreads();
+        if (threadIdx.x == 0) { ws[0] = f2u(gamax); ws[1] = (uint32_t)(s_i[0] + s_i[1] + s_i[2] + s_i[3]); }
+    }
+    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < nb; i += (int64_t)gridDim.x * WG)
+        block_amax[i] = scaling_factor(gamax, block_amax[i], ss_mode);
+}
+
+// One element of FQ:1133-1162: zeros give +0 and no error; others E4M3 through the hardware-cast model.
+// The power-of-two path is taken for ss_mode 2 (the reference tests the strategy against SF_E8 = 2, FQ:1138).
+template <bool E8, bool EMU>
+__device__ __forceinline__ float bs_element(float x, const Scale& sc, float& err) {
+    if (x == 0.0f) return EMU ? x : 0.0f;
+    float dq = sqdd_exact<FMT_E4M3, E8, EMU>(x, sc);
+    err += fabsf((dq - x) / x);
+    return dq;
+}
+// Fast version on magnitudes for scales in the fast range: hardware convert; q = c / s by a reciprocal-multiply
+// with one exact-residual correction (r = 1 / s correctly rounded, the result is then the rounded quotient);
+// error term |q - x| / x through the hardware reciprocal (relative 1e-7, tolerance on the sum 1e-6).
+// No selects: a zero element has q = 0, so its term is 0 * min(1 / 0, FLT_MAX) = 0 and its magnitude bits are 0;
+// the sign of the input is kept for non-zero halves only (zero inputs come back as +0, FQ:1133-1134), through a
+// packed 16-bit mask.
+// ERR / OUT: whether the error terms / the output word are wanted (the in-place phases need one of them each).
+template <bool E8, bool ERR = true, bool OUT = true>
+__device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, float rs, float& err) {
+    const float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
+    float qa, qb;
+    if constexpr (E8) {
+        // scaled converts from the packed word; a zero code of a non-zero element is the reference's 2^(-e8-127) for
+        // e8 < 0 (its exponent subtraction, FQ:296-303), zero inputs are skipped by the reference (FQ:1133) and stay 0
+        const f32x2 q = e8_pair_values<FMT_E4M3>(w & 0x7FFF7FFFu, sc.e8);
+        const float art = u2f(sc.e8 < 0 ? (uint32_t)(-sc.e8) << 23 : 0u);
+        qa = (a == 0.0f) ? 0.0f : fmaxf(q.x, art);
+        qb = (b == 0.0f) ? 0.0f : fmaxf(q.y, art);
+    } else {
+        const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc.s, b * sc.s));
+        qa = div_by_scale(c.x, sc.s, rs);
+        qb = div_by_scale(c.y, sc.s, rs);
+    }
+    if constexpr (ERR) {
+        const float ya = fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), yb = fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f);
+        err = fmaf(fabsf(qa - a), ya, err);
+        err = fmaf(fabsf(qb - b), yb, err);
+    }
+    if constexpr (!OUT) return 0u;
+    const uint32_t nonzero = pk_min_u16(w & 0x7FFF7FFFu, 0x00010001u);        // 1 in each half that is not +-0
+    return store_pair<false>(qa, qb) | (w & (nonzero << 15));
+}
+template <bool E8, bool ERR, bool OUT>
+__device__ __forceinline__ uint4 bs_vec_fast(uint4 v, const Scale& sc, float& err) {
+    uint4 q;
+    q.x = bs_pair_fast<E8, ERR, OUT>(v.x, sc, sc.r, err);
+    q.y = bs_pair_fast<E8, ERR, OUT>(v.y, sc, sc.r, err);
+    q.z = bs_pair_fast<E8, ERR, OUT>(v.z, sc, sc.r, err);
+    q.w = bs_pair_fast<E8, ERR, OUT>(v.w, sc, sc.r, err);
+    return q;
+}
+
+// pass 2 / pass 4: quantize every element with its block's scale (looked up per chunk, or per column in column
+// mode), accumulate the relative error, optionally write.  GATE > 0: run only if meta[0] == GATE.
+template <bool E8, bool EMU, bool COL, bool WRITE, bool ERR>
+__global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* out, uint32_t* ws, const float* scales,
+                                                 const int32_t* meta, int gate, Shape sh, int vec, DivU32 d_rowchunks,
+                                                 DivU32 d_brows, DivU32 d_bchunks, DivU32 d_bcols) {
+    __shared__ float s_f[WAVES];
+    if (gate > 0 && meta[0] != gate) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float err = 0.0f;
+    if (vec) {
+        const uint32_t row_chunks = (uint32_t)(sh.cols >> 3);
+        const uint32_t nchunks = (uint32_t)sh.rows * row_chunks;
+        const uint4* in4 = reinterpret_cast<const uint4*>(in);
+        uint4* out4 = reinterpret_cast<uint4*>(out);
+        for (uint32_t c = blockIdx.x * WG + threadIdx.x; c < nchunks; c += gridDim.x * WG) {
+            const uint32_t row = div_u32(c, d_rowchunks), cc = c - row * row_chunks;
+            const uint32_t by = div_u32(row, d_brows);
+            uint4 v = load16_rt(in4 + c, streams_in(sh.rows * sh.cols));
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            if constexpr (COL) {
+                const float* sp = scales + (int64_t)by * sh.cols + (int64_t)cc * 8;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const Scale s0 = make_scale(sp[2 * j]), s1 = make_scale(sp[2 * j + 1]);
+                    float q0 = bs_element<E8, EMU>(bf16_lo(w[j]), s0, err);
+                    float q1 = bs_element<E8, EMU>(bf16_hi(w[j]), s1, err);
+                    w[j] = store_pair<EMU>(q0, q1);
+                }
+            } else {
+                const uint32_t bx = div_u32(cc, d_bchunks);
+                const Scale sc = make_scale(scales[(int64_t)by * sh.gx + bx]);
+                if (!EMU && sc.fast && !vec_has_nan(v)) {
+                    const float rs = 1.0f / sc.s;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) w[j] = bs_pair_fast<E8, ERR, WRITE>(w[j], sc, rs, err);
+                } else {
+#pragma unroll 1
+                    for (int j = 0; j < 4; ++j) {
+                        float q0 = bs_element<E8, EMU>(bf16_lo(w[j]), sc, err);
+                        float q1 = bs_element<E8, EMU>(bf16_hi(w[j]), sc, err);
+                        w[j] = store_pair<EMU>(q0, q1);
+                    }
+                }
+            }
+            if constexpr (WRITE) store16_rt(out4 + c, make_uint4(w[0], w[1], w[2], w[3]), streams_out(sh.rows * sh.cols));
+        }
+    } else {
+        const int64_t n = sh.rows * sh.cols;
+        for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) {
+            const int64_t row = i / sh.cols, col = i - row * sh.cols;
+            const int64_t by = row / sh.brows, bx = col / sh.bcols;
+            const Scale sc = make_scale(scales[by * sh.gx + bx]);
+            float q = bs_element<E8, EMU>(bf16_one(in[i]), sc, err);
+            if constexpr (WRITE) out[i] = store_bf16<EMU>(q);
+        }
+    }
+    if constexpr (ERR) {
+        err = wave_sum(err);
+        if (lane == 0) s_f[wave] = err;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+        }
+    }
+}
+
+// pass 2 / pass 4 for column blocks N x 1 with aligned rows (the geometry of k_bs_amax_col): a thread owns 8 adjacent
+// columns over a segment of rows, so its 8 scales and their reciprocals are computed once.  Threads whose scales are
+// not all in the fast range use the exact arithmetic.
+template <bool WRITE, bool ERR>
+__global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_t* out, uint32_t* ws, const float* scales,
+                                                     const int32_t* meta, int gate, Shape sh, int rows_per_wg) {
+    __shared__ float s_f[WAVES];
+    if (gate > 0 && meta[0] != gate) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t col0 = ((int64_t)blockIdx.x * WG + threadIdx.x) * 8;
+    const int64_t segs_per_block = (sh.brows + rows_per_wg - 1) / rows_per_wg;
+    const int64_t row_stride = sh.cols >> 3;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    uint4* out4 = reinterpret_cast<uint4*>(out);
+    float err = 0.0f;
+    const bool nt = streams_out(sh.rows * sh.cols);
+    if (col0 < sh.cols) {
+        for (int64_t seg = blockIdx.y; seg < sh.gy * segs_per_block; seg += gridDim.y) {
+            const int64_t by = seg / segs_per_block;
+            const int64_t r_begin = by * sh.brows + (seg - by * segs_per_block) * rows_per_wg;
+            const int64_t r_end = min(r_begin + rows_per_wg, (by + 1) * sh.brows);
+            const float* sp = scales + by * sh.cols + col0;
+            Scale sc[8];
+            float rs[8];
+            bool fast = true;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { sc[j] = make_scale(sp[j]); rs[j] = 1.0f / sc[j].s; fast = fast && sc[j].fast; }
+            if (fast) {
+#pragma unroll 1
+                for (int64_t r = r_begin; r < r_end; r += 4) {
+                    uint4 v[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        v[k] = make_uint4(0, 0, 0, 0);
+                        if (r + k < r_end) v[k] = load16_rt(in4 + (r + k) * row_stride + (col0 >> 3), streams_in(sh.rows * sh.cols));
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+                        float row_err = 0.0f;
+                        if (vec_has_nan(v[k])) {          // a NaN among the 8 values: the exact arithmetic for this vector (rare)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                float q0 = bs_element<false, false>(bf16_lo(w[j]), sc[2 * j], row_err);
+                                float q1 = bs_element<false, false>(bf16_hi(w[j]), sc[2 * j + 1], row_err);
+                                w[j] = store_pair<false>(q0, q1);
+                            }
+                        } else
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            // as bs_pair_fast, with a scale of its own for each of the two columns of the word
+                            const float a = fabsf(bf16_lo(w[j])), b = fabsf(bf16_hi(w[j]));
+                            const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc[2 * j].s, b * sc[2 * j + 1].s));
+                            const float qa = div_by_scale(c.x, sc[2 * j].s, rs[2 * j]);
+                            const float qb = div_by_scale(c.y, sc[2 * j + 1].s, rs[2 * j + 1]);
+                            if constexpr (ERR) {
+                                row_err = fmaf(fabsf(qa - a), fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), row_err);
+                                row_err = fmaf(fabsf(qb - b), fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f), row_err);
+                            }
+                            if constexpr (WRITE) {
+                                const uint32_t nonzero = pk_min_u16(w[j] & 0x7FFF7FFFu, 0x00010001u);
+                                w[j] = store_pair<false>(qa, qb) | (w[j] & (nonzero << 15));
+                            }
+                        }
+                        err += row_err;
+                        if constexpr (WRITE) {
+                            if (r + k < r_end) store16_rt(out4 + (r + k) * row_stride + (col0 >> 3), make_uint4(w[0], w[1], w[2], w[3]), nt);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll 1
+                for (int64_t r = r_begin; r < r_end; ++r) {
+                    const uint4 v = in4[r * row_stride + (col0 >> 3)];
+                    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float s0 = sp[2 * j], s1 = sp[2 * j + 1];
+                        float q0 = bs_element<false, false>(bf16_lo(w[j]), make_scale(s0), err);
+                        float q1 = bs_element<false, false>(bf16_hi(w[j]), make_scale(s1), err);
+                        w[j] = store_pair<false>(q0, q1);
+                    }
+                    if constexpr (WRITE) out4[r * row_stride + (col0 >> 3)] = make_uint4(w[0], w[1], w[2], w[3]);
+                }
+            }
+        }
+    }
+    if constexpr (ERR) {
+        err = wave_sum(err);
+        if (lane == 0) s_f[wave] = err;
+        __syncthreads();
+        if (threadIdx.x == 0)
+            reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x + gridDim.x * blockIdx.y] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+    }
+}
+
+// pass 3 (FQ:1178-1241): total error (fixed summation order), the bf16 decision, the scalar outputs.
+// npart_stats > 0: the tensor amax and the non-zero count are still per-workgroup partials (single-pass kernel)
+// and are reduced here; otherwise they are in the header words.
+__global__ __launch_bounds__(WG) void k_bs_finalize(const uint32_t* ws, int npartials, int npart_stats, float threshold,
+                                                    int32_t* meta, float* gamax_o, int32_t* gnnz_o, float* gerr_o) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    const float* part = reinterpret_cast<const float*>(ws) + WS_ERR;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float gamax = u2f(ws[0]);
+    int gnnz = (int)ws[1];
+    float acc = 0.0f;
+    if (npart_stats > 0 && npart_stats == npartials) {
+        // the three partial arrays in one sweep, all loads of a batch in flight (three sweeps in a row were 6.4 us
+        // of one workgroup's load latency); every sum keeps the order of the separate sweeps
+        const float* pa = reinterpret_cast<const float*>(ws) + WS_PAMAX;
+        const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
+        float a = 0.0f;
+        int n = 0;
+#pragma unroll 8
+        for (int i = threadIdx.x; i < npartials; i += WG) {
+            a = fmaxf(a, pa[i]);
+            n += pn[i];
+            acc += part[i];
+        }
+        a = group_max(a, 64);
+        n = wave_sum_i(n);
+        if (lane == 0) { s_f[wave] = a; s_i[wave] = n; }
+        __syncthreads();
+        gamax = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        gnnz = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    } else {
+        if (npart_stats > 0) {
+            gamax = reduce_partial_amax(ws, npart_stats, s_f);
+            const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
+            int n = 0;
+#pragma unroll 8
+            for (int i = threadIdx.x; i < npart_stats; i += WG) n += pn[i];
+            n = wave_sum_i(n);
+            if (lane == 0) s_i[wave] = n;
+            __syncthreads();
+            gnnz = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+        }
+#pragma unroll 8
+        for (int i = threadIdx.x; i < npartials; i += WG) acc += part[i];
+    }
+    acc = wave_sum(acc);
+    __syncthreads();
+    if (lane == 0) s_f[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float gerr = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+        const float avg = gerr / (float)gnnz;        // 0 / 0 = NaN on an all-zero tensor: not above the threshold
+        meta[0] = (avg > threshold) ? 3 : 1;
+        gamax_o[0] = gamax;
+        gnnz_o[0] = gnnz;
+        gerr_o[0] = gerr;
+    }
+}
+
+// Single pass for the strategies whose scale depends on the block alone (ss_mode 2 and 3, FQ:1079-1088), out of
+// place: one workgroup per block of up to 16384 elements holds it in registers (as k_wgblock does), finds amax and
+// the non-zero count, quantizes, accumulates the relative error and stores -- one read and one write of the tensor
+// instead of two reads.  Workgroups walk the blocks grid-stride and publish one partial each of the tensor amax, the
+// non-zero count and the error sum.  A block whose scale is outside the fast range is redone from memory with the
+// exact arithmetic.
+template <bool E8, int NV, bool FULL, int WGS = WG>
+__global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, uint32_t* ws, Shape sh, int ss_mode,
+                                                 int cpr, int cpr_shift, int64_t nblocks, const int32_t* meta, int phase) {
+    constexpr int NW = WGS / 64, LG = WGS == 256 ? 8 : WGS == 512 ? 9 : 10;       // waves; log2 of the workgroup size
+    __shared__ float s_f[NW];
+    __shared__ int s_i[NW];
+    // sums and maxima over the waves' LDS slots (four waves: pairwise, the order the sums have always had)
+    auto red_fsum = [&]() { if constexpr (NW == 4) return (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]); else return lds_sum<NW>(s_f); };
+    auto red_fmax = [&]() { if constexpr (NW == 4) return fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3])); else return lds_fmax<NW>(s_f); };
+    // phase 0: out of place (write and publish the partials); in place the input must survive until the decision:
+    // phase 1 publishes the partials without writing, phase 2 writes if the decision was E4M3 (meta[0] == 1)
+    if (phase == 2 && meta[0] != 1) return;
+    const bool write = phase != 1;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3);
+    const int nch = (int)sh.brows * cpr;
+    const bool nt = streams_out(sh.rows * sh.cols);
+    const bool bands = (cpr_shift & 256) != 0;      // XCD bands of block columns, as in k_wgblock (gx and the grid multiples of 8)
+    cpr_shift &= 255;
+    // chunk k * 256 + tid of a block is at off_k(k) + off_tid; cpr is a power of two, so off_k is uniform (no per-lane
+    // index arithmetic is carried through the loop over blocks)
+    const uint32_t off_tid = cpr_shift <= LG ? (uint32_t)(tid >> cpr_shift) * row_stride + (uint32_t)(tid & (cpr - 1)) : (uint32_t)tid;
+    auto off_k = [&](int k) -> uint32_t {
+        return cpr_shift <= LG ? (uint32_t)(k << (LG - cpr_shift)) * row_stride
+                               : (uint32_t)(k >> (cpr_shift - LG)) * row_stride + (uint32_t)((k & ((1 << (cpr_shift - LG)) - 1)) << LG);
+    };
+    float gmax = 0.0f, err = 0.0f;
+    int nnz_total = 0;
+    for (int64_t t = blockIdx.x; t < nblocks; t += gridDim.x) {
+        int64_t bid = t;
+        if (bands) {
+            const int64_t xcd = t & 7, j = t >> 3, per = sh.gx >> 3, byb = j / per;
+            bid = byb * sh.gx + xcd * per + (j - byb * per);
+        }
+        const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+        const int64_t base = by * sh.brows * row_stride + ((bx * sh.bcols) >> 3);
+        uint4 v[NV];
+        bool ok[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            ok[k] = FULL || (k * WGS + tid < nch);
+            v[k] = make_uint4(0, 0, 0, 0);
+            if (ok[k]) v[k] = in[base + off_k(k) + off_tid];
+        }
+        // amax and the non-zero count.  Large blocks: on packed 16-bit magnitudes, the data staying packed in its
+        // registers from pass to pass (NV = 8: 100 registers instead of 220).  Small blocks: float maxima, whose
+        // unpacked magnitudes the quantize pass then uses again (measured faster for NV <= 2).
+        constexpr bool PACKED = NV > 2;
+        uint32_t amax_b, nnz2 = 0;
+        if constexpr (PACKED) {
+            uint32_t amax2 = 0;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+                acc_nnz_pk(nnz2, v[k].x); acc_nnz_pk(nnz2, v[k].y); acc_nnz_pk(nnz2, v[k].z); acc_nnz_pk(nnz2, v[k].w);
+                opaque(v[k]);
+            }
+            amax_b = group_umax(amax_bits_of(amax2), 64);
+        } else {
+            uint32_t amax2 = 0;
+            int nnzf = 0;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+                nnzf += nnz_word(v[k].x) + nnz_word(v[k].y) + nnz_word(v[k].z) + nnz_word(v[k].w);
+            }
+            nnz2 = (uint32_t)nnzf;
+            amax_b = group_umax(amax_bits_of(amax2), 64);
+        }
+        __syncthreads();                          // the previous block's readers of s_f are done
+        if (lane == 0) s_f[wave] = u2f(amax_b);
+        __syncthreads();
+        amax_b = f2u(lds_umaxf<NW>(s_f));
+        float amax = u2f(amax_b);
+        const bool has_nan = amax_b > 0x7F800000u;
+        if (has_nan) {                            // the float maximum and the count of the reference skip a NaN (rare)
+            amax = 0.0f;
+            int nans = 0;
+#pragma unroll 1
+            for (int ch = tid; ch < nch; ch += WGS) {              // from memory again: no second use of the registers
+                const int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
+                const uint4 x = in[base + (uint32_t)r * row_stride + (uint32_t)(ch - r * cpr)];
+                acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
+                if constexpr (PACKED) nans += nan_word(x.x) + nan_word(x.y) + nan_word(x.z) + nan_word(x.w);
+            }
+            nnz_total -= nans;                    // the packed count took them for non-zero values
+            amax = group_max(amax, 64);
+            __syncthreads();
+            if (lane == 0) s_f[wave] = amax;
+            __syncthreads();
+            amax = red_fmax();
+        }
+        gmax = fmaxf(gmax, amax);
+        nnz_total += (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
+        const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
+        if (!has_nan && (sc.fast || !(amax > 0.0f))) {          // an all-zero block gives +0 whatever its (clamped) scale is
+            // For large blocks every vector is finished before the next begins (register barriers): otherwise the
+            // compiler hoists work from all of them, and sinks the whole chain of error terms below the last store
+            // with every magnitude and quotient alive, which doubles the registers.
+            if (phase == 1) {                      // decision pass of the in-place variant: error terms only
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    if constexpr (PACKED) opaque(v[k]);
+                    bs_vec_fast<E8, true, false>(v[k], sc, err);
+                    if constexpr (PACKED) asm volatile("" : "+v"(err));
+                }
+            } else if (phase == 2) {               // write pass of the in-place variant: no error terms
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    if constexpr (PACKED) opaque(v[k]);
+                    uint4 q = bs_vec_fast<E8, false, true>(v[k], sc, err);
+                    if constexpr (PACKED) opaque(q);
+                    if (ok[k]) store16_rt(out + base + off_k(k) + off_tid, q, nt);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    if constexpr (PACKED) opaque(v[k]);
+                    uint4 q = bs_vec_fast<E8, true, true>(v[k], sc, err);
+                    if constexpr (PACKED) { opaque(q); asm volatile("" : "+v"(err)); }
+                    if (ok[k]) store16_rt(out + base + off_k(k) + off_tid, q, nt);
+                }
+            }
+        } else {
+            const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in);
+            uint16_t* out16 = reinterpret_cast<uint16_t*>(out);
+            const int64_t e0 = by * sh.brows * sh.cols + bx * sh.bcols;
+#pragma unroll 1
+            for (int64_t i = tid; i < sh.brows * sh.bcols; i += WGS) {
+                const int64_t r = i / sh.bcols, c = i - r * sh.bcols;
+                const float q = bs_element<E8, false>(bf16_one(in16[e0 + r * sh.cols + c]), sc, err);
+                if (write) out16[e0 + r * sh.cols + c] = store_bf16<false>(q);
+            }
+        }
+    }
+    err = wave_sum(err);
+    nnz_total = wave_sum_i(nnz_total);
+    gmax = group_max(gmax, 64);
+    __syncthreads();
+    if (lane == 0) { s_f[wave] = err; s_i[wave] = nnz_total; }
+    __syncthreads();
+    const float e = red_fsum();
+    int n = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) n += s_i[w];
+    __syncthreads();
+    if (lane == 0) s_f[wave] = gmax;
+    __syncthreads();
+    if (tid == 0 && phase != 2) {
+        reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = e;
+        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
+        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = red_fmax();
+    }
+}
+
+// The same single pass for row blocks of 1 x 8G elements, G <= 64 lanes (MX 1 x 32 through the channel op is G = 4):
+// the flat chunk array in tiles of 4 * 256 chunks, a block is G consecutive lanes (amax by DPP), as in k_rowgroup.
+// Groups whose scale is outside the fast range are redone from memory by a second, non-unrolled loop.
+constexpr int BS_ROWS_NV = 4;         // vectors per lane and tile (2 is not faster here: 55.9 against 54.5 us)
+template <bool E8>
+__global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* out, uint32_t* ws, int64_t nchunks, int G, int ss_mode,
+                                                      const int32_t* meta, int phase) {
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    if (phase == 2 && meta[0] != 1) return;          // phases as in k_bs_fused
+    const bool write = phase != 1;
+    constexpr int NV = BS_ROWS_NV;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool nt = streams_out(nchunks * 8);
+    float gmax = 0.0f, err = 0.0f;
+    int nnz = 0;
+    const int64_t ntiles = (nchunks + NV * WG - 1) / (NV * WG);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t base = tile * (NV * WG) + tid;
+        uint4 v[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            v[k] = make_uint4(0, 0, 0, 0);
+            if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_in(nchunks * 8));
+        }
+        uint32_t slow = 0;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int64_t c = base + k * WG;
+            float amax = 0.0f;
+            acc_amax_nnz(amax, nnz, v[k]);
+            amax = group_max(amax, G);
+            gmax = fmaxf(gmax, amax);
+            const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
+            float e = 0.0f;
+            uint4 q;
+            if (phase == 1) q = bs_vec_fast<E8, true, false>(v[k], sc, e);          // in place: decision pass,
+            else if (phase == 2) q = bs_vec_fast<E8, false, true>(v[k], sc, e);     // write pass
+            else q = bs_vec_fast<E8, true, true>(v[k], sc, e);
+            const bool has_nan = group_umax(vec_has_nan(v[k]) ? 1u : 0u, G) != 0u;          // exact arithmetic for such a block
+            if (!has_nan && (sc.fast || !(amax > 0.0f))) {      // an all-zero block gives +0 whatever its (clamped) scale is
+                err += e;
+                if (c < nchunks && write) store16_rt(out + c, q, nt);
+            } else if (c < nchunks) slow |= 1u << k;
+        }
+        if (slow) {
+#pragma unroll 1
+            for (int k = 0; k < NV; ++k) {
+                if (!((slow >> k) & 1u)) continue;              // uniform over the lanes of a group
+                const int64_t c = base + k * WG;
+                const uint4 x = in[c];
+                float amax = 0.0f;
+                acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
+                amax = group_max(amax, G);
+                const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
+                uint32_t w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    w[j] = store_pair<false>(bs_element<E8, false>(bf16_lo(w[j]), sc, err), bs_element<E8, false>(bf16_hi(w[j]), sc, err));
+                if (write) out[c] = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+    }
+    err = wave_sum(err);
+    nnz = wave_sum_i(nnz);
+    gmax = group_max(gmax, 64);
+    if (lane == 0) { s_f[wave] = err; s_i[wave] = nnz; }
+    __syncthreads();
+    const float e = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+    const int n = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    __syncthreads();
+    if (lane == 0) s_f[wave] = gmax;
+    __syncthreads();
+    if (tid == 0 && phase != 2) {
+        reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = e;
+        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
+        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+    }
+}
+
+// pass 4 for the out-of-place ops (FQ:1217-1235): copy the input over the quantized output when meta[0] == 3
+__global__ __launch_bounds__(WG) void k_copy_if(const uint16_t* in, uint16_t* out, const int32_t* meta, int gate, int64_t n, int64_t nvec) {
+    if (meta[0] != gate) return;
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    uint4* out4 = reinterpret_cast<uint4*>(out);
+    for (int64_t c = gtid; c < nvec; c += stride) out4[c] = in4[c];
+    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = in[i];
+}
+
+// FQ:1243-1327: keep MB mantissa bits by comparing the 23-bit mantissa with the reference's threshold tables
+// (on bf16 inputs they are the midpoints with ties to even; on scaled inputs, whose low 16 bits are not zero,
+// they are what they are).  Exponent 0 loses its mantissa, exponent 255 is left alone, a carry out of exponent
+// 254 saturates.
+template <int MB> __device__ __forceinline__ float quant_e8m(float v) {
+    uint32_t b = f2u(v);
+    uint32_t sign = b & 0x80000000u;
+    uint32_t e = (b >> 23) & 0xFF, m = b & 0x7FFFFFu;
+    if (e == 0) m = 0;
+    else if (e != 255) {
+        // The reference's thresholds, in units of 2^16: even j -> j*S + S/2, odd j -> j*S + S/2 - 1 with S = 2^(7-MB);
+        // k = number of thresholds below the mantissa.  With h = mantissa >> 16 plus one if any lower bit is set and
+        // u = h - S/2 this count is floor(u / S) plus one if that quotient is odd or the division leaves a remainder
+        // (nearest even on bf16 inputs, the same tables on inputs with low bits).
+        constexpr int S = 1 << (7 - MB);
+        const int u = (int)(m >> 16) + ((m & 0xFFFFu) != 0 ? 1 : 0) - S / 2;
+        const uint32_t q = (uint32_t)max(u, 0) >> (7 - MB);
+        const uint32_t k = (u < 0) ? 0u : q + (((q & 1u) | (((uint32_t)u & (S - 1)) != 0 ? 1u : 0u)));
+        if (k == (1u << MB)) {
+            m = 0; e++;
+            if (e == 255) { e = 254; m = ((1u << MB) - 1u) << (23 - MB); }
+        } else m = k << (23 - MB);
+    }
+    return u2f(sign | (e << 23) | m);
+}
+
+// FQ:1335-1359
+template <int MB> __device__ __forceinline__ float e8mx_scale(float gamax, int strategy) {
+    if (strategy != 1) return 1.0f;
+    uint32_t y = f2u(gamax);
+    uint32_t e = (y >> 23) + 1;
+    float fp_max = u2f((e << 23) | (((1u << MB) - 1u) << (23 - MB)));
+    float sf = fp_max / gamax;
+    if (sf >= 2.0f) sf /= 2.0f;
+    return sf;
+}
+
+// One element of FQ:1399-1419.  UNIT: the scale is 1 (no tensor-amax strategy), so the multiply and the divide are
+// exact no-ops.  Otherwise dq / sf is a reciprocal-multiply with one exact-residual correction (rs = 1 / sf correctly
+// rounded), which gives the rounded quotient when the operands are well inside the exponent range and the
+// significand of sf is not all ones; the IEEE division covers the rest.
+template <int MB, bool UNIT> __device__ __forceinline__ float e8mx_element(float x, float sf, float rs, bool markstein_ok) {
+    if constexpr (UNIT) {
+        return (x != 0.0f) ? quant_e8m<MB>(x) : 0.0f;
+    } else {
+        float v = x * sf;
+        float dq = 0.0f;
+        if (v != 0.0f) dq = quant_e8m<MB>(v);
+        const uint32_t e = (f2u(dq) >> 23) & 0xFF;
+        if (markstein_ok && e > 30 && e < 225) {
+            float t = dq * rs;
+            return fmaf(fmaf(-t, sf, dq), rs, t);
+        }
+        return dq / sf;
+    }
+}
+
+// FQ:1361-1428
+template <int MB, bool EMU, bool UNIT>
+__global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, const uint32_t* ws, int npart, int strategy, int64_t n, int64_t nvec) {
+    __shared__ float s_f[WAVES];
+    const float gamax = (!UNIT && strategy == 1) ? reduce_partial_amax(ws, npart, s_f) : 0.0f;
+    const float sf = UNIT ? 1.0f : e8mx_scale<MB>(gamax, strategy);
+    const float rs = 1.0f / sf;
+    const bool mk = (f2u(sf) & 0x7FFFFFu) != 0x7FFFFFu;
+    const int64_t stride = (int64_t)gridDim.x * WG;
+    const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    const uint4* in4 = reinterpret_cast<const uint4*>(in);
+    uint4* out4 = reinterpret_cast<uint4*>(out);
+    constexpr int NV = 2;                       // a workgroup takes tiles of NV * 256 consecutive 16-byte chunks
+    const int64_t ntiles = (nvec + NV * WG - 1) / (NV * WG);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t c0 = tile * (NV * WG) + threadIdx.x;
+        uint4 v[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) { v[k] = make_uint4(0, 0, 0, 0); if (c0 + k * WG < nvec) v[k] = load16_rt(in4 + c0 + k * WG, streams_in(n)); }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                w[j] = store_pair<EMU>(e8mx_element<MB, UNIT>(bf16_lo(w[j]), sf, rs, mk), e8mx_element<MB, UNIT>(bf16_hi(w[j]), sf, rs, mk));
+            if (c0 + k * WG < nvec) store16_rt(out4 + c0 + k * WG, make_uint4(w[0], w[1], w[2], w[3]), streams_out(n));
+        }
+    }
+    for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = store_bf16<EMU>(e8mx_element<MB, UNIT>(bf16_one(in[i]), sf, rs, mk));
+}
+
+}  // namespace mor
+
+using namespace mor;
+
+extern "C" size_t mor_workspace_bytes(int op, int64_t rows, int64_t cols, int64_t brows, int64_t bcols) {
+    if (rows <= 0 || cols <= 0 || brows <= 0 || bcols <= 0) return 0;
+    switch (op) {
+        case MOR_OP_BLOCK_SCALING:
+        case MOR_OP_CHANNEL_SCALING:
+            return (size_t)(WS_BLOCKS + cdiv(rows, brows) * cdiv(cols, bcols)) * 4;
+        case MOR_OP_E8MX:
+            return (size_t)WS_BLOCKS * 4;
+        default:
+            return 0;
+    }
+}
+
+template <bool E8, bool EMU, bool COL>
+static void launch_bs_quant(bool write, bool err, int grid, hipStream_t st, const uint16_t* in, uint16_t* out, uint32_t* ws,
+                            const float* scales, const int32_t* meta, int gate, const Shape& sh, int vec,
+                            DivU32 d0, DivU32 d1, DivU32 d2, DivU32 d3) {
+    if (write && err) k_bs_quant<E8, EMU, COL, true, true><<<grid, WG, 0, st>>>(in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3);
+    else if (write) k_bs_quant<E8, EMU, COL, true, false><<<grid, WG, 0, st>>>(in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3);
+    else k_bs_quant<E8, EMU, COL, false, true><<<grid, WG, 0, st>>>(in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3);
+}
+
+static void dispatch_bs_quant(bool e8, bool emu, bool col, bool write, bool err, int grid, hipStream_t st, const uint16_t* in,
+                              uint16_t* out, uint32_t* ws, const float* scales, const int32_t* meta, int gate, const Shape& sh,
+                              int vec, DivU32 d0, DivU32 d1, DivU32 d2, DivU32 d3) {
+#define BSQ(E8, EMU, COL) launch_bs_quant<E8, EMU, COL>(write, err, grid, st, in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3)
+    if (e8) {
+        if (emu) { if (col) BSQ(true, true, true); else BSQ(true, true, false); }
+        else { if (col) BSQ(true, false, true); else BSQ(true, false, false); }
+    } else {
+        if (emu) { if (col) BSQ(false, true, true); else BSQ(false, true, false); }
+        else { if (col) BSQ(false, false, true); else BSQ(false, false, false); }
+    }
+#undef BSQ
+}
+
+extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
+                                 float* global_amax, int32_t* global_non_zero, float* global_error,
+                                 int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                                 double e4m3_threshold, int64_t ss_mode, int channel,
+                                 void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+    if (int rc = mor_validate_shape(input, rows, cols, brows, bcols)) return rc;
+    if (!output || !meta || !global_amax || !global_non_zero || !global_error) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
+    if (rows % brows != 0 || cols % bcols != 0)      // FQ:2019-2020, 2437-2438
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "block dims %lld x %lld do not divide the tensor %lld x %lld", (long long)brows, (long long)bcols, (long long)rows, (long long)cols);
+    if (ss_mode < 1 || ss_mode > 4) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "ss_mode must be 1..4 (got %lld)", (long long)ss_mode);
+    if (channel && brows != 1 && bcols != 1)         // FQ:2501
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "channel scaling needs block_rows == 1 or block_cols == 1");
+    if (rows * cols >= (1ll << 34)) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor too large");
+    const size_t need = mor_workspace_bytes(MOR_OP_BLOCK_SCALING, rows, cols, brows, bcols);
+    if (!workspace || workspace_bytes < need) return mor_fail(MOR_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
+    Shape sh{rows, cols, brows, bcols, rows / brows, cols / bcols};
+    const int64_t nb = sh.gy * sh.gx;
+    uint32_t* ws = static_cast<uint32_t*>(workspace);
+    float* blocks = reinterpret_cast<float*>(ws + WS_BLOCKS);
+    const uint16_t* in16 = static_cast<const uint16_t*>(input);
+    uint16_t* out16 = static_cast<uint16_t*>(output);
+    const bool inplace = (input == output);
+    const int vec = (aligned16(input) && aligned16(output) && cols % 8 == 0) ? 1 : 0;
+    const bool col = (bcols == 1 && brows > 1);
+
+    // block-local scales: one pass out of place; in place one pass for the decision and one gated pass that writes
+    const int64_t blk_chunks = (bcols % 8 == 0) ? brows * (bcols / 8) : 0;
+    // (a decision pass that computes no output words and a write pass that computes no error terms; 128 x 128 blocks
+    // in place at 8192^2: 83 us against 99 through the general three-pass path; blocks that fill less than a workgroup
+    // take the general path)
+    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG && blk_chunks <= 8 * 1024
+        && brows * (cols / 8) < 0x7FFFFFFFll && (is_pow2(bcols / 8) || brows == 1)) {
+        const int cpr = (int)(bcols / 8);
+        const int nv = (int)cdiv(blk_chunks, WG);
+        const int NVc = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
+        // up to 8 * 256 chunks: 256 threads; up to 32768 / 65536 elements: 8 vectors per lane of 512 / 1024 threads
+        const int wgs = blk_chunks <= 8 * WG ? WG : blk_chunks <= 8 * 512 ? 512 : 1024;
+        const bool full = blk_chunks == (int64_t)(wgs == WG ? NVc : 8) * wgs;
+        const int grid = (int)std::min<int64_t>(nb, 4096);      // partials: one per workgroup (the finalize kernel reads them all)
+        // tensors beyond the last-level cache: XCD bands of block columns (16384 x 14336, 128 x 128 blocks: 193 -> 185 us)
+        const bool bands = rows * cols > ((int64_t)128 << 20) && sh.gx % 8 == 0 && grid % 8 == 0 && nb % 8 == 0;
+        // a one-row block is contiguous whatever its width: chunk k * 256 + tid is at that offset (shift 20: row 0 always)
+        const int shift = (brows == 1 ? 20 : ilog2(cpr)) | (bands ? 256 : 0);
+        const uint4* i4 = static_cast<const uint4*>(input);
+        uint4* o4 = static_cast<uint4*>(output);
+#define MOR_BS_FUSED(E8, NV, PHASE) do { \
+        if (full) k_bs_fused<E8, NV, true><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); \
+        else k_bs_fused<E8, NV, false><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); } while (0)
+#define MOR_BS_FUSED_W(E8, WGS_, PHASE) do { \
+        if (full) k_bs_fused<E8, 8, true, WGS_><<<grid, WGS_, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); \
+        else k_bs_fused<E8, 8, false, WGS_><<<grid, WGS_, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); } while (0)
+#define MOR_BS_FUSED_ALL(PHASE) do { \
+        if (wgs == 512) { if (ss_mode == 2) MOR_BS_FUSED_W(true, 512, PHASE); else MOR_BS_FUSED_W(false, 512, PHASE); } \
+        else if (wgs == 1024) { if (ss_mode == 2) MOR_BS_FUSED_W(true, 1024, PHASE); else MOR_BS_FUSED_W(false, 1024, PHASE); } \
+        else if (ss_mode == 2) { switch (NVc) { case 1: MOR_BS_FUSED(true, 1, PHASE); break; case 2: MOR_BS_FUSED(true, 2, PHASE); break; case 4: MOR_BS_FUSED(true, 4, PHASE); break; default: MOR_BS_FUSED(true, 8, PHASE); break; } } \
+        else { switch (NVc) { case 1: MOR_BS_FUSED(false, 1, PHASE); break; case 2: MOR_BS_FUSED(false, 2, PHASE); break; case 4: MOR_BS_FUSED(false, 4, PHASE); break; default: MOR_BS_FUSED(false, 8, PHASE); break; } } } while (0)
+        MOR_BS_FUSED_ALL(inplace ? 1 : 0);
+        k_bs_finalize<<<1, WG, 0, st>>>(ws, grid, grid, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        if (inplace) MOR_BS_FUSED_ALL(2);
+        else {
+            const int64_t n_all = rows * cols;
+            k_copy_if<<<grid_for(n_all / 8, 4), WG, 0, st>>>(in16, out16, meta, 3, n_all, n_all / 8);
+        }
+#undef MOR_BS_FUSED_ALL
+#undef MOR_BS_FUSED_W
+#undef MOR_BS_FUSED
+        return mor_check_launch("mor_block_scaling (single pass)");
+    }
+
+    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && brows == 1 && bcols % 8 == 0 && is_pow2(bcols / 8)
+        && bcols / 8 <= 64) {
+        const int64_t nchunks = rows * cols / 8;
+        const int grid = (int)std::min<int64_t>(cdiv(nchunks, BS_ROWS_NV * WG), MAX_PARTIALS);
+        const uint4* i4 = static_cast<const uint4*>(input);
+        uint4* o4 = static_cast<uint4*>(output);
+        const int G = (int)(bcols / 8);
+        for (int phase = inplace ? 1 : 0; phase <= (inplace ? 2 : 0); ++phase) {
+            if (ss_mode == 2) k_bs_fused_rows<true><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, G, (int)ss_mode, meta, phase);
+            else k_bs_fused_rows<false><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, G, (int)ss_mode, meta, phase);
+            if (phase != 2) k_bs_finalize<<<1, WG, 0, st>>>(ws, grid, grid, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        }
+        if (!inplace) k_copy_if<<<grid_for(nchunks, 4), WG, 0, st>>>(in16, out16, meta, 3, rows * cols, nchunks);
+        return mor_check_launch("mor_block_scaling (single pass, row blocks)");
+    }
+
+    // pass 1: per-block amax, per-workgroup partials of the tensor amax and the non-zero count
+    const int64_t G = bcols / 8;
+    int npart;
+    if (col) {
+        k_zero_f32<<<grid_for(nb), WG, 0, st>>>(blocks, nb);
+        const int rows_per_wg = (int)std::min<int64_t>(brows, 256);
+        const unsigned gx = (unsigned)cdiv(cols, 256);
+        const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
+        if ((int64_t)gx > MAX_PARTIALS) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many columns (%lld)", (long long)cols);
+        const unsigned gy = (unsigned)std::min<int64_t>(segs, std::max<int64_t>(MAX_PARTIALS / gx, 1));
+        npart = (int)(gx * gy);
+        k_bs_amax_col<<<dim3(gx, gy), WG, 0, st>>>(in16, ws, blocks, sh, rows_per_wg, vec);
+    } else if (vec && brows == 1 && bcols % 8 == 0 && is_pow2(G) && G <= 64) {
+        const int64_t nchunks = rows * cols / 8;
+        npart = (int)std::min<int64_t>(cdiv(nchunks, 8 * WG), MAX_PARTIALS);
+        k_bs_amax_flat<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, blocks, nchunks, (int)G, ilog2(G));
+    } else if (vec && bcols % 8 == 0 && brows * (bcols / 8) < WG && brows * (cols / 8) < 0x7FFFFFFFll) {
+        const int nchb = (int)(brows * (bcols / 8));
+        int logL = 0;
+        while ((4 << logL) < nchb && logL < 6) ++logL;               // about four vectors per lane
+        const int groups = WG >> logL;
+        npart = (int)std::min<int64_t>(cdiv(nb, groups), MAX_PARTIALS);
+        k_bs_amax_sub<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, blocks, sh, 1 << logL, logL, make_div((uint32_t)sh.gx),
+                                            make_div((uint32_t)(bcols / 8)));
+    } else {
+        const int v1 = (vec && bcols % 8 == 0 && brows * (cols / 8) < 0x7FFFFFFFll) ? 1 : 0;
+        npart = (int)std::min<int64_t>(nb, MAX_PARTIALS);
+        k_bs_amax_block<<<npart, WG, 0, st>>>(in16, ws, blocks, sh, v1, make_div((uint32_t)sh.gx),
+                                              make_div((uint32_t)std::max<int64_t>(bcols / 8, 1)));
+    }
+    // pass 1.5: tensor amax and non-zero count into the header, block scales
+    k_bs_scales<<<(int)std::min<int64_t>(cdiv(nb, WG), 256), WG, 0, st>>>(ws, blocks, nb, (int)ss_mode, npart);
+    // pass 2: quantize (out of place: write now; in place: error only), error partials
+    // pass 3: decision and scalars
+    // pass 4: bf16 fallback (out of place: copy if meta == 3) or the quantized write (in place: only if meta == 1)
+    const bool e8 = (ss_mode == 2);
+    const int64_t n = rows * cols;
+    if (col && vec && !emu && !e8) {
+        const int rows_per_wg = (int)std::min<int64_t>(brows, 16);
+        const unsigned gx = (unsigned)cdiv(cdiv(cols, 8), WG);
+        const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
+        const dim3 grid(gx, (unsigned)std::min<int64_t>(segs, std::max<int64_t>(MAX_PARTIALS / gx, 1)));
+        if (inplace) k_bs_quant_col<false, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 0, sh, rows_per_wg);
+        else k_bs_quant_col<true, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 0, sh, rows_per_wg);
+        k_bs_finalize<<<1, WG, 0, st>>>(ws, (int)(grid.x * grid.y), 0, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        if (inplace) k_bs_quant_col<true, false><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 1, sh, rows_per_wg);
+    } else {
+        const bool vec2 = vec && (col || bcols % 8 == 0) && n / 8 < 0xFFFFFFFFll;
+        const int64_t work = vec2 ? n / 8 : n;
+        const int grid2 = (int)std::min<int64_t>(std::max<int64_t>(cdiv(work, WG), 1), MAX_PARTIALS);
+        DivU32 d0 = make_div((uint32_t)std::max<int64_t>(cols / 8, 1)), d1 = make_div((uint32_t)brows),
+               d2 = make_div((uint32_t)std::max<int64_t>(bcols / 8, 1)), d3 = make_div((uint32_t)bcols);
+        dispatch_bs_quant(e8, emu, col, !inplace, true, grid2, st, in16, out16, ws, blocks, meta, 0, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
+        k_bs_finalize<<<1, WG, 0, st>>>(ws, grid2, 0, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+        if (inplace) dispatch_bs_quant(e8, emu, col, true, false, grid2, st, in16, out16, ws, blocks, meta, 1, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
+    }
+    if (!inplace) {
+        const int64_t nvec = vec ? n / 8 : 0;
+        k_copy_if<<<grid_for(nvec > 0 ? nvec : n, 4), WG, 0, st>>>(in16, out16, meta, 3, n, nvec);
+    }
+    return mor_check_launch("mor_block_scaling");
+}
+
+extern "C" int mor_e8mx(const void* input, void* output, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                        int64_t quantize_type, int64_t scaling_strategy, void* workspace, size_t workspace_bytes,
+                        uint32_t flags, void* stream) {
+    if (int rc = mor_validate_shape(input, rows, cols, brows, bcols)) return rc;
+    if (!output) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output is NULL");
+    if (quantize_type < 1 || quantize_type > 3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "quantize_type must be 1..3 (got %lld)", (long long)quantize_type);
+    const size_t need = mor_workspace_bytes(MOR_OP_E8MX, rows, cols, brows, bcols);
+    if (!workspace || workspace_bytes < need) return mor_fail(MOR_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
+    uint32_t* ws = static_cast<uint32_t*>(workspace);
+    const uint16_t* in16 = static_cast<const uint16_t*>(input);
+    uint16_t* out16 = static_cast<uint16_t*>(output);
+    const int64_t n = rows * cols;
+    const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
+    const int grid = nvec > 0 ? (int)std::min<int64_t>(cdiv(nvec, 2 * WG), 1 << 20) : grid_for(n, 16);
+    const int strategy = (int)scaling_strategy;
+    int npart = 0;
+    if (strategy == 1) {
+        if (nvec > 0 && nvec * 8 == n) {
+            npart = (int)std::min<int64_t>(cdiv(nvec, 8 * WG), 1024);
+            k_bs_amax_flat<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, nullptr, nvec, 1, 0);
+        } else {
+            npart = (int)std::min<int64_t>(cdiv(n, WG), 1024);
+            k_amax_scalar<<<npart, WG, 0, st>>>(in16, ws, n);
+        }
+    }
+#define E8MX(MB) do { \
+        if (strategy != 1) { if (emu) k_e8mx<MB, true, true><<<grid, WG, 0, st>>>(in16, out16, ws, npart, strategy, n, nvec); \
+                             else k_e8mx<MB, false, true><<<grid, WG, 0, st>>>(in16, out16, ws, npart, strategy, n, nvec); } \
+        else { if (emu) k_e8mx<MB, true, false><<<grid, WG, 0, st>>>(in16, out16, ws, npart, strategy, n, nvec); \
+               else k_e8mx<MB, false, false><<<grid, WG, 0, st>>>(in16, out16, ws, npart, strategy, n, nvec); } } while (0)
+    if (quantize_type == 1) E8MX(1); else if (quantize_type == 2) E8MX(2); else E8MX(3);
+#undef E8MX
+    return mor_check_launch("mor_e8mx");
+}

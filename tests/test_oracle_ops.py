@@ -158,12 +158,12 @@ def test_block_modes_vs_emulation(fmt, mode, e8):
 
 
 def test_block_scaling_fixture_e4m3():
-    """test_fake_quantize_block_scaling.py:100-135: meta 1, amax/nnz equal torch's, error within 1e-3, output equal."""
+    """test_fake_quantize_block_scaling.py:100-135: meta 1, amax/nnz equal torch's, error within 1e-6 of a float64 sum (the reference asserts 1e-3), output equal."""
     a = E.fixture_words(256, 256)
     out, meta, gamax, gnnz, gerr = O.block_scaling(a, 128, 128, 0.045, 1)
     emu, total, amax, nnz = E.block_scaling_tensor(a, 128, 128)
     assert meta[0] == 1 and gamax[0] == amax and gnnz[0] == nnz
-    assert abs(gerr[0] - total) <= 1e-5 * total
+    assert abs(gerr[0] - total) <= 1e-6 * total
     assert np.array_equal(out, emu)
 
 
@@ -173,7 +173,7 @@ def test_block_scaling_fixture_bf16_fallback():
     out, meta, gamax, gnnz, gerr = O.block_scaling(a, 128, 128, 0.045, 1)
     _, total, amax, nnz = E.block_scaling_tensor(a, 128, 128)
     assert meta[0] == 3 and gamax[0] == amax and gnnz[0] == nnz
-    assert abs(gerr[0] - total) <= 1e-5 * total
+    assert abs(gerr[0] - total) <= 1e-6 * total
     assert np.array_equal(out, a)
 
 
@@ -186,7 +186,7 @@ def test_block_and_channel_scaling_random(lo, hi, seed, shape):
     out, meta, gamax, gnnz, gerr = O.block_scaling(a, br, bc, 0.045, 1, channel=channel, flavour=O.EMU)
     emu, total, amax, nnz = E.block_scaling_tensor(a, br, bc)
     assert gamax[0] == amax and gnnz[0] == nnz
-    assert abs(gerr[0] - total) <= 1e-5 * total
+    assert abs(gerr[0] - total) <= 1e-6 * total
     want_meta = 3 if gerr[0] / gnnz[0] > 0.045 else 1
     assert meta[0] == want_meta
     assert np.array_equal(out, emu if want_meta == 1 else a)
