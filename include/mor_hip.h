@@ -103,6 +103,23 @@ MOR_API int mor_block_scaling(const void* input, void* output, int32_t* meta,
                       double e4m3_threshold, int64_t ss_mode, int channel,
                       void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
 
+/*
+ * mor_block_scaling without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
+ * launchers allocate three temporaries per call (FQ:2069-2078).  The workspace is a static device array inside the
+ * library, MOR_STATIC_MAX_BLOCKS * 4 + 98320 bytes on each GPU the library runs on, kept until the process ends; the
+ * entry point calls no allocating routine.  Tensors of more than MOR_STATIC_MAX_BLOCKS blocks are refused with
+ * MOR_ERR_WORKSPACE.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two host
+ * threads) race.  The first call on a GPU looks the array's address up (hipGetSymbolAddress); make that call outside a
+ * graph capture.  Results are those of mor_block_scaling, bit for bit.
+ */
+#define MOR_STATIC_MAX_BLOCKS (1 << 20)
+MOR_API int mor_block_scaling_static(const void* input, void* output, int32_t* meta,
+                             float* global_amax, int32_t* global_non_zero, float* global_error,
+                             int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
+                             double e4m3_threshold, int64_t ss_mode, int channel,
+                             uint32_t flags, void* stream);
+
 /* fake_quantize_e8mx(_inplace): FQ:2232-2397.  quantize_type 1/2/3 = E8M1/2/3;
  * scaling_strategy 1 = scale by the tensor amax, else no scale.  output may alias input. */
 MOR_API int mor_e8mx(const void* input, void* output, int64_t rows, int64_t cols,

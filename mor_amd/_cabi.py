@@ -24,6 +24,7 @@ SIGNATURES = {
     "mor_fake_quantize": (_int, [_vp, _vp, _i32p, _i64, _i64, _i64, _i64, _f64, _i64, _i64, _u32, _vp]),
     "mor_block_format": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _i64, _u32, _vp]),
     "mor_block_scaling": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f64, _i64, _int, _vp, _sz, _u32, _vp]),
+    "mor_block_scaling_static": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f64, _i64, _int, _u32, _vp]),
     "mor_e8mx": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _sz, _u32, _vp]),
     "mor_quant_dequant": (_int, [_vp, _vp, _i64, _int, _vp]),
     "mor_e4m3_with_e8_scale": (_int, [_vp, _vp, _i64, _int, _vp]),

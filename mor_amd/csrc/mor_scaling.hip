@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <algorithm>
+#include <atomic>
 
 #include "mor_common.h"
 #include "mor_host.h"
@@ -951,11 +952,10 @@ static void dispatch_bs_quant(bool e8, bool emu, bool col, bool write, bool err,
 #undef BSQ
 }
 
-extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
-                                 float* global_amax, int32_t* global_non_zero, float* global_error,
-                                 int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
-                                 double e4m3_threshold, int64_t ss_mode, int channel,
-                                 void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+// Argument checks of the block / channel scaling entry points (FQ:2019-2020, 2437-2438, 2501).
+static int block_scaling_check(const void* input, void* output, int32_t* meta, float* global_amax, int32_t* global_non_zero,
+                               float* global_error, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                               int64_t ss_mode, int channel) {
     if (int rc = mor_validate_shape(input, rows, cols, brows, bcols)) return rc;
     if (!output || !meta || !global_amax || !global_non_zero || !global_error) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
     if (rows % brows != 0 || cols % bcols != 0)      // FQ:2019-2020, 2437-2438
@@ -964,8 +964,31 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
     if (channel && brows != 1 && bcols != 1)         // FQ:2501
         return mor_fail(MOR_ERR_INVALID_ARGUMENT, "channel scaling needs block_rows == 1 or block_cols == 1");
     if (rows * cols >= (1ll << 34)) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor too large");
+    return MOR_OK;
+}
+
+static int block_scaling_run(const void* input, void* output, int32_t* meta,
+                             float* global_amax, int32_t* global_non_zero, float* global_error,
+                             int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                             double e4m3_threshold, int64_t ss_mode, void* workspace, uint32_t flags, void* stream);
+
+extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
+                                 float* global_amax, int32_t* global_non_zero, float* global_error,
+                                 int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                                 double e4m3_threshold, int64_t ss_mode, int channel,
+                                 void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+    if (int rc = block_scaling_check(input, output, meta, global_amax, global_non_zero, global_error, rows, cols, brows, bcols, ss_mode, channel)) return rc;
     const size_t need = mor_workspace_bytes(MOR_OP_BLOCK_SCALING, rows, cols, brows, bcols);
     if (!workspace || workspace_bytes < need) return mor_fail(MOR_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    return block_scaling_run(input, output, meta, global_amax, global_non_zero, global_error, rows, cols, brows, bcols,
+                             e4m3_threshold, ss_mode, workspace, flags, stream);
+}
+
+// The launches of mor_block_scaling; `workspace` holds at least mor_workspace_bytes(MOR_OP_BLOCK_SCALING, ...) bytes.
+static int block_scaling_run(const void* input, void* output, int32_t* meta,
+                             float* global_amax, int32_t* global_non_zero, float* global_error,
+                             int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                             double e4m3_threshold, int64_t ss_mode, void* workspace, uint32_t flags, void* stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
     Shape sh{rows, cols, brows, bcols, rows / brows, cols / bcols};
@@ -1099,6 +1122,50 @@ extern "C" int mor_block_scaling(const void* input, void* output, int32_t* meta,
         k_copy_if<<<grid_for(nvec > 0 ? nvec : n, 4), WG, 0, st>>>(in16, out16, meta, 3, n, nvec);
     }
     return mor_check_launch("mor_block_scaling");
+}
+
+// ------------------------------------------------------------------------------------------------
+// mor_block_scaling_static: the same op for callers that cannot allocate (and so cannot bring a workspace).  The
+// workspace is this file-scope device array, one copy per GPU, held until the process ends: the header, the three
+// partial arrays and one float for each of up to MOR_STATIC_MAX_BLOCKS blocks.  Calls on one GPU share it, so calls that
+// overlap on one GPU race; every word a call reads was written by a kernel of that call (the general path clears the
+// per-column maxima with a fill kernel), so stale contents of an earlier call are never read.
+constexpr size_t STATIC_SCRATCH_WORDS = (size_t)WS_BLOCKS + (size_t)MOR_STATIC_MAX_BLOCKS;
+static __device__ __align__(256) uint32_t scratch[STATIC_SCRATCH_WORDS];
+
+// The device address of `scratch` on the current GPU.  In host code the array's name is only a handle: the address a
+// kernel can use comes from hipGetSymbolAddress, once per device with that device current, and is kept per device.
+constexpr int STATIC_MAX_DEVICES = 64;
+static std::atomic<void*> g_scratch_ptr[STATIC_MAX_DEVICES];
+static int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return mor_fail(MOR_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "device %d out of range", dev);
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return mor_fail(MOR_ERR_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+        g_scratch_ptr[dev].store(p, std::memory_order_release);      // (two threads racing here store the same address)
+    }
+    *out = p;
+    return MOR_OK;
+}
+
+extern "C" int mor_block_scaling_static(const void* input, void* output, int32_t* meta,
+                                        float* global_amax, int32_t* global_non_zero, float* global_error,
+                                        int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
+                                        double e4m3_threshold, int64_t ss_mode, int channel,
+                                        uint32_t flags, void* stream) {
+    if (int rc = block_scaling_check(input, output, meta, global_amax, global_non_zero, global_error, rows, cols, brows, bcols, ss_mode, channel)) return rc;
+    const int64_t nb = (rows / brows) * (cols / bcols);
+    if (nb > (int64_t)MOR_STATIC_MAX_BLOCKS)
+        return mor_fail(MOR_ERR_WORKSPACE, "mor_block_scaling_static takes at most %lld blocks (got %lld): use mor_block_scaling with a workspace",
+                        (long long)MOR_STATIC_MAX_BLOCKS, (long long)nb);
+    void* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    return block_scaling_run(input, output, meta, global_amax, global_non_zero, global_error, rows, cols, brows, bcols,
+                             e4m3_threshold, ss_mode, ws, flags, stream);
 }
 
 extern "C" int mor_e8mx(const void* input, void* output, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
