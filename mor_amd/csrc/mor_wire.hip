@@ -696,11 +696,16 @@ extern "C" int mor_fake_quantize_dual(const void* input, void* output_rows, int3
     return mor_check_launch("k_fq_dual");
 }
 
+namespace mor {
+__global__ void k_wire_zero_u64(unsigned long long* p, int n) {
+    if ((int)threadIdx.x < n) p[threadIdx.x] = 0ull;
+}
+}  // namespace mor
+
 extern "C" int mor_selftest_hw_wire(uint64_t* mismatches, void* stream) {
     if (!mismatches) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mismatches is NULL");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = hipMemsetAsync(mismatches, 0, 4 * sizeof(uint64_t), st);
-    if (e != hipSuccess) return mor_fail(MOR_ERR_LAUNCH, "hipMemsetAsync: %s", hipGetErrorString(e));
+    k_wire_zero_u64<<<1, 64, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches), 4);       // (a fill kernel: capturable in a HIP graph)
     const unsigned grid = (2048u * 253u + WWG - 1) / WWG;
     k_selftest_hw_fp6<FMT_E2M3><<<grid, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));
     k_selftest_hw_fp6<FMT_E3M2><<<grid, WWG, 0, st>>>(reinterpret_cast<unsigned long long*>(mismatches));

@@ -15,7 +15,9 @@
 
 namespace {
 
-uint32_t g_flags = MOR_FLAG_DEFAULT;      // set through mor_torch_set_flags (mor.ops.set_flavour)
+// set through mor_torch_set_flags (mor.ops.set_flavour); per host thread, so that a thread that switches the flavour
+// for a debugging session does not change the results of the others
+thread_local uint32_t g_flags = MOR_FLAG_DEFAULT;
 
 void check(int rc) { TORCH_CHECK(rc == 0, "mor_hip: ", mor_last_error()); }
 
@@ -160,7 +162,7 @@ at::Tensor e8mx_autograd(const at::Tensor& input, int64_t dim_x, int64_t dim_y, 
 
 }  // namespace
 
-// mor.ops.set_flavour: MOR_FLAG_* bits for every later call
+// mor.ops.set_flavour: MOR_FLAG_* bits for every later call of the calling thread
 extern "C" __attribute__((visibility("default"))) void mor_torch_set_flags(uint32_t flags) { g_flags = flags; }
 
 TORCH_LIBRARY_IMPL(mor, CUDA, m) {

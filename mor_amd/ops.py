@@ -11,6 +11,7 @@ Differences from the reference, all of them relaxations:
   * an all-zero tensor does not trap in the block / channel scaling ops (FQ:1047).
 There is no CPU implementation, as in the reference: CPU tensors are rejected by the dispatcher.
 """
+import threading
 from typing import List
 
 import torch
@@ -30,17 +31,23 @@ __all__ = [
 _L = _cabi.lib()          # raises ImportError when the HIP library has not been built
 
 # Which of the reference's two behaviours the ops return: 0 = its CUDA kernel (default), 1 = its torch emulation.
-_flags = _cabi.FLAG_DEFAULT
+# The setting is per host thread (here and in the C++ registrations), so switching it in one thread does not change
+# what the ops return in another.
+class _Flavour(threading.local):
+    flags = _cabi.FLAG_DEFAULT
+
+
+_flavour = _Flavour()
 
 
 def set_flavour(name: str) -> None:
     """'kernel' (default): bit-compatible with the reference CUDA kernel.  'torch_emulation': bit-compatible with
-    the PyTorch emulation in the reference's tests (nearest-even store, true zeros).  A debugging aid."""
-    global _flags
-    _flags = {"kernel": _cabi.FLAG_DEFAULT, "torch_emulation": _cabi.FLAG_TORCH_EMULATION,
-              "software_cast": _cabi.FLAG_SOFTWARE_CAST}[name]
+    the PyTorch emulation in the reference's tests (nearest-even store, true zeros).  A debugging aid; it applies to
+    the calling thread's later calls only."""
+    _flavour.flags = {"kernel": _cabi.FLAG_DEFAULT, "torch_emulation": _cabi.FLAG_TORCH_EMULATION,
+                      "software_cast": _cabi.FLAG_SOFTWARE_CAST}[name]
     if _native is not None:
-        _native.mor_torch_set_flags(_flags)
+        _native.mor_torch_set_flags(_flavour.flags)
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -117,7 +124,7 @@ def _fake_quantize_impl(input, dim_x, dim_y, block_x, block_y, clamp_threshold, 
         out = torch.empty_like(x)
         meta = torch.empty((_cdiv(dim_x, block_x), _cdiv(dim_y, block_y)), dtype=torch.int32, device=x.device)
         _cabi.check(_L.mor_fake_quantize(x.data_ptr(), out.data_ptr(), meta.data_ptr(), dim_x, dim_y, block_x, block_y,
-                                         clamp_threshold, mode, sf_type, _flags, _stream(x)))
+                                         clamp_threshold, mode, sf_type, _flavour.flags, _stream(x)))
     return [out, meta]
 
 
@@ -129,7 +136,7 @@ def _fake_quantize_no_alloc_impl(input, dim_x, dim_y, block_x, block_y, clamp_th
     with _on_device(x.device):
         meta = torch.empty((_cdiv(dim_x, block_x), _cdiv(dim_y, block_y)), dtype=torch.int32, device=x.device)
         _cabi.check(_L.mor_fake_quantize(x.data_ptr(), result.data_ptr(), meta.data_ptr(), dim_x, dim_y, block_x, block_y,
-                                         clamp_threshold, mode, sf_type, _flags, _stream(x)))
+                                         clamp_threshold, mode, sf_type, _flavour.flags, _stream(x)))
     return meta
 
 
@@ -151,7 +158,7 @@ def _scaling_impl(input, dim_x, dim_y, block_x, block_y, e4m3_threshold, ss_mode
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         _cabi.check(_L.mor_block_scaling(x.data_ptr(), out.data_ptr(), meta.data_ptr(), gamax.data_ptr(), gnnz.data_ptr(),
                                          gerr.data_ptr(), dim_x, dim_y, block_x, block_y, e4m3_threshold, ss_mode,
-                                         1 if channel else 0, ws.data_ptr(), nbytes, _flags, _stream(x)))
+                                         1 if channel else 0, ws.data_ptr(), nbytes, _flavour.flags, _stream(x)))
         if inplace and x.data_ptr() != input.data_ptr():
             input.copy_(x)            # a non-contiguous input was quantized through a contiguous copy
     return [meta, gamax, gnnz, gerr] if inplace else [out, meta, gamax, gnnz, gerr]
@@ -168,7 +175,7 @@ def _e8mx_impl(input, dim_x, dim_y, block_x, block_y, quantize_type, scaling_str
         nbytes = _L.mor_workspace_bytes(_cabi.OP_E8MX, dim_x, dim_y, block_x, block_y)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         _cabi.check(_L.mor_e8mx(x.data_ptr(), out.data_ptr(), dim_x, dim_y, block_x, block_y, quantize_type, scaling_strategy,
-                                ws.data_ptr(), nbytes, _flags, _stream(x)))
+                                ws.data_ptr(), nbytes, _flavour.flags, _stream(x)))
     return out
 
 
@@ -259,13 +266,13 @@ def _fake_like(i):
 
 torch.library.register_fake("mor::fake_quantize")(
     lambda i, x, y, bx, by, c, m, s: [_fake_like(i), _fake_meta(i, bx, by, x, y)])
-torch.library.register_fake("mor::fake_quantize_no_alloc")(
-    lambda i, x, y, bx, by, c, m, s, result: _fake_meta(i, bx, by, x, y))
 for _name in ("fake_quantize_block_scaling", "fake_quantize_channel_scaling"):
     torch.library.register_fake(f"mor::{_name}")(lambda i, x, y, bx, by, t, s: [_fake_like(i)] + _fake_scalars(i))
-    torch.library.register_fake(f"mor::{_name}_inplace")(lambda i, x, y, bx, by, t, s: _fake_scalars(i))
 torch.library.register_fake("mor::fake_quantize_e8mx")(lambda i, x, y, bx, by, q, s: _fake_like(i))
-torch.library.register_fake("mor::fake_quantize_e8mx_inplace")(lambda i, x, y, bx, by, q, s, result: None)
+# The ops that write into an argument (fake_quantize_no_alloc, the *_inplace ops) get no fake kernel: their schemas,
+# kept verbatim from the reference, declare no aliasing, so a tracing compiler would take them for pure functions and
+# could drop or reorder the writes.  Their Python entry points below are excluded from compilation instead
+# (torch.compiler.disable: a graph break, the op runs eagerly and its results are right).
 for _name in ("quant_dequant_e4m3", "quant_dequant_e5m2", "quant_dequant_e3m2", "quant_dequant_e2m3",
               "e4m3_with_e8_scale_rne", "e4m3_with_e8_scale_rz"):
     torch.library.register_fake(f"mor::{_name}")(lambda i, x, y, bx, by: _fake_like(i))
@@ -291,6 +298,7 @@ def fake_quantize(a: Tensor, dim_x: int, dim_y: int, block_x: int, block_y: int,
     return torch.ops.mor.fake_quantize.default(a, dim_x, dim_y, block_x, block_y, clamp_threshold, mode, sf_type)
 
 
+@torch.compiler.disable
 def fake_quantize_no_alloc(a: Tensor, dim_x: int, dim_y: int, block_x: int, block_y: int, clamp_threshold: float, mode: int, sf_type: int, output: Tensor) -> Tensor:
     """Quantize the input bf16 Tensor into the given output tensor (which may be the input).  Returns meta."""
     return torch.ops.mor.fake_quantize_no_alloc.default(a, dim_x, dim_y, block_x, block_y, clamp_threshold, mode, sf_type, output)
@@ -301,6 +309,7 @@ def fake_quantize_block_scaling(a: Tensor, dim_x: int, dim_y: int, block_x: int,
     return torch.ops.mor.fake_quantize_block_scaling.default(a, dim_x, dim_y, block_x, block_y, e4m3_threshold, ss_mode)
 
 
+@torch.compiler.disable
 def fake_quantize_block_scaling_inplace(a: Tensor, dim_x: int, dim_y: int, block_x: int, block_y: int, e4m3_threshold: float, ss_mode: int) -> List[Tensor]:
     """As fake_quantize_block_scaling, overwriting a.  Returns [meta, global_amax, global_non_zero, global_error]."""
     return torch.ops.mor.fake_quantize_block_scaling_inplace.default(a, dim_x, dim_y, block_x, block_y, e4m3_threshold, ss_mode)
@@ -311,6 +320,7 @@ def fake_quantize_channel_scaling(a: Tensor, dim_x: int, dim_y: int, block_x: in
     return torch.ops.mor.fake_quantize_channel_scaling.default(a, dim_x, dim_y, block_x, block_y, e4m3_threshold, ss_mode)
 
 
+@torch.compiler.disable
 def fake_quantize_channel_scaling_inplace(a: Tensor, dim_x: int, dim_y: int, block_x: int, block_y: int, e4m3_threshold: float, ss_mode: int) -> List[Tensor]:
     """As fake_quantize_channel_scaling, overwriting a."""
     return torch.ops.mor.fake_quantize_channel_scaling_inplace.default(a, dim_x, dim_y, block_x, block_y, e4m3_threshold, ss_mode)
@@ -321,6 +331,7 @@ def fake_quantize_e8mx(a: Tensor, dim_x: int, dim_y: int, block_x: int, block_y:
     return torch.ops.mor.fake_quantize_e8mx.default(a, dim_x, dim_y, block_x, block_y, quantize_type, scaling_strategy)
 
 
+@torch.compiler.disable
 def fake_quantize_e8mx_inplace(a: Tensor, dim_x: int, dim_y: int, block_x: int, block_y: int, quantize_type: int, scaling_strategy: int, output: Tensor) -> None:
     """As fake_quantize_e8mx, into the given output tensor (which may be the input)."""
     return torch.ops.mor.fake_quantize_e8mx_inplace.default(a, dim_x, dim_y, block_x, block_y, quantize_type, scaling_strategy, output)

@@ -104,11 +104,9 @@ def test_c4_mor_16384x14336(G):
     out, meta = G.fake_quantize(a, 128, 128, 1e-15, 1, 1)
     want, wmeta, stats = O.fake_quantize(a, 128, 128, 1e-15, 1, 1, want_stats=True)
     flip = meta != wmeta
-    if flip.any():     # only sums that tie to 1e-6 may decide differently
-        e4, e5 = stats[..., 2][flip], stats[..., 3][flip]
-        assert np.all(np.abs(e4 - e5) <= 1e-6 * np.maximum(e4, e5)), (int(flip.sum()), e4, e5)
-    keep = np.repeat(np.repeat(~flip, 128, 0), 128, 1)
-    same(np.where(keep, out, 0), np.where(keep, want, 0), "C4")
+    print("C4 format decisions that differ from the oracle's:", int(flip.sum()), "of", meta.size, flush=True)
+    assert not flip.any(), (int(flip.sum()), stats[..., 2][flip], stats[..., 3][flip])     # no change in format choice
+    same(out, want, "C4")
     hist = np.bincount(meta.ravel(), minlength=5)
     n = meta.size
     assert hist[1] + hist[3] + hist[4] == n                  # error mode never returns E5M2
@@ -136,11 +134,9 @@ def test_c5_layer_sweep(G, shape):
     out, meta = G.fake_quantize(a, 128, 128, 1e-15, 1, 1)                       # MoR
     want, wmeta, stats = O.fake_quantize(a, 128, 128, 1e-15, 1, 1, want_stats=True)
     flip = meta != wmeta
-    if flip.any():
-        e4, e5 = stats[..., 2][flip], stats[..., 3][flip]
-        assert np.all(np.abs(e4 - e5) <= 1e-6 * np.maximum(e4, e5))
-    keep = np.repeat(np.repeat(~flip, 128, 0), 128, 1)
-    same(np.where(keep, out, 0), np.where(keep, want, 0), f"C5 MoR {shape}")
+    print("C5", shape, "format decisions that differ from the oracle's:", int(flip.sum()), "of", meta.size, flush=True)
+    assert not flip.any(), (int(flip.sum()), stats[..., 2][flip], stats[..., 3][flip])     # no change in format choice
+    same(out, want, f"C5 MoR {shape}")
     for mode in (2, 3):                                                          # block 128x128
         out, meta = G.fake_quantize(a, 128, 128, 0.0, mode, 1)
         want, wmeta = O.fake_quantize(a, 128, 128, 0.0, mode, 1)

@@ -135,14 +135,9 @@ def test_shapes_modes_vs_oracle(G, shape, mode, sf):
     print("shape", shape, mode, sf, flush=True)
     out, meta = G.fake_quantize(a, br, bc, 1e-15, mode, sf)
     want, wmeta, stats = O.fake_quantize(a, br, bc, 1e-15, mode, sf, want_stats=True)
-    if mode == 1:
-        # a decision between E4M3 and BF16 may legitimately flip only if the two error sums tie to 1e-6
-        flip = meta != wmeta
-        if flip.any():
-            e4, e5 = stats[..., 2][flip], stats[..., 3][flip]
-            assert np.all(np.abs(e4 - e5) <= 1e-6 * np.maximum(e4, e5)), (e4, e5)
-            pytest.skip("error sums tie within 1e-6")
-    assert np.array_equal(meta, wmeta)
+    # no change in format choice: the decisions are the oracle's in every block (none of these seeded cases holds a
+    # block whose two error sums tie to within their own summation noise)
+    assert np.array_equal(meta, wmeta), (int((meta != wmeta).sum()), stats[..., 2][meta != wmeta], stats[..., 3][meta != wmeta])
     assert_same(out, want, f"{shape} mode {mode} sf {sf}")
 
 

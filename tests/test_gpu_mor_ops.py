@@ -271,6 +271,57 @@ def test_ops_trace_under_torch_compile(mor):
     assert torch.equal(got, want) and torch.equal(w.grad, g_eager) and torch.all(g_eager == 1)
 
 
+def test_inplace_ops_under_torch_compile_run_eagerly_and_write(mor):
+    """The ops that write into an argument are excluded from compilation (their schemas declare no aliasing): a compiled
+    function that calls them breaks the graph there, the writes happen, and the values equal the eager ones."""
+    def f(t, buf):
+        y = t * 1.0
+        mor.ops.fake_quantize_e8mx_inplace(y, 256, 512, 128, 128, 2, 1, y)
+        meta = mor.ops.fake_quantize_no_alloc(y, 256, 512, 1, 32, 0.0, 2, 2, buf)
+        stats = mor.ops.fake_quantize_block_scaling_inplace(buf, 256, 512, 128, 128, 0.045, 3)
+        return y + 0.0, meta, stats[0]
+
+    x = random_bf16(77, -8.0, 8.0, 256, 512).cuda()
+    b1, b2 = torch.zeros_like(x), torch.zeros_like(x)
+    want = f(x, b1)
+    got = torch.compile(f, backend="aot_eager")(x, b2)
+    torch.cuda.synchronize()
+    assert torch.equal(b1, b2) and b1.abs().sum() > 0
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    e = mor.ops.fake_quantize_e8mx(x, 256, 512, 128, 128, 2, 1)
+    assert torch.equal(want[0], e)
+
+
+def test_flavour_is_per_thread(mor):
+    """set_flavour applies to the calling thread only."""
+    import threading
+    # blocks of 1 x 32 with amax 1000 and a power-of-two scale: 1e-3 casts to zero, which the CUDA kernel's exponent
+    # arithmetic returns as 2^(2-127) and the torch emulation as 0
+    x = torch.zeros(256, 256)
+    x[:, 0], x[:, 1] = 1000.0, 1e-3
+    x = x.to(torch.bfloat16).cuda()
+    args = (x, 256, 256, 1, 32, 0.0, 2, 2)
+    base = mor.ops.fake_quantize(*args)[0]
+    mor.ops.set_flavour("torch_emulation")
+    emu_here = mor.ops.fake_quantize(*args)[0]
+    mor.ops.set_flavour("kernel")
+    assert base[0, 1].item() > 0 and emu_here[0, 1].item() == 0
+    res = {}
+
+    def other():
+        mor.ops.set_flavour("torch_emulation")
+        res["emu"] = mor.ops.fake_quantize(*args)[0]
+        torch.cuda.synchronize()
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    again = mor.ops.fake_quantize(*args)[0]
+    assert torch.equal(base, again)
+    assert torch.equal(emu_here, res["emu"])
+
+
 def test_concurrent_streams_and_host_threads(mor):
     """The library keeps no state between calls: four host threads, each on its own stream with its own tensors,
     interleave different ops and get what a single-threaded run gets."""

@@ -78,16 +78,10 @@ def test_fake_quantize_sweep(G, case):
     print("sweep", case, flush=True)
     out, meta = G.fake_quantize(a, br, bc, clamp, mode, sf)
     want, wmeta, stats = O.fake_quantize(a, br, bc, clamp, mode, sf, want_stats=True)
-    ok_blocks = np.ones(meta.shape, bool)
-    if mode in (1, 101):
-        flip = meta != wmeta                       # a decision may differ only where the two error sums tie to 1e-6
-        if flip.any():
-            e4, e5 = stats[..., 2][flip], stats[..., 3][flip]
-            assert np.all(np.abs(e4 - e5) <= 1e-6 * np.maximum(e4, e5)), (case, e4, e5)
-            ok_blocks = ~flip
-    assert np.array_equal(meta[ok_blocks], wmeta[ok_blocks]), case
-    mask = np.repeat(np.repeat(ok_blocks, br, 0), bc, 1)[:rows, :cols]
-    bad = np.argwhere((out != want) & mask)
+    # no change in format choice in any block of any case
+    flip = meta != wmeta
+    assert not flip.any(), (case, int(flip.sum()), stats[..., 2][flip], stats[..., 3][flip])
+    bad = np.argwhere(out != want)
     assert len(bad) == 0, (case, len(bad), tuple(bad[0]), hex(int(out[tuple(bad[0])])), hex(int(want[tuple(bad[0])])))
 
 
@@ -128,7 +122,7 @@ def test_scaling_sweep(G, case):
     out, meta, gamax, gnnz, gerr = G.block_scaling(a, br, bc, thr, ss, channel=channel, inplace=inplace)
     want, wmeta, wamax, wnnz, werr = O.block_scaling(a, br, bc, thr, ss, channel=channel)
     assert gamax[0] == wamax[0] and gnnz[0] == wnnz[0], case
-    np.testing.assert_allclose(gerr[0], werr[0], rtol=2e-6, atol=0)
+    np.testing.assert_allclose(gerr[0], werr[0], rtol=1e-6, atol=0)
     avg = werr[0] / max(wnnz[0], 1)
     if abs(avg - thr) > 1e-5 * thr:
         assert meta[0] == wmeta[0], case
