@@ -4,11 +4,13 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
 
 One step = one pass of the MX block-scaling workload (BASELINE configs[1]) over an 8192 x 8192 bf16 tensor
-resident in HBM: 1 x 32 blocks, power-of-two (E8M0) shared scale, elements cast to E4M3, E5M2 and E2M3 (three
-launches).  The printed JSON line reports algorithmic HBM GB/s (2 B read + 2 B written per element + 4 B of meta per
-block where the op returns meta) for the whole step, the roofline fraction of the slowest of the three kernels
-from HIP events recorded around every launch in the timed region, the other configurations, and the CPU oracle
-timed on a bounded sample of the same workload on the host cores.
+resident in HBM -- 1 x 32 blocks, power-of-two (E8M0) shared scale, elements cast to E4M3, E5M2 and E2M3 -- plus one
+MoR 128 x 128 pass over an 8192 x 8192 N(0,1) tensor (four launches).  The launches rotate over several input /
+output buffer pairs, so that every byte comes from HBM and not from the 256 MB last-level cache.  The printed JSON
+line reports algorithmic HBM GB/s (2 B read + 2 B written per element + 4 B of meta per block where the op returns
+meta) for the whole step, the roofline fraction of the kernel furthest below the roofline from HIP events recorded
+around its launches in the timed region (with the cache-warm figure of every kernel beside it), the other
+configurations, and the CPU oracle timed on bounded samples of the same workloads on the host cores.
 """
 import argparse
 import json
@@ -30,6 +32,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
+    ap.add_argument("--no-warm", action="store_true", help="skip the same-buffer (cache-warm) and plain-copy side measurements")
+    ap.add_argument("--rotate", type=int, default=6, help="input / output buffer pairs the timed launches rotate over")
     ap.add_argument("--rows", type=int, default=8192)
     ap.add_argument("--cols", type=int, default=8192)
     return ap.parse_args()
@@ -67,14 +71,14 @@ class Launcher:
     def stream(self):
         return self.torch.cuda.current_stream().cuda_stream
 
-    def fake_quantize(self, x, out, meta, br, bc, clamp, mode, sf):
+    def fake_quantize(self, x, out, meta, br, bc, clamp, mode, sf, flags=0):
         r, c = x.shape
         self.cabi.check(self.L.mor_fake_quantize(x.data_ptr(), out.data_ptr(), meta.data_ptr(), r, c, br, bc,
-                                                 float(clamp), mode, sf, 0, self.stream()))
+                                                 float(clamp), mode, sf, flags, self.stream()))
 
-    def block_format(self, x, out, br, bc, fmt, sf):
+    def block_format(self, x, out, br, bc, fmt, sf, flags=0):
         r, c = x.shape
-        self.cabi.check(self.L.mor_block_format(x.data_ptr(), out.data_ptr(), r, c, br, bc, fmt, sf, 0, self.stream()))
+        self.cabi.check(self.L.mor_block_format(x.data_ptr(), out.data_ptr(), r, c, br, bc, fmt, sf, flags, self.stream()))
 
 
     def scaling_state(self, rows, cols, br, bc, channel):
@@ -110,17 +114,18 @@ def time_launches(torch, fn, steps, warmup):
 
 
 def read_traffic(kernel):
-    """HBM bytes per launch of `kernel` from the committed counter summary (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
-    each scaled by the same counter's reading for the library's plain copy kernel); None when there is no summary."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")
+    """-> (HBM bytes per launch of `kernel`, where the figure comes from).  Hardware counters cannot be read from inside
+    the run: the figure is the one in the committed counter summary (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+    script, each scaled by the same counter's reading for the library's plain copy kernel); None when it holds none."""
+    rel = os.path.join("profiles", "hbm_traffic_counters.txt")
     try:
-        for line in open(path):
+        for line in open(os.path.join(ROOT, rel)):
             f = line.split()
             if len(f) >= 3 and f[0] == "traffic_bytes" and f[1] == kernel:
-                return int(f[2])
+                return int(f[2]), rel + " (rocprofv3 --pmc, not measured in this run)"
     except OSError:
         pass
-    return None
+    return None, None
 
 
 def main():
@@ -144,49 +149,79 @@ def main():
     rows, cols = args.rows, args.cols
     K, W = args.steps, args.warmup
 
-    x = gen_c2_gpu(torch, rows, cols)
-    out = torch.empty_like(x)
+    # Inputs and outputs of the timed step, ROT copies of each so that no launch finds its data in the 256 MB last-level
+    # cache: the MX tensor (Student-t, outliers) and the MoR tensor (N(0,1)), both rows x cols bf16.
+    ROT = args.rotate
+    x_mx = gen_c2_gpu(torch, rows, cols)
+    g = torch.Generator(device="cuda").manual_seed(1001)
+    x_mor = torch.randn(rows, cols, device="cuda", generator=g).to(torch.bfloat16)
+    xs_mx = [x_mx] + [x_mx.clone() for _ in range(ROT - 1)]
+    xs_mor = [x_mor] + [x_mor.clone() for _ in range(ROT - 1)]
+    outs = [torch.empty_like(x_mx) for _ in range(ROT)]
     meta = torch.empty((rows, cols // 32), dtype=torch.int32, device="cuda")
+    meta_mor = torch.empty(((rows + 127) // 128, (cols + 127) // 128), dtype=torch.int32, device="cuda")
     nelem = rows * cols
     nblocks = nelem // 32
     launches = [
-        ("mx_e4m3", lambda: run.fake_quantize(x, out, meta, 1, 32, 0.0, 2, 2), nelem * 4 + nblocks * 4),
-        ("mx_e5m2", lambda: run.fake_quantize(x, out, meta, 1, 32, 0.0, 3, 2), nelem * 4 + nblocks * 4),
-        ("mx_e2m3", lambda: run.block_format(x, out, 1, 32, _cabi.FMT_E2M3, 2), nelem * 4),
+        ("mx_e4m3", lambda i: run.fake_quantize(xs_mx[i], outs[i], meta, 1, 32, 0.0, 2, 2), nelem * 4 + nblocks * 4),
+        ("mx_e5m2", lambda i: run.fake_quantize(xs_mx[i], outs[i], meta, 1, 32, 0.0, 3, 2), nelem * 4 + nblocks * 4),
+        ("mx_e2m3", lambda i: run.block_format(xs_mx[i], outs[i], 1, 32, _cabi.FMT_E2M3, 2), nelem * 4),
+        ("mor_128x128", lambda i: run.fake_quantize(xs_mor[i], outs[i], meta_mor, 128, 128, 1e-15, 1, 1), nelem * 4 + meta_mor.numel() * 4),
     ]
     bytes_per_step = sum(b for _, _, b in launches)
 
-    def step():
-        for _, fn, _ in launches:
-            fn()
+    turn = [0]
+
+    def rotating(fn):
+        turn[0] = (turn[0] + 1) % ROT
+        fn(turn[0])
 
     for _ in range(W):
-        step()
+        for _, fn, _ in launches:
+            rotating(fn)
     torch.cuda.synchronize()
-    # The timed region holds exactly K steps of work.  Its launches are grouped by format (K x E4M3, K x E5M2,
-    # K x E2M3) so that one pair of HIP events brackets the K launches of each kernel: an event between every two
-    # launches would add its own few microseconds to 45-microsecond kernels.
+    # The timed region holds exactly K steps of work.  Its launches are grouped by kernel (K x E4M3, K x E5M2,
+    # K x E2M3, K x MoR) so that one pair of HIP events brackets the K launches of each kernel: an event between every
+    # two launches would add its own few microseconds to 45-microsecond kernels.  Events and launches share torch's
+    # current stream.
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(len(launches) + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     marks[0].record()
     for i, (_, fn, _) in enumerate(launches):
         for _ in range(K):
-            fn()
+            rotating(fn)
         marks[i + 1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / K
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
 
+    def rate(nbytes, ms):
+        return {"ms": round(ms, 5), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
     per_kernel = {}
-    for i, (name, _, nbytes) in enumerate(launches):
-        ms = marks[i].elapsed_time(marks[i + 1]) / K
-        per_kernel[name] = {"ms": round(ms, 5), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
-                            "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "bytes": nbytes}
-    dom = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
+    for i, (name, fn, nbytes) in enumerate(launches):
+        per_kernel[name] = dict(rate(nbytes, marks[i].elapsed_time(marks[i + 1]) / K), bytes=nbytes)
+    # The same kernels on one buffer pair, launch after launch: the 268 MB working set is then about the size of the
+    # last-level cache, which serves part of it -- reported beside the HBM figure, never as it.  And the library's plain
+    # copy over the same rotation: what the memory system gives a kernel that only moves the bytes.
+    if not args.no_warm:
+        for name, fn, nbytes in launches:
+            ms = time_launches(torch, lambda: fn(0), max(K, 20), 3)[0]
+            per_kernel[name]["same_buffers_warm_cache"] = rate(nbytes, ms)
+        copy_ms = time_launches(torch, lambda: rotating(lambda i: run.fake_quantize(xs_mx[i], outs[i], meta_mor, 128, 128, 0.0, 7, 1)), max(K, 20), 3)[0]
+        per_kernel["plain_copy_mode7"] = dict(rate(nelem * 4 + meta_mor.numel() * 4, copy_ms), bytes=nelem * 4 + meta_mor.numel() * 4,
+                                              note="not part of the step: the library's bf16 copy over the same rotating buffers")
+    timed = [n for n, _, _ in launches]
+    dom = min(timed, key=lambda n: per_kernel[n]["frac"])
+    traffic, traffic_src = read_traffic(dom)
     roofline = {"bound": "hbm", "kernel": dom, "achieved": per_kernel[dom]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": per_kernel[dom]["frac"], "traffic": read_traffic(dom), "per_kernel": per_kernel}
+                "frac": per_kernel[dom]["frac"], "traffic": traffic, "traffic_source": traffic_src,
+                "buffers": f"{ROT} input / output pairs in rotation ({ROT * 2 * nelem * 2 / 2**30:.1f} GiB): nothing is cache-resident",
+                "per_kernel": per_kernel}
+    x = x_mx
+    del xs_mx, xs_mor, outs
 
     extra = {}
     if not args.no_extra:
@@ -194,16 +229,18 @@ def main():
 
     cpu = None
     if not args.no_cpu:
-        cpu = cpu_baseline(torch, x)
+        cpu = cpu_baseline(torch, x, x_mor)
 
     line = {
-        "metric": "fake-quant HBM GB/s (rd+wr), MX 1x32 E8M0 block scaling on 8192x8192 bf16 (E4M3+E5M2+E2M3)",
+        "metric": "fake-quant HBM GB/s (rd+wr), MX 1x32 E8M0 block scaling (E4M3+E5M2+E2M3) and MoR 128x128 on 8192x8192 bf16",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"configs[1]: MX block scaling {rows}x{cols} bf16, 1x32 blocks, E8M0 scale, E4M3+E5M2+E2M3 per step",
+        "config": {"workload": f"configs[1]: MX block scaling {rows}x{cols} bf16, 1x32 blocks, E8M0 scale, E4M3+E5M2+E2M3, "
+                               f"plus MoR 128x128 (fp32 scale, error criterion) on a {rows}x{cols} N(0,1) tensor, per step; "
+                               f"{ROT} buffer pairs in rotation",
                    "arithmetic": "bf16 tensors, fp32 / integer arithmetic, gfx950 fp8 / fp6 converts",
-                   "elements_per_s": round(3 * nelem / (ms_per_step * 1e-3), 0), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+                   "elements_per_s": round(4 * nelem / (ms_per_step * 1e-3), 0), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "other_configs": extra,
@@ -222,13 +259,13 @@ def other_configs(torch, run, cabi, K, W):
         res[name] = {"ms": round(ms, 5), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "elements_per_s": round(nelem / (ms * 1e-3), 0)}
 
-    # MoR 128x128 on 8192x8192 N(0,1) and on the C4 mixture at its full size
+    # (every figure in this function is taken on one buffer pair, launch after launch; tensors of up to 128 MiB are then
+    # partly served by the 256 MB last-level cache -- only the 16384 x 14336 cases are pure HBM figures)
     g = torch.Generator(device="cuda").manual_seed(1001)
     x = torch.randn(8192, 8192, device="cuda", generator=g).to(torch.bfloat16)
     out = torch.empty_like(x)
     meta = torch.empty((64, 64), dtype=torch.int32, device="cuda")
     n = x.numel()
-    add("mor_128x128_8192x8192_normal", lambda: run.fake_quantize(x, out, meta, 128, 128, 1e-15, 1, 1), n * 4 + meta.numel() * 4, n)
     add("copy_mode7_8192x8192", lambda: run.fake_quantize(x, out, meta, 128, 128, 0.0, 7, 1), n * 4 + meta.numel() * 4, n)
     add("block_e4m3_128x128_8192x8192_fp32scale", lambda: run.fake_quantize(x, out, meta, 128, 128, 0.0, 2, 1), n * 4 + meta.numel() * 4, n)
     # blocks beyond the 16384 elements a 256-thread workgroup keeps in registers (same 67.1 M elements)
@@ -237,22 +274,6 @@ def other_configs(torch, run, cabi, K, W):
     add("mor_256x256_8192x8192_normal", lambda: run.fake_quantize(x, out, meta, 256, 256, 1e-15, 1, 1), n * 4, n)
     add("per_row_e4m3_2048x32768", lambda: run.fake_quantize(x.view(2048, 32768), out.view(2048, 32768), meta, 1, 32768, 0.0, 2, 1), n * 4, n)
     add("per_row_e4m3_512x131072", lambda: run.fake_quantize(x.view(512, 131072), out.view(512, 131072), meta, 1, 131072, 0.0, 2, 1), n * 4, n)
-    # the benchmark kernel with nothing left in the 256 MB last-level cache: 6 input / output pairs (1.6 GB) in rotation
-    xs6 = [x] + [x.clone() for _ in range(5)]
-    os6 = [torch.empty_like(x) for _ in range(6)]
-    mx_meta = torch.empty((8192, 256), dtype=torch.int32, device="cuda")
-    turn = [0]
-
-    def rotating():
-        i = turn[0] = (turn[0] + 1) % 6
-        run.fake_quantize(xs6[i], os6[i], mx_meta, 1, 32, 0.0, 2, 2)
-    add("mx_e4m3_8192x8192_rotating_buffers_cold_cache", rotating, n * 4 + (n // 32) * 4, n)
-
-    def rotating_copy():          # the floor of that run: the library's plain copy over the same rotation
-        i = turn[0] = (turn[0] + 1) % 6
-        run.fake_quantize(xs6[i], os6[i], meta, 128, 128, 0.0, 7, 1)
-    add("copy_mode7_8192x8192_rotating_buffers_cold_cache", rotating_copy, n * 4 + meta.numel() * 4, n)
-    del xs6, os6, mx_meta
     # C1: per-tensor E4M3, 4096x4096, scale from the tensor amax (the quantize pass only: 4 B/element)
     x1 = x[:4096, :4096].contiguous()
     o1 = torch.empty_like(x1)
@@ -286,6 +307,7 @@ def other_configs(torch, run, cabi, K, W):
     hist = torch.bincount(m4.flatten(), minlength=13).tolist()
     res["c4_mor_128x128_16384x14336_mixture"]["meta_histogram"] = {str(i): h for i, h in enumerate(hist) if h}
     del x4, o4
+    res["flavour_differences"] = flavour_differences(torch, run, cabi)
     res["c5_llama3_8b_layer"] = c5_sweep(torch, run, max(3, K // 4), 2)
     res["mx_wire_format_8192x8192"] = wire_format(torch, run, K, W)
     # launch overhead: a 1x32 tensor
@@ -311,6 +333,44 @@ def other_configs(torch, run, cabi, K, W):
     for key, t in (("mor_ops_us_per_call", xs), ("mor_ops_requires_grad_us_per_call", xg)):
         ms, wall = time_launches(torch, lambda: mor.ops.fake_quantize(t, 1, 32, 1, 32, 0.0, 2, 2), 500, 50)
         res["tiny_1x32"][key] = round(wall * 1e3, 2)
+    return res
+
+
+def flavour_differences(torch, run, cabi):
+    """Per configuration, the number of elements on which the two flavours of the library differ: what the reference's
+    CUDA kernel returns (the default: round-half-up bf16 store, exponent-field power-of-two scaling, +0 from the
+    software cast) against what its torch emulation returns (nearest-even store, true zeros, signed zeros)."""
+    EMU = cabi.FLAG_TORCH_EMULATION
+    res = {}
+
+    def count(name, x, call):
+        a, b = torch.empty_like(x), torch.empty_like(x)
+        call(a, 0)
+        call(b, EMU)
+        torch.cuda.synchronize()
+        d = a.view(torch.int16) != b.view(torch.int16)
+        res[name] = {"elements": x.numel(), "differ": int(d.sum().item()),
+                     "differ_ignoring_sign_of_zero": int((d & ((a != 0) | (b != 0))).sum().item())}
+
+    g = torch.Generator(device="cuda").manual_seed(1001)
+    x1 = torch.randn(4096, 4096, device="cuda", generator=g).to(torch.bfloat16)
+    m = torch.empty(4096 * 4096 // 32, dtype=torch.int32, device="cuda")
+    scale = float(448.0 / x1.float().abs().max().item())
+    count("c1_per_tensor_e4m3_4096x4096", x1, lambda o, f: run.fake_quantize(x1, o, m, 128, 128, scale, 4, 1, f))
+    x2 = gen_c2_gpu(torch, 4096, 8192)
+    m2 = torch.empty(x2.numel() // 32, dtype=torch.int32, device="cuda")
+    count("c2_mx_e4m3_half_tensor", x2, lambda o, f: run.fake_quantize(x2, o, m2, 1, 32, 0.0, 2, 2, f))
+    count("c2_mx_e5m2_half_tensor", x2, lambda o, f: run.fake_quantize(x2, o, m2, 1, 32, 0.0, 3, 2, f))
+    count("c2_mx_e2m3_half_tensor", x2, lambda o, f: run.block_format(x2, o, 1, 32, cabi.FMT_E2M3, 2, f))
+    g = torch.Generator(device="cuda").manual_seed(1003)
+    w = torch.randn(8192, 4096, device="cuda", generator=g) * 0.02
+    w[torch.randperm(8192, device="cuda", generator=g)[:82]] *= 100
+    w[7] = 0
+    w = w.to(torch.bfloat16)
+    count("c3_per_row_e4m3_half_tensor", w, lambda o, f: run.fake_quantize(w, o, m, 1, 4096, 0.0, 2, 1, f))
+    count("c3_per_row_e5m2_half_tensor", w, lambda o, f: run.fake_quantize(w, o, m, 1, 4096, 0.0, 3, 1, f))
+    x4 = gen_c4_gpu(torch, 4096, 14336)
+    count("c4_mor_128x128_quarter_tensor", x4, lambda o, f: run.fake_quantize(x4, o, m, 128, 128, 1e-15, 1, 1, f))
     return res
 
 
@@ -420,48 +480,76 @@ def c5_sweep(torch, run, K, W):
     return fam
 
 
-def cpu_baseline(torch, x_gpu):
-    """The CPU oracle (a port of the reference arithmetic) on the first rows of the same tensor, all host threads."""
+def cpu_baseline(torch, x_gpu, x_mor_gpu):
+    """The CPU oracle (a port of the reference arithmetic, OpenMP over blocks, all host threads) on bounded samples:
+    the benchmark step (`value`) and one row per configuration (`per_config`), each about two seconds of CPU work; plus
+    a vectorised restatement of the reference's torch emulation (its own CPU path, test/test_fake_quantize.py:33-143,
+    432-436) where that exists for the configuration."""
     from oracle import mor_oracle as O
     import numpy as np
+    import torch_emulation as E
     O.lib()
+    torch.set_num_threads(os.cpu_count() or 1)
+
+    def bits(t):
+        return t.contiguous().cpu().view(torch.int16).numpy().view(np.uint16).copy()
+
+    def timed(fn, budget_s, max_reps=200):
+        fn()                                           # warm-up (page faults, thread pool)
+        reps, t_total, t_start = 0, 0.0, time.perf_counter()
+        while True:
+            t0 = time.perf_counter()
+            fn()
+            t_total += time.perf_counter() - t0
+            reps += 1
+            if time.perf_counter() - t_start > budget_s or reps >= max_reps:
+                return t_total / reps, reps
+
     rows = 2048
-    a = x_gpu[:rows].cpu().view(torch.int16).numpy().view(np.uint16).copy()
+    a = bits(x_gpu[:rows])
+    am = bits(x_mor_gpu[:rows])
     n = a.size
-    nbytes = 0
-    t_total = 0.0
-    reps = 0
-    t_start = time.perf_counter()
-    while True:
-        t0 = time.perf_counter()
+    step_bytes = 4 * n * 4 + 2 * (n // 32) * 4 + (n // 16384) * 4
+
+    def step():
         O.fake_quantize(a, 1, 32, 0.0, 2, 2)
         O.fake_quantize(a, 1, 32, 0.0, 3, 2)
         O.block_format(a, 1, 32, O.E2M3, 2)
-        t_total += time.perf_counter() - t0
-        nbytes += 3 * n * 4 + 2 * (n // 32) * 4
-        reps += 1
-        if time.perf_counter() - t_start > 10.0 or reps >= 2000:
-            break
-    res = {"value": round(nbytes / t_total / 1e9, 3), "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
-           "sample": f"first {rows} rows of the benchmark tensor ({n} elements), E4M3+E5M2+E2M3, {reps} repetitions, "
-                     f"C oracle with OpenMP over blocks"}
-    # the reference's own CPU path is its torch emulation (test/test_fake_quantize.py:33-143): a vectorised restatement
-    # of it on the same sample, all host threads, median of 5 runs after 2 warm-up runs
-    try:
-        import torch_emulation as E
-        torch.set_num_threads(os.cpu_count() or 1)
-        times = []
-        for i in range(7):
-            t0 = time.perf_counter()
-            for fmt in ("e4m3", "e5m2", "e2m3"):
-                E.block_format_fast(a, 1, 32, fmt, e8=True)
-            if i >= 2:
-                times.append(time.perf_counter() - t0)
-        med = sorted(times)[len(times) // 2]
-        res["torch_emulation"] = {"value": round((3 * n * 4 + 2 * (n // 32) * 4) / med / 1e9, 3), "unit": "GB/s",
-                                  "threads": torch.get_num_threads(), "what": "vectorised torch CPU emulation (float8 casts), same sample"}
-    except Exception as e:                                   # the emulation is a courtesy figure, never a failure
-        res["torch_emulation"] = {"error": repr(e)}
+        O.fake_quantize(am, 128, 128, 1e-15, 1, 1)
+
+    sec, reps = timed(step, 6.0)
+    res = {"value": round(step_bytes / sec / 1e9, 3), "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+           "sample": f"first {rows} rows of the two benchmark tensors ({n} elements each): MX E4M3 + E5M2 + E2M3 and MoR 128x128, "
+                     f"{reps} repetitions, C oracle with OpenMP over blocks"}
+    per = {}
+
+    def row(name, nbytes, what, oracle_fn, emu_fn=None, budget=2.0):
+        sec, reps = timed(oracle_fn, budget)
+        per[name] = {"oracle_GBps": round(nbytes / sec / 1e9, 3), "elements_per_s": round(nbytes / 4 / sec, 0), "sample": what, "repetitions": reps}
+        if emu_fn is not None:
+            try:
+                sec, reps = timed(emu_fn, budget, 20)
+                per[name]["torch_emulation_GBps"] = round(nbytes / sec / 1e9, 3)
+            except Exception as e:                                   # the emulation is a courtesy figure, never a failure
+                per[name]["torch_emulation_error"] = repr(e)
+
+    # C1: the reference's own CPU-runnable case, at full size: per-tensor E4M3 on 4096 x 4096 N(0,1)
+    g = torch.Generator().manual_seed(1001)
+    t1 = torch.randn(4096, 4096, generator=g).to(torch.bfloat16)
+    a1 = bits(t1)
+    amax1 = t1.float().abs().max().item()
+    s1 = float(np.float32(448.0) / np.float32(amax1))
+    row("c1_per_tensor_e4m3_4096x4096", a1.size * 4, "the whole tensor, scale 448 / amax",
+        lambda: O.fake_quantize(a1, 128, 128, s1, 4, 1),
+        lambda: E.quant_dequant_scaled(t1.float(), "e4m3", amax1).to(torch.bfloat16))
+    row("c2_mx_e4m3_8192x8192", n * 4, f"first {rows} rows", lambda: O.fake_quantize(a, 1, 32, 0.0, 2, 2),
+        lambda: E.block_format_fast(a, 1, 32, "e4m3", e8=True))
+    a3 = a.reshape(rows * 2, 4096)
+    row("c3_per_row_e4m3_16384x4096", a3.size * 4, f"{a3.shape[0]} rows of 4096 elements", lambda: O.fake_quantize(a3, 1, 4096, 0.0, 2, 1),
+        lambda: E.block_format_fast(a3, 1, 4096, "e4m3"))
+    a4 = bits(gen_c4_gpu(torch, 1024, 14336))
+    row("c4_mor_128x128_16384x14336", a4.size * 4, "1024 rows of the tile mixture (896 tiles)", lambda: O.fake_quantize(a4, 128, 128, 1e-15, 1, 1))
+    res["per_config"] = per
     try:
         with open("/proc/cpuinfo") as f:
             res["cpu_model"] = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "unknown")

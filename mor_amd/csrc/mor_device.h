@@ -60,6 +60,11 @@ __device__ __forceinline__ void store16_rt(uint4* p, uint4 v, bool nt) {
 // cache: nothing of such a tensor is found there again (MX 1 x 32 on 16384 x 14336: 160 -> 150 us; at 8192^2 streaming
 // loads cost 39 -> 44 us).
 __device__ __forceinline__ bool streams_in(int64_t bf16_elements) { return bf16_elements > ((int64_t)128 << 20); }
+// The last (or only) read a kernel makes of a tensor of 32 MiB or more streams as well: nothing reads those lines again,
+// and with streaming loads a tensor that comes from HBM does not push the caller's data out of the caches on its way
+// (8192^2 from HBM, 1 x 32 blocks: 45.5 -> 43 us; repeated launches on one buffer pair, which find part of their input in
+// the last-level cache only because the previous launch left it there, lose that: 39 -> 44 us).
+__device__ __forceinline__ bool streams_last_read(int64_t bf16_elements) { return bf16_elements >= ((int64_t)16 << 20); }
 __device__ __forceinline__ uint4 load16_rt(const uint4* p, bool nt) { return nt ? load16<true>(p) : load16<false>(p); }
 
 // ---------------------------------------------------------------- bf16 <-> fp32
@@ -166,6 +171,12 @@ template <int F> __device__ __forceinline__ uint32_t hw_pack2_low(float a, float
     const s16x2 z = {0, 0};
     if constexpr (F == FMT_E4M3) return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(z, a, b, 1.0f, false));
     else return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(z, a, b, 1.0f, false));
+}
+// the same with the other half of the result register taken from `old` (its contents do not matter to the caller)
+template <int F> __device__ __forceinline__ uint32_t hw_pack2_low_keep(float a, float b, uint32_t old) {
+    const s16x2 o = __builtin_bit_cast(s16x2, old);
+    if constexpr (F == FMT_E4M3) return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, a, b, 1.0f, false));
+    else return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(o, a, b, 1.0f, false));
 }
 template <int F> __device__ __forceinline__ f32x2 hw_unpack2_low(uint32_t p) {
     if constexpr (F == FMT_E4M3) return __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(p, 1.0f, false);

@@ -53,7 +53,7 @@ __global__ __launch_bounds__(WG) void k_elementwise_fast(const uint16_t* in, uin
     const int64_t base = (int64_t)blockIdx.x * (EW_NV * WG) + threadIdx.x;
     uint4 v[EW_NV];
 #pragma unroll
-    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = load16_rt(in4 + c, streams_in(n)); }
+    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = load16_rt(in4 + c, streams_last_read(n)); }
     const bool nt = streams_out(n);
     if (fmt == FMT_E4M3) {
 #pragma unroll
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(WG) void k_copy(const uint16_t* in, uint16_t* out, 
     const int64_t base = (int64_t)blockIdx.x * (EW_NV * WG) + threadIdx.x;
     uint4 v[EW_NV];
 #pragma unroll
-    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = load16_rt(in4 + c, streams_in(n)); }
+    for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; v[k] = make_uint4(0, 0, 0, 0); if (c < nvec) v[k] = load16_rt(in4 + c, streams_last_read(n)); }
 #pragma unroll
     for (int k = 0; k < EW_NV; ++k) { int64_t c = base + k * WG; if (c < nvec) store16_rt(out4 + c, v[k], streams_out(n)); }
     for (int64_t i = nvec * 8 + gtid; i < n; i += stride) out[i] = in[i];
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(WG) void k_rowgroup(const uint4* in, uint4* out, in
                                                  int64_t nchunks, int G, int logG, int meta_val) {
     if constexpr (GT > 0) { G = GT; }
     const int64_t base = (int64_t)blockIdx.x * (NV * WG) + threadIdx.x;
-    const bool lnt = streams_in(nchunks * 8);
+    const bool lnt = streams_last_read(nchunks * 8);
     uint4 v[NV];
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
@@ -207,7 +207,9 @@ __global__ __launch_bounds__(WG) void k_block_stats(const uint16_t* __restrict__
     __shared__ float s_f[WAVES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t bid = first + blockIdx.x;
-    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    uint32_t by32, bx32;
+    block_of(sh, (uint32_t)bid, by32, bx32);                  // (fewer than 2^31 blocks)
+    const int64_t by = by32, bx = bx32;
     const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
     const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
     float amax = 0.0f;
@@ -376,24 +378,25 @@ static void launch_rowgroup_f(const uint4* i4, uint4* o4, int32_t* meta, int64_t
         else k_rowgroup<F, E8, NV, 256, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
         return;
     }
-    // Two vectors per lane: many small workgroups interleave their loads and stores more finely than few large ones
-    // (measured at 8192^2 with 8 / 4 / 2 / 1 vectors per lane: E4M3 41.3 / 40.6 / 39.3 / 42.4 us, E2M3 41.8 / 40.1 /
-    // 37.9 / 38.6 us).
-    constexpr int NV = 2;
-    if (nchunks * 16 >= ((int64_t)4 << 20) && nchunks % ((int64_t)NV * WG) == 0 && (G == 4 || G == 16)) {
-        const int64_t grid64 = nchunks / ((int64_t)NV * WG);
-        if (grid64 <= 0x7FFFFFFFll) {
-            const int grid = (int)grid64;
-            if (G == 4) k_rowgroup<F, E8, NV, 4, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
-            else k_rowgroup<F, E8, NV, 16, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
-            return;
-        }
-    }
-    {
-        const int grid = (int)cdiv(nchunks, (int64_t)NV * WG);
-        if (nchunks * 16 >= ((int64_t)4 << 20)) k_rowgroup<F, E8, NV, 0, false, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
-        else k_rowgroup<F, E8, NV, 0, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val);
-    }
+    // Few vectors per lane: many small workgroups interleave their loads and stores more finely than few large ones.
+    // Tensors of 32 MiB and more (they come from HBM) take one vector per lane: a plain copy of 8192^2 from HBM runs at
+    // 0.79 of the peak rate with one, 0.76 with two, 0.73 with eight vectors per lane; at 16384 x 14336: 0.82 / 0.76 /
+    // 0.73.  Smaller tensors take two (fewer workgroups to launch).
+    // (the software casts of E2M3 / E3M2 cost more instructions per element and are better off with two: 49.6 -> 45.4 us)
+    const bool big = nchunks * 16 >= ((int64_t)32 << 20) && Fmt<F>::hw;
+    const bool nt_out = nchunks * 16 >= ((int64_t)4 << 20);
+#define MOR_ROWGROUP(NV) do { \
+        if (nt_out && nchunks % ((int64_t)NV * WG) == 0 && (G == 4 || G == 16) && nchunks / ((int64_t)NV * WG) <= 0x7FFFFFFFll) { \
+            const int grid = (int)(nchunks / ((int64_t)NV * WG)); \
+            if (G == 4) k_rowgroup<F, E8, NV, 4, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); \
+            else k_rowgroup<F, E8, NV, 16, true, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); \
+        } else { \
+            const int grid = (int)cdiv(nchunks, (int64_t)NV * WG); \
+            if (nt_out) k_rowgroup<F, E8, NV, 0, false, true><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); \
+            else k_rowgroup<F, E8, NV, 0, false><<<grid, WG, 0, st>>>(i4, o4, meta, nchunks, G, lg, meta_val); \
+        } } while (0)
+    if (big) MOR_ROWGROUP(1); else MOR_ROWGROUP(2);
+#undef MOR_ROWGROUP
 }
 
 template <bool E8>
@@ -412,7 +415,7 @@ static void launch_rowgroup(int fmt, const void* in, void* out, int32_t* meta, i
 static int run_quantize(const void* input, void* output, int32_t* meta, float* stats,
                         int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
                         const QuantArgs& qa, bool e8, uint32_t flags, hipStream_t st) {
-    Shape sh{rows, cols, brows, bcols, cdiv(rows, brows), cdiv(cols, bcols)};
+    const Shape sh = make_shape(rows, cols, brows, bcols);
     const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
     const bool fast_ok = !emu && !(flags & MOR_FLAG_SOFTWARE_CAST);
     const int64_t nblocks = sh.gy * sh.gx;
@@ -531,7 +534,7 @@ extern "C" int mor_block_stats(const void* input, int64_t rows, int64_t cols, in
                                float fmax, float* amax, float* scale, int32_t* e8m0, void* stream) {
     if (int rc = mor_validate_shape(input, rows, cols, brows, bcols)) return rc;
     if (!amax || !scale || !e8m0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output pointer is NULL");
-    Shape sh{rows, cols, brows, bcols, cdiv(rows, brows), cdiv(cols, bcols)};
+    const Shape sh = make_shape(rows, cols, brows, bcols);
     for_slices(sh.gy * sh.gx, [&](int64_t first, int count) {
         k_block_stats<<<count, WG, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const uint16_t*>(input), sh, fmax, amax, scale, e8m0, first);
     });

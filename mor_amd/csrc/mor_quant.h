@@ -87,16 +87,18 @@ __device__ __forceinline__ void err_terms_exact(float x, bool e8, const Scale& s
 
 // ------------------------------------------------------------------------------------------------
 // quantize one packed word with an fp32 scale: |x| * s, hardware convert, divide by s, round-half-up store, sign
-template <int F> __device__ __forceinline__ uint32_t fq_pair_div(uint32_t w, float s, float r) {
-    const f32x2 c = hw_unpack2_low<F>(hw_pack2_low<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s));
+// (`codes`: the register the converts write half of, carried from word to word so that no fresh zero is needed)
+template <int F> __device__ __forceinline__ uint32_t fq_pair_div(uint32_t w, float s, float r, uint32_t& codes) {
+    codes = hw_pack2_low_keep<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s, codes);
+    const f32x2 c = hw_unpack2_low<F>(codes);
     return store_pair<false>(div_by_scale(c.x, s, r), div_by_scale(c.y, s, r)) | (w & 0x80008000u);
 }
-template <int F> __device__ __forceinline__ uint4 fq_vec_div(uint4 v, float s, float r) {
+template <int F> __device__ __forceinline__ uint4 fq_vec_div(uint4 v, float s, float r, uint32_t& codes) {
     uint4 o;
-    o.x = fq_pair_div<F>(v.x, s, r);
-    o.y = fq_pair_div<F>(v.y, s, r);
-    o.z = fq_pair_div<F>(v.z, s, r);
-    o.w = fq_pair_div<F>(v.w, s, r);
+    o.x = fq_pair_div<F>(v.x, s, r, codes);
+    o.y = fq_pair_div<F>(v.y, s, r, codes);
+    o.z = fq_pair_div<F>(v.z, s, r, codes);
+    o.w = fq_pair_div<F>(v.w, s, r, codes);
     return o;
 }
 
@@ -186,7 +188,9 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
                                               float (*s_f)[WGS / 64], uint32_t* s_u, bool allow_fast = false) {
     constexpr int NW = WGS / 64;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    uint32_t by32, bx32;
+    block_of(sh, (uint32_t)bid, by32, bx32);                  // (fewer than 2^31 blocks)
+    const int64_t by = by32, bx = bx32;
     const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
     const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
     float amax = 0.0f;
@@ -247,7 +251,7 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
     }
     if (tid == 0) {
         if (meta && meta_val >= 0) meta[bid] = meta_val;
-        if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+        if (stats) { float* s = stats + 4 * (int64_t)bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
     }
     if (!out) return;
     const bool copy = (fmt < 0) || !(amax > 0.0f);

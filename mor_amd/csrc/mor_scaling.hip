@@ -367,7 +367,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
         for (uint32_t c = blockIdx.x * WG + threadIdx.x; c < nchunks; c += gridDim.x * WG) {
             const uint32_t row = div_u32(c, d_rowchunks), cc = c - row * row_chunks;
             const uint32_t by = div_u32(row, d_brows);
-            uint4 v = load16_rt(in4 + c, streams_in(sh.rows * sh.cols));
+            uint4 v = load16_rt(in4 + c, streams_last_read(sh.rows * sh.cols));
             uint32_t w[4] = {v.x, v.y, v.z, v.w};
             if constexpr (COL) {
                 const float* sp = scales + (int64_t)by * sh.cols + (int64_t)cc * 8;
@@ -450,7 +450,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         v[k] = make_uint4(0, 0, 0, 0);
-                        if (r + k < r_end) v[k] = load16_rt(in4 + (r + k) * row_stride + (col0 >> 3), streams_in(sh.rows * sh.cols));
+                        if (r + k < r_end) v[k] = load16_rt(in4 + (r + k) * row_stride + (col0 >> 3), streams_last_read(sh.rows * sh.cols));
                     }
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
@@ -607,12 +607,10 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
     float gmax = 0.0f, err = 0.0f;
     int nnz_total = 0;
     for (int64_t t = blockIdx.x; t < nblocks; t += gridDim.x) {
-        int64_t bid = t;
-        if (bands) {
-            const int64_t xcd = t & 7, j = t >> 3, per = sh.gx >> 3, byb = j / per;
-            bid = byb * sh.gx + xcd * per + (j - byb * per);
-        }
-        const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+        const uint32_t bid = bands ? band_order(sh, (uint32_t)t) : (uint32_t)t;          // (fewer than 2^31 blocks)
+        uint32_t by32, bx32;
+        block_of(sh, bid, by32, bx32);
+        const int64_t by = by32, bx = bx32;
         const int64_t base = by * sh.brows * row_stride + ((bx * sh.bcols) >> 3);
         uint4 v[NV];
         bool ok[NV];
@@ -756,7 +754,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             v[k] = make_uint4(0, 0, 0, 0);
-            if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_in(nchunks * 8));
+            if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_last_read(nchunks * 8));
         }
         uint32_t slow = 0;
 #pragma unroll
@@ -899,7 +897,7 @@ __global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, 
         const int64_t c0 = tile * (NV * WG) + threadIdx.x;
         uint4 v[NV];
 #pragma unroll
-        for (int k = 0; k < NV; ++k) { v[k] = make_uint4(0, 0, 0, 0); if (c0 + k * WG < nvec) v[k] = load16_rt(in4 + c0 + k * WG, streams_in(n)); }
+        for (int k = 0; k < NV; ++k) { v[k] = make_uint4(0, 0, 0, 0); if (c0 + k * WG < nvec) v[k] = load16_rt(in4 + c0 + k * WG, streams_last_read(n)); }
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
@@ -991,7 +989,7 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
                              double e4m3_threshold, int64_t ss_mode, void* workspace, uint32_t flags, void* stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool emu = flags & MOR_FLAG_TORCH_EMULATION;
-    Shape sh{rows, cols, brows, bcols, rows / brows, cols / bcols};
+    const Shape sh = make_shape(rows, cols, brows, bcols);
     const int64_t nb = sh.gy * sh.gx;
     uint32_t* ws = static_cast<uint32_t*>(workspace);
     float* blocks = reinterpret_cast<float*>(ws + WS_BLOCKS);

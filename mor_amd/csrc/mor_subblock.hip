@@ -43,7 +43,7 @@ __global__ __launch_bounds__(WG) void k_subblock(const uint4* in, uint4* out, in
     const int rows_valid = (int)min(sh.brows, sh.rows - r0);
     const int cols_valid = (int)min((int64_t)cpr, (sh.cols - c0) >> 3);
     const int nchb = (int)sh.brows * cpr;
-    const bool nt_in = streams_in(sh.rows * sh.cols), nt_out = streams_out(sh.rows * sh.cols);
+    const bool nt_in = streams_last_read(sh.rows * sh.cols), nt_out = streams_out(sh.rows * sh.cols);
 
     uint4 v[NV];
     uint32_t off[NV];
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(WG) void k_subblock(const uint4* in, uint4* out, in
     if (valid && !hard) {
         if (l == 0) {
             if (meta && meta_val >= 0) meta[bid] = meta_val;
-            if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+            if (stats) { float* s = stats + 4 * (int64_t)bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
         }
         // pass 3: quantize and store, FQ:733-851
         if (out) {
@@ -114,12 +114,13 @@ __global__ __launch_bounds__(WG) void k_subblock(const uint4* in, uint4* out, in
                 }
             } else if (!E8 && (fmt == FMT_E4M3 || fmt == FMT_E5M2)) {
                 const float r4 = 1.0f / s4.s;            // 1 / s5 = r4 / 128 exactly
+                uint32_t qcodes = 0;
                 if (fmt == FMT_E4M3) {
 #pragma unroll
-                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_div<FMT_E4M3>(v[k], s4.s, r4), nt_out);
+                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_div<FMT_E4M3>(v[k], s4.s, r4, qcodes), nt_out);
                 } else {
 #pragma unroll
-                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f), nt_out);
+                    for (int k = 0; k < NV; ++k) if (ok[k]) store16_rt(bout + off[k], fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f, qcodes), nt_out);
                 }
             } else {
                 const Scale sc = make_scale(fmax_of(fmt) / amax);
@@ -167,7 +168,9 @@ __global__ __launch_bounds__(BIG_WG) void k_bigblock(const uint4* in, uint4* out
     __shared__ uint32_t s_u[NW];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t bid = first + blockIdx.x;
-    const int64_t by = bid / sh.gx, bx = bid - by * sh.gx;
+    uint32_t by32, bx32;
+    block_of(sh, (uint32_t)bid, by32, bx32);                  // (fewer than 2^31 blocks)
+    const int64_t by = by32, bx = bx32;
     const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
     const uint32_t row_stride = (uint32_t)(sh.cols >> 3);          // chunks per tensor row
     const uint4* bin = in + (r0 * row_stride + (c0 >> 3));
@@ -266,12 +269,12 @@ __global__ __launch_bounds__(BIG_WG) void k_bigblock(const uint4* in, uint4* out
     }
     if (tid == 0) {
         if (meta && meta_val >= 0) meta[bid] = meta_val;
-        if (stats) { float* s = stats + 4 * bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+        if (stats) { float* s = stats + 4 * (int64_t)bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
     }
     if (!out) return;
 
     // pass 3: quantize and store, FQ:733-851 (the last read of the block: streamed when the tensor streams)
-    const bool nt_in = streams_in(sh.rows * sh.cols), nt_out = streams_out(sh.rows * sh.cols);
+    const bool nt_in = streams_last_read(sh.rows * sh.cols), nt_out = streams_out(sh.rows * sh.cols);
     if ((fmt < 0) || !(amax > 0.0f)) {
         if (out != in) sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, v, nt_out); });
         return;
@@ -279,8 +282,9 @@ __global__ __launch_bounds__(BIG_WG) void k_bigblock(const uint4* in, uint4* out
     if constexpr (!E8) {
         if (fmt == FMT_E4M3 || fmt == FMT_E5M2) {
             const float r4 = 1.0f / s4.s;            // 1 / s5 = r4 / 128 exactly
-            if (fmt == FMT_E4M3) sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_div<FMT_E4M3>(v, s4.s, r4), nt_out); });
-            else sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_div<FMT_E5M2>(v, s5.s, r4 * 0.0078125f), nt_out); });
+            uint32_t qcodes = 0;
+            if (fmt == FMT_E4M3) sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_div<FMT_E4M3>(v, s4.s, r4, qcodes), nt_out); });
+            else sweep(nt_in, [&](uint4 v, uint32_t off) { store16_rt(bout + off, fq_vec_div<FMT_E5M2>(v, s5.s, r4 * 0.0078125f, qcodes), nt_out); });
             return;
         }
     }

@@ -1,0 +1,241 @@
+// k_wgblock: one workgroup per quantization block held in registers (the kernel template; its launchers are in
+// mor_wgblock.hip).  "FQ" below is the reference file mor/csrc/cuda/fake_quantize.cu.
+#pragma once
+
+#include "mor_quant.h"
+
+namespace mor {
+
+// k_wgblock: one workgroup per quantization block, the block held in registers (NV 16-byte vectors per lane).
+// Chunk ch = k * 256 + tid of the block sits at block row ch / cpr, chunk column ch % cpr.
+// MOR: per-block format selection (FQ:610-682), else one forced format.  FULL: every block is complete and has
+// exactly NV * 256 chunks, so no predicates.  NT: streaming loads and stores.  Blocks outside the fast range go
+// through generic_block.  WGS threads per workgroup: 256, or 512 for one-row blocks of more than 8192 elements.
+// GATHER: the block's elements are read and written pair by pair (odd column counts, pointers or block widths that are
+// not multiples of 16 bytes): a lane's words are pairs of neighbouring elements of a row; every later step is
+// elementwise, so nothing else changes.
+template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false>
+__global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
+                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift,
+                                                 int64_t first) {
+    constexpr int NW = WGS / 64;
+    __shared__ float s_f[2][NW];
+    __shared__ uint32_t s_u[NW];
+    __shared__ float s_e[2][NW];           // the error sums have slots of their own: no barrier between pass 1's readers and pass 2's writers
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // Workgroup -> block.  cpr_shift bit 8 (large tensors whose block grid is a multiple of 8 wide): consecutive
+    // workgroup ids go round the 8 XCDs, and each XCD takes a band of gx / 8 block columns, walking it row by row.
+    uint32_t bid = (uint32_t)(first + blockIdx.x);       // (a launch holds a slice of the blocks, see for_slices; fewer than 2^31 blocks)
+    if (cpr_shift >= 256) {            // (a negative cpr_shift means a chunk count per row that is not a power of two)
+        bid = band_order(sh, bid);
+        cpr_shift &= 255;
+        if (cpr_shift == 255) cpr_shift = -1;
+    }
+    uint32_t by32, bx32;
+    block_of(sh, bid, by32, bx32);
+    const int64_t by = by32, bx = bx32;
+    const int64_t r0 = by * sh.brows, c0 = bx * sh.bcols;
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3);          // chunks per tensor row
+    const uint4* bin = in + (r0 * row_stride + (c0 >> 3));
+    uint4* bout = out ? out + (r0 * row_stride + (c0 >> 3)) : nullptr;
+    const int rows_valid = (int)min(sh.brows, sh.rows - r0);
+    const int cols_valid = (int)min((int64_t)cpr, (sh.cols - c0) >> 3);
+    const int nch = (int)sh.brows * cpr;
+
+    uint4 v[NV];
+    uint32_t off[NV];
+    bool ok[NV];
+    // GATHER: word s of a lane is pair s * WGS + tid of the block's valid part, pairs counted row by row (the last pair of
+    // a row of odd width has one element); the walk advances by WGS pairs per word, without a division per word.  A pair
+    // is one 4-byte access at a 2-byte-aligned address.
+    typedef uint32_t u32_a2 __attribute__((aligned(2)));
+    const int g_bw = (int)min(sh.bcols, sh.cols - c0);
+    const int g_pr = (g_bw + 1) >> 1;                                   // pairs per row
+    const int g_step_r = WGS / g_pr, g_step_c = WGS % g_pr;
+    const uint32_t g_cols = (uint32_t)sh.cols;
+    if constexpr (GATHER) {
+        const uint16_t* src = reinterpret_cast<const uint16_t*>(in) + (r0 * sh.cols + c0);
+        int r = tid / g_pr, cp = tid - r * g_pr;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            ok[k] = true;
+            off[k] = 0;
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                w[j] = 0;
+                if (r < rows_valid) {
+                    const uint16_t* p = src + ((uint32_t)r * g_cols + 2u * (uint32_t)cp);
+                    w[j] = (2 * cp + 1 < g_bw) ? *reinterpret_cast<const u32_a2*>(p) : (uint32_t)*p;
+                }
+                r += g_step_r; cp += g_step_c;
+                if (cp >= g_pr) { cp -= g_pr; ++r; }
+            }
+            v[k] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    } else {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        int ch = k * WGS + tid;
+        int r = cpr_shift >= 0 ? (ch >> cpr_shift) : (ch / cpr);
+        int cc = ch - r * cpr;
+        ok[k] = FULL || ((ch < nch) && (r < rows_valid) && (cc < cols_valid));
+        off[k] = (uint32_t)r * row_stride + (uint32_t)cc;
+        if (ok[k]) v[k] = load16<(NT == 1)>(bin + off[k]);
+    }
+    }
+    // the store of one result vector (GATHER: pair by pair along the same walk, which `put` is called in order of)
+    int g_r = tid / g_pr, g_cp = tid - g_r * g_pr;
+    auto put = [&](int k, uint4 q) {
+        if constexpr (GATHER) {
+            uint16_t* dst = reinterpret_cast<uint16_t*>(out) + (r0 * sh.cols + c0);
+            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (g_r < rows_valid) {
+                    uint16_t* p = dst + ((uint32_t)g_r * g_cols + 2u * (uint32_t)g_cp);
+                    if (2 * g_cp + 1 < g_bw) *reinterpret_cast<u32_a2*>(p) = w[j];
+                    else *p = (uint16_t)w[j];
+                }
+                g_r += g_step_r; g_cp += g_step_c;
+                if (g_cp >= g_pr) { g_cp -= g_pr; ++g_r; }
+            }
+        } else {
+            store16<(NT != 0)>(bout + off[k], q);
+        }
+    };
+
+    // pass 1 (registers): amax and min over non-zero magnitudes, FQ:407-485
+    // (packed 16-bit integer maxima / minima of both halves of a word; the data stays packed in its registers)
+    uint32_t amax2 = 0, amin2_m1 = AMIN2_INIT_M1;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+        if (ok[k]) {
+            acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+            if constexpr (MOR) { acc_amin_pk(amin2_m1, v[k].x); acc_amin_pk(amin2_m1, v[k].y); acc_amin_pk(amin2_m1, v[k].z); acc_amin_pk(amin2_m1, v[k].w); }
+            opaque(v[k]);
+        }
+    uint32_t amax_b = group_umax(amax_bits_of(amax2), 64);
+    uint32_t amin_m1 = AMIN_INIT_M1;
+    if constexpr (MOR) amin_m1 = group_umin(amin_m1_of(amin2_m1), 64);
+    if (lane == 0) { s_f[0][wave] = u2f(amax_b); s_u[wave] = amin_m1; }
+    __syncthreads();
+    amax_b = f2u(lds_umaxf<NW>(s_f[0]));
+    amin_m1 = lds_umin<NW>(s_u);
+    const float amax = u2f(amax_b);
+    const float amin = u2f(amin_m1 + 1u);
+
+    // scales of the two fp8 formats; the fp6 scales differ from s4 by 2^4 / 2^6, inside the margin of `fast`
+    // (57344 / amax is 128 * (448 / amax) exactly: one division for both)
+    const Scale s4 = make_scale(448.0f / amax);
+    Scale s5 = s4;
+    s5.s = s4.s * 128.0f;
+    s5.e8 = s4.e8 + 7;
+    // (a NaN in the block shows as amax_b above the bits of infinity: the exact path takes its maximum as the reference does)
+    if (amax_b > 0x7F800000u || (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast))) {           // uniform over the workgroup
+        generic_block<false, false, WGS>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
+                             sh, qa, E8, bid, s_f, s_u);
+        return;
+    }
+
+    int fmt = qa.fmt;
+    int meta_val = qa.meta_val;
+    float e4 = 0.0f, e5 = 0.0f;
+    if constexpr (MOR) {
+        int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
+        if (qt == Q_UNKNOWN) {
+            // pass 2 (registers): the two error sums, FQ:487-584.  amax > 0 here.
+            uint32_t codes = 0;
+#pragma unroll
+            for (int k = 0; k < NV; ++k)
+                if (ok[k]) {
+                    err_pair_fast<E8>(v[k].x, s4, e4, e5, codes);
+                    err_pair_fast<E8>(v[k].y, s4, e4, e5, codes);
+                    err_pair_fast<E8>(v[k].z, s4, e4, e5, codes);
+                    err_pair_fast<E8>(v[k].w, s4, e4, e5, codes);
+                }
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) opaque(v[k]);
+            e4 = wave_sum(e4);
+            e5 = wave_sum(e5);
+            if (lane == 0) { s_e[0][wave] = e4; s_e[1][wave] = e5; }
+            __syncthreads();
+            e4 = lds_sum<NW>(s_e[0]);
+            e5 = lds_sum<NW>(s_e[1]);
+            if (!(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) {
+                // The sums above divide with a Newton step.  When they are too close for that to be trusted with
+                // the decision, repeat them with IEEE divisions (from memory, non-unrolled: this is rare).
+                const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in);
+                const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
+                e4 = 0.0f; e5 = 0.0f;
+#pragma unroll 1
+                for (int64_t i = tid; i < bh * bw; i += WGS) {
+                    int64_t r = i / bw, c = i - r * bw;
+                    err_terms_exact<false>(bf16_one(in16[(r0 + r) * sh.cols + c0 + c]), E8, s4, s5, e4, e5);
+                }
+                e4 = wave_sum(e4);
+                e5 = wave_sum(e5);
+                __syncthreads();                 // every wave has read the first sums
+                if (lane == 0) { s_e[0][wave] = e4; s_e[1][wave] = e5; }
+                __syncthreads();
+                e4 = lds_sum<NW>(s_e[0]);
+                e5 = lds_sum<NW>(s_e[1]);
+            }
+            qt = mor_decide_error(amax, qa.clamp, e4, e5);
+        }
+        meta_val = qt;
+        fmt = mor_fmt_of(qt);
+    }
+    if (tid == 0) {
+        if (meta && meta_val >= 0) meta[bid] = meta_val;
+        if (stats) { float* s = stats + 4 * (int64_t)bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
+    }
+    if (!out) return;
+
+    // pass 3 (registers): quantize and store, FQ:733-851
+    if ((fmt < 0) || !(amax > 0.0f)) {
+        if (out != in) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) put(k, v[k]);
+        }
+        return;
+    }
+    if constexpr (!E8) {
+        if (fmt == FMT_E4M3 || fmt == FMT_E5M2) {
+            const float r4 = s4.r;                    // 1 / s5 = r4 / 128 exactly
+            uint32_t codes = 0;                       // (the converts write half of this register: carried from word to word)
+            if (fmt == FMT_E4M3) {
+#pragma unroll
+                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_div<FMT_E4M3>(v[k], s4.s, r4, codes));
+            } else {
+#pragma unroll
+                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f, codes));
+            }
+            return;
+        }
+    }
+    const Scale sc = make_scale(fmax_of(fmt) / amax);
+    switch (fmt) {
+        case FMT_E4M3:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_fast<FMT_E4M3, E8>(v[k], sc));
+            break;
+        case FMT_E5M2:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_fast<FMT_E5M2, E8>(v[k], sc));
+            break;
+        case FMT_E3M2:
+            if constexpr (!MOR) {
+#pragma unroll
+                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_fast<FMT_E3M2, E8>(v[k], sc));
+            }
+            break;
+        default:
+#pragma unroll
+            for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_fast<FMT_E2M3, E8>(v[k], sc));
+            break;
+    }
+}
+
+
+}  // namespace mor

@@ -151,7 +151,7 @@ __global__ __launch_bounds__(WWG) void k_mx_quantize(const uint4* in, uint8_t* p
     for (int k = 0; k < NV; ++k) {
         const int64_t c = base + k * WWG;
         v[k] = make_uint4(0, 0, 0, 0);
-        if (c < nchunks) v[k] = load16_rt(in + c, streams_in(nchunks * 8));
+        if (c < nchunks) v[k] = load16_rt(in + c, streams_last_read(nchunks * 8));
     }
 #pragma unroll
     for (int k = 0; k < NV; ++k) {

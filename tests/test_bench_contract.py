@@ -36,3 +36,8 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["unit"] == "GB/s" and cb["sample"]
     assert d["value"] > 100 * cb["value"] / 10          # a GPU, not the fallback of anything
+    # MX and MoR are both in the timed step; the roofline kernel is the one furthest below the roofline
+    pk = rf["per_kernel"]
+    assert {"mx_e4m3", "mx_e5m2", "mx_e2m3", "mor_128x128"} <= set(pk)
+    assert rf["kernel"] == min(("mx_e4m3", "mx_e5m2", "mx_e2m3", "mor_128x128"), key=lambda k: pk[k]["frac"])
+    assert "c1_per_tensor_e4m3_4096x4096" in cb["per_config"]
