@@ -20,7 +20,9 @@
 namespace mor {
 
 constexpr int WS_HEADER = 4;
-constexpr int MAX_PARTIALS = 8192;
+constexpr int MAX_PARTIALS = 8192;     // slots of each partial array in the workspace
+constexpr int PASS1_MAX = 1024;        // workgroups (= partials) of a pass-1 kernel: every pass-2 workgroup reduces them again
+constexpr int PASS2_MAX = 2048;        // workgroups (= error partials) of a pass-2 kernel: every workgroup of the last kernel adds them
 constexpr int WS_ERR = WS_HEADER;
 constexpr int WS_PAMAX = WS_HEADER + MAX_PARTIALS;
 constexpr int WS_PNNZ = WS_HEADER + 2 * MAX_PARTIALS;
@@ -278,24 +280,62 @@ __device__ __forceinline__ float scaling_factor(float global_amax, float block_a
     return sf;
 }
 
-// pass 1.5 (FQ:1017-1049 + the scale of every block): tensor amax and non-zero count from the partials into the
-// header, block amax -> block scale in place
-__global__ __launch_bounds__(WG) void k_bs_scales(uint32_t* ws, float* block_amax, int64_t nb, int ss_mode, int npart) {
-    __shared__ float s_f[WAVES];
-    __shared__ int s_i[WAVES];
-    const float gamax = reduce_partial_amax(ws, npart, s_f);
-    if (blockIdx.x == 0) {
-        const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
-        int n = 0;
-#pragma unroll 8
-        for (int i = threadIdx.x; i < npart; i += WG) n += pn[i];
-        n = wave_sum_i(n);
-        if ((threadIdx.x & 63) == 0) s_i[threadIdx.x >> 6] = n;
-        __syncthreads();
-        if (threadIdx.x == 0) { ws[0] = f2u(gamax); ws[1] = (uint32_t)(s_i[0] + s_i[1] + s_i[2] + s_i[3]); }
+// The scale of one block (FQ:1059-1093) from the tensor amax and the block's amax, computed where it is used: the
+// quantize kernels reduce the pass-1 partials to the tensor amax themselves (every workgroup, a few loads per thread)
+// instead of waiting for a kernel of its own to do that and to turn every block amax into a scale.  ss_mode 4 takes
+// the tensor amax alone; no per-block amax is kept for it.
+__device__ __forceinline__ float block_scale(float gamax, const float* block_amax, int64_t idx, int ss_mode) {
+    return scaling_factor(gamax, ss_mode == 4 ? 1.0f : block_amax[idx], ss_mode);
+}
+
+// The end of the op (FQ:1178-1241), evaluated by every workgroup of the kernel that acts on the decision (the gated
+// copy or the gated write) instead of by a one-workgroup kernel of its own: the error partials are added in a fixed
+// order (the same in every workgroup), the tensor amax and the non-zero count are reduced from the pass-1 partials,
+// workgroup 0 writes the scalar outputs.  Returns meta: 3 (bf16 fallback) or 1 (E4M3).
+struct Finish {
+    const uint32_t* ws;
+    int nerr, nstat;                  // error partials (pass 2), amax / non-zero partials (pass 1)
+    float threshold;
+    int32_t* meta;
+    float* gamax_o;
+    int32_t* gnnz_o;
+    float* gerr_o;
+};
+// (WGS: threads of the calling workgroup; the first 256 do the sums, so that the order of the additions does not depend
+// on the workgroup size; s_f: 8 floats, s_i: 4 ints of LDS)
+template <int WGS = WG>
+__device__ __forceinline__ int finish_decision(const Finish& f, float* s_f, int* s_i) {
+    const float* part = reinterpret_cast<const float*>(f.ws) + WS_ERR;
+    const float* pa = reinterpret_cast<const float*>(f.ws) + WS_PAMAX;
+    const int* pn = reinterpret_cast<const int*>(f.ws) + WS_PNNZ;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float acc = 0.0f, a = 0.0f;
+    int n = 0;
+    if (WGS == WG || threadIdx.x < WG) {
+#pragma unroll 4
+        for (int i = threadIdx.x; i < f.nerr; i += WG) acc += part[i];
+#pragma unroll 4
+        for (int i = threadIdx.x; i < f.nstat; i += WG) { a = fmaxf(a, pa[i]); n += pn[i]; }
     }
-    for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < nb; i += (int64_t)gridDim.x * WG)
-        block_amax[i] = scaling_factor(gamax, block_amax[i], ss_mode);
+    acc = wave_sum(acc);
+    a = group_max(a, 64);
+    n = wave_sum_i(n);
+    __syncthreads();
+    if (lane == 0 && wave < WAVES) { s_f[wave] = acc; s_f[4 + wave] = a; s_i[wave] = n; }
+    __syncthreads();
+    const float gerr = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+    const float gamax = fmaxf(fmaxf(s_f[4], s_f[5]), fmaxf(s_f[6], s_f[7]));
+    const int gnnz = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    const float avg = gerr / (float)gnnz;        // 0 / 0 = NaN on an all-zero tensor: not above the threshold
+    const int m = (avg > f.threshold) ? 3 : 1;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+        f.meta[0] = m;
+        f.gamax_o[0] = gamax;
+        f.gnnz_o[0] = gnnz;
+        f.gerr_o[0] = gerr;
+    }
+    __syncthreads();
+    return m;
 }
 
 // One element of FQ:1133-1162: zeros give +0 and no error; others E4M3 through the hardware-cast model.
@@ -349,14 +389,17 @@ __device__ __forceinline__ uint4 bs_vec_fast(uint4 v, const Scale& sc, float& er
     return q;
 }
 
-// pass 2 / pass 4: quantize every element with its block's scale (looked up per chunk, or per column in column
-// mode), accumulate the relative error, optionally write.  GATE > 0: run only if meta[0] == GATE.
+// pass 2 / pass 4: quantize every element with its block's scale (from the block's amax, per chunk, or per column in
+// column mode), accumulate the relative error, optionally write.  gate > 0: the gated write of the in-place op: the
+// decision is evaluated first (finish_decision) and the pass runs only if it is `gate`.
 template <bool E8, bool EMU, bool COL, bool WRITE, bool ERR>
 __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* out, uint32_t* ws, const float* scales,
-                                                 const int32_t* meta, int gate, Shape sh, int vec, DivU32 d_rowchunks,
+                                                 Finish fin, int gate, int ss_mode, int npart1, Shape sh, int vec, DivU32 d_rowchunks,
                                                  DivU32 d_brows, DivU32 d_bchunks, DivU32 d_bcols) {
-    __shared__ float s_f[WAVES];
-    if (gate > 0 && meta[0] != gate) return;
+    __shared__ float s_f[2 * WAVES];
+    __shared__ int s_i[WAVES];
+    if (gate > 0 && finish_decision(fin, s_f, s_i) != gate) return;
+    const float gamax = reduce_partial_amax(ws, npart1, s_f);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float err = 0.0f;
     if (vec) {
@@ -370,17 +413,17 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
             uint4 v = load16_rt(in4 + c, streams_last_read(sh.rows * sh.cols));
             uint32_t w[4] = {v.x, v.y, v.z, v.w};
             if constexpr (COL) {
-                const float* sp = scales + (int64_t)by * sh.cols + (int64_t)cc * 8;
+                const int64_t sp = (int64_t)by * sh.cols + (int64_t)cc * 8;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const Scale s0 = make_scale(sp[2 * j]), s1 = make_scale(sp[2 * j + 1]);
+                    const Scale s0 = make_scale(block_scale(gamax, scales, sp + 2 * j, ss_mode)), s1 = make_scale(block_scale(gamax, scales, sp + 2 * j + 1, ss_mode));
                     float q0 = bs_element<E8, EMU>(bf16_lo(w[j]), s0, err);
                     float q1 = bs_element<E8, EMU>(bf16_hi(w[j]), s1, err);
                     w[j] = store_pair<EMU>(q0, q1);
                 }
             } else {
                 const uint32_t bx = div_u32(cc, d_bchunks);
-                const Scale sc = make_scale(scales[(int64_t)by * sh.gx + bx]);
+                const Scale sc = make_scale(block_scale(gamax, scales, (int64_t)by * sh.gx + bx, ss_mode));
                 if (!EMU && sc.fast && !vec_has_nan(v)) {
                     const float rs = 1.0f / sc.s;
 #pragma unroll
@@ -401,13 +444,14 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
         for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG) {
             const int64_t row = i / sh.cols, col = i - row * sh.cols;
             const int64_t by = row / sh.brows, bx = col / sh.bcols;
-            const Scale sc = make_scale(scales[by * sh.gx + bx]);
+            const Scale sc = make_scale(block_scale(gamax, scales, by * sh.gx + bx, ss_mode));
             float q = bs_element<E8, EMU>(bf16_one(in[i]), sc, err);
             if constexpr (WRITE) out[i] = store_bf16<EMU>(q);
         }
     }
     if constexpr (ERR) {
         err = wave_sum(err);
+        __syncthreads();                   // every wave has read the tensor amax from these slots
         if (lane == 0) s_f[wave] = err;
         __syncthreads();
         if (threadIdx.x == 0) {
@@ -421,9 +465,11 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
 // not all in the fast range use the exact arithmetic.
 template <bool WRITE, bool ERR>
 __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_t* out, uint32_t* ws, const float* scales,
-                                                     const int32_t* meta, int gate, Shape sh, int rows_per_wg) {
-    __shared__ float s_f[WAVES];
-    if (gate > 0 && meta[0] != gate) return;
+                                                     Finish fin, int gate, int ss_mode, int npart1, Shape sh, int rows_per_wg) {
+    __shared__ float s_f[2 * WAVES];
+    __shared__ int s_i[WAVES];
+    if (gate > 0 && finish_decision(fin, s_f, s_i) != gate) return;
+    const float gamax = reduce_partial_amax(ws, npart1, s_f);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t col0 = ((int64_t)blockIdx.x * WG + threadIdx.x) * 8;
     const int64_t segs_per_block = (sh.brows + rows_per_wg - 1) / rows_per_wg;
@@ -437,12 +483,12 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
             const int64_t by = seg / segs_per_block;
             const int64_t r_begin = by * sh.brows + (seg - by * segs_per_block) * rows_per_wg;
             const int64_t r_end = min(r_begin + rows_per_wg, (by + 1) * sh.brows);
-            const float* sp = scales + by * sh.cols + col0;
+            const int64_t sp = by * sh.cols + col0;
             Scale sc[8];
             float rs[8];
             bool fast = true;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) { sc[j] = make_scale(sp[j]); rs[j] = 1.0f / sc[j].s; fast = fast && sc[j].fast; }
+            for (int j = 0; j < 8; ++j) { sc[j] = make_scale(block_scale(gamax, scales, sp + j, ss_mode)); rs[j] = sc[j].r; fast = fast && sc[j].fast; }
             if (fast) {
 #pragma unroll 1
                 for (int64_t r = r_begin; r < r_end; r += 4) {
@@ -493,9 +539,8 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
                     uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const float s0 = sp[2 * j], s1 = sp[2 * j + 1];
-                        float q0 = bs_element<false, false>(bf16_lo(w[j]), make_scale(s0), err);
-                        float q1 = bs_element<false, false>(bf16_hi(w[j]), make_scale(s1), err);
+                        float q0 = bs_element<false, false>(bf16_lo(w[j]), sc[2 * j], err);
+                        float q1 = bs_element<false, false>(bf16_hi(w[j]), sc[2 * j + 1], err);
                         w[j] = store_pair<false>(q0, q1);
                     }
                     if constexpr (WRITE) out4[r * row_stride + (col0 >> 3)] = make_uint4(w[0], w[1], w[2], w[3]);
@@ -505,70 +550,11 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
     }
     if constexpr (ERR) {
         err = wave_sum(err);
+        __syncthreads();                   // every wave has read the tensor amax from these slots
         if (lane == 0) s_f[wave] = err;
         __syncthreads();
         if (threadIdx.x == 0)
             reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x + gridDim.x * blockIdx.y] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
-    }
-}
-
-// pass 3 (FQ:1178-1241): total error (fixed summation order), the bf16 decision, the scalar outputs.
-// npart_stats > 0: the tensor amax and the non-zero count are still per-workgroup partials (single-pass kernel)
-// and are reduced here; otherwise they are in the header words.
-__global__ __launch_bounds__(WG) void k_bs_finalize(const uint32_t* ws, int npartials, int npart_stats, float threshold,
-                                                    int32_t* meta, float* gamax_o, int32_t* gnnz_o, float* gerr_o) {
-    __shared__ float s_f[WAVES];
-    __shared__ int s_i[WAVES];
-    const float* part = reinterpret_cast<const float*>(ws) + WS_ERR;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    float gamax = u2f(ws[0]);
-    int gnnz = (int)ws[1];
-    float acc = 0.0f;
-    if (npart_stats > 0 && npart_stats == npartials) {
-        // the three partial arrays in one sweep, all loads of a batch in flight (three sweeps in a row were 6.4 us
-        // of one workgroup's load latency); every sum keeps the order of the separate sweeps
-        const float* pa = reinterpret_cast<const float*>(ws) + WS_PAMAX;
-        const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
-        float a = 0.0f;
-        int n = 0;
-#pragma unroll 8
-        for (int i = threadIdx.x; i < npartials; i += WG) {
-            a = fmaxf(a, pa[i]);
-            n += pn[i];
-            acc += part[i];
-        }
-        a = group_max(a, 64);
-        n = wave_sum_i(n);
-        if (lane == 0) { s_f[wave] = a; s_i[wave] = n; }
-        __syncthreads();
-        gamax = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
-        gnnz = s_i[0] + s_i[1] + s_i[2] + s_i[3];
-    } else {
-        if (npart_stats > 0) {
-            gamax = reduce_partial_amax(ws, npart_stats, s_f);
-            const int* pn = reinterpret_cast<const int*>(ws) + WS_PNNZ;
-            int n = 0;
-#pragma unroll 8
-            for (int i = threadIdx.x; i < npart_stats; i += WG) n += pn[i];
-            n = wave_sum_i(n);
-            if (lane == 0) s_i[wave] = n;
-            __syncthreads();
-            gnnz = s_i[0] + s_i[1] + s_i[2] + s_i[3];
-        }
-#pragma unroll 8
-        for (int i = threadIdx.x; i < npartials; i += WG) acc += part[i];
-    }
-    acc = wave_sum(acc);
-    __syncthreads();
-    if (lane == 0) s_f[wave] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const float gerr = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
-        const float avg = gerr / (float)gnnz;        // 0 / 0 = NaN on an all-zero tensor: not above the threshold
-        meta[0] = (avg > threshold) ? 3 : 1;
-        gamax_o[0] = gamax;
-        gnnz_o[0] = gnnz;
-        gerr_o[0] = gerr;
     }
 }
 
@@ -580,7 +566,7 @@ __global__ __launch_bounds__(WG) void k_bs_finalize(const uint32_t* ws, int npar
 // exact arithmetic.
 template <bool E8, int NV, bool FULL, int WGS = WG>
 __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, uint32_t* ws, Shape sh, int ss_mode,
-                                                 int cpr, int cpr_shift, int64_t nblocks, const int32_t* meta, int phase) {
+                                                 int cpr, int cpr_shift, int64_t nblocks, Finish fin, int phase, int npart1) {
     constexpr int NW = WGS / 64, LG = WGS == 256 ? 8 : WGS == 512 ? 9 : 10;       // waves; log2 of the workgroup size
     __shared__ float s_f[NW];
     __shared__ int s_i[NW];
@@ -588,8 +574,16 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
     auto red_fsum = [&]() { if constexpr (NW == 4) return (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]); else return lds_sum<NW>(s_f); };
     auto red_fmax = [&]() { if constexpr (NW == 4) return fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3])); else return lds_fmax<NW>(s_f); };
     // phase 0: out of place (write and publish the partials); in place the input must survive until the decision:
-    // phase 1 publishes the partials without writing, phase 2 writes if the decision was E4M3 (meta[0] == 1)
-    if (phase == 2 && meta[0] != 1) return;
+    // phase 1 publishes the partials without writing, phase 2 evaluates the decision and writes if it was E4M3
+    if (phase == 2) {
+        __shared__ float s_d[2 * WAVES];
+        __shared__ int s_di[WAVES];
+        if (finish_decision<WGS>(fin, s_d, s_di) != 1) return;
+    }
+    // npart1 > 0: the strategies that take the tensor amax (ss_mode 1 and 4) after a pass that found it; the amax and
+    // non-zero partials of that pass stand, this kernel then publishes error partials only
+    const float gamax = npart1 > 0 ? reduce_partial_amax(ws, npart1, s_f) : 0.0f;
+    __syncthreads();
     const bool write = phase != 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t row_stride = (uint32_t)(sh.cols >> 3);
@@ -670,7 +664,7 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
         }
         gmax = fmaxf(gmax, amax);
         nnz_total += (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
-        const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
+        const Scale sc = make_scale(scaling_factor(gamax, amax, ss_mode));
         if (!has_nan && (sc.fast || !(amax > 0.0f))) {          // an all-zero block gives +0 whatever its (clamped) scale is
             // For large blocks every vector is finished before the next begins (register barriers): otherwise the
             // compiler hoists work from all of them, and sinks the whole chain of error terms below the last store
@@ -726,8 +720,10 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
     __syncthreads();
     if (tid == 0 && phase != 2) {
         reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = e;
-        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
-        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = red_fmax();
+        if (npart1 == 0) {
+            reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
+            reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = red_fmax();
+        }
     }
 }
 
@@ -735,12 +731,18 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
 // the flat chunk array in tiles of 4 * 256 chunks, a block is G consecutive lanes (amax by DPP), as in k_rowgroup.
 // Groups whose scale is outside the fast range are redone from memory by a second, non-unrolled loop.
 constexpr int BS_ROWS_NV = 4;         // vectors per lane and tile (2 is not faster here: 55.9 against 54.5 us)
-template <bool E8>
+// GM: 0 = the scale depends on the block alone (ss_mode 2 / 3; this kernel also publishes the amax and non-zero partials),
+// 1 = tensor-amax mantissa shared by the blocks (ss_mode 1), 2 = one scale for the tensor (ss_mode 4: G is 1 whatever
+// the block shape is); for 1 and 2 a pass over the tensor has left its amax and non-zero partials (npart1 of them).
+template <bool E8, int GM>
 __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* out, uint32_t* ws, int64_t nchunks, int G, int ss_mode,
-                                                      const int32_t* meta, int phase) {
-    __shared__ float s_f[WAVES];
+                                                      Finish fin, int phase, int npart1) {
+    __shared__ float s_f[2 * WAVES];
     __shared__ int s_i[WAVES];
-    if (phase == 2 && meta[0] != 1) return;          // phases as in k_bs_fused
+    if (phase == 2 && finish_decision(fin, s_f, s_i) != 1) return;          // phases as in k_bs_fused
+    const float gamax = GM != 0 ? reduce_partial_amax(ws, npart1, s_f) : 0.0f;
+    __syncthreads();
+    const Scale scu = make_scale(scaling_factor(gamax, 1.0f, 4));           // (GM == 2)
     const bool write = phase != 1;
     constexpr int NV = BS_ROWS_NV;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -756,36 +758,44 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
             v[k] = make_uint4(0, 0, 0, 0);
             if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_last_read(nchunks * 8));
         }
-        uint32_t slow = 0;
+        uint32_t slow = 0, nnz2 = 0;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const int64_t c = base + k * WG;
-            float amax = 0.0f;
-            acc_amax_nnz(amax, nnz, v[k]);
-            amax = group_max(amax, G);
-            gmax = fmaxf(gmax, amax);
-            const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
+            // the block maximum on packed 16-bit magnitudes; a NaN wins it and sends the block to the exact arithmetic
+            uint32_t amax2 = 0;
+            acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+            if constexpr (GM == 0) { acc_nnz_pk(nnz2, v[k].x); acc_nnz_pk(nnz2, v[k].y); acc_nnz_pk(nnz2, v[k].z); acc_nnz_pk(nnz2, v[k].w); }
+            const uint32_t amax_b = group_umax(amax_bits_of(amax2), G);
+            const bool has_nan = amax_b > 0x7F800000u;
+            const float amax = u2f(amax_b);
+            if constexpr (GM == 0) { if (!has_nan) gmax = fmaxf(gmax, amax); }
+            const Scale sc = GM == 2 ? scu : make_scale(scaling_factor(gamax, amax, ss_mode));
             float e = 0.0f;
             uint4 q;
             if (phase == 1) q = bs_vec_fast<E8, true, false>(v[k], sc, e);          // in place: decision pass,
             else if (phase == 2) q = bs_vec_fast<E8, false, true>(v[k], sc, e);     // write pass
             else q = bs_vec_fast<E8, true, true>(v[k], sc, e);
-            const bool has_nan = group_umax(vec_has_nan(v[k]) ? 1u : 0u, G) != 0u;          // exact arithmetic for such a block
             if (!has_nan && (sc.fast || !(amax > 0.0f))) {      // an all-zero block gives +0 whatever its (clamped) scale is
                 err += e;
                 if (c < nchunks && write) store16_rt(out + c, q, nt);
             } else if (c < nchunks) slow |= 1u << k;
         }
+        nnz += (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
         if (slow) {
 #pragma unroll 1
             for (int k = 0; k < NV; ++k) {
                 if (!((slow >> k) & 1u)) continue;              // uniform over the lanes of a group
                 const int64_t c = base + k * WG;
                 const uint4 x = in[c];
-                float amax = 0.0f;
+                float amax = 0.0f;                               // the float maximum skips a NaN, as the reference's does
                 acc_amax(amax, x.x); acc_amax(amax, x.y); acc_amax(amax, x.z); acc_amax(amax, x.w);
                 amax = group_max(amax, G);
-                const Scale sc = make_scale(scaling_factor(0.0f, amax, ss_mode));
+                if constexpr (GM == 0) {
+                    gmax = fmaxf(gmax, amax);
+                    nnz -= nan_word(x.x) + nan_word(x.y) + nan_word(x.z) + nan_word(x.w);      // the packed count took them for non-zero values
+                }
+                const Scale sc = make_scale(scaling_factor(gamax, amax, ss_mode));
                 uint32_t w[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
@@ -806,14 +816,19 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
     __syncthreads();
     if (tid == 0 && phase != 2) {
         reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = e;
-        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
-        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        if constexpr (GM == 0) {
+            reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
+            reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+        }
     }
 }
 
-// pass 4 for the out-of-place ops (FQ:1217-1235): copy the input over the quantized output when meta[0] == 3
-__global__ __launch_bounds__(WG) void k_copy_if(const uint16_t* in, uint16_t* out, const int32_t* meta, int gate, int64_t n, int64_t nvec) {
-    if (meta[0] != gate) return;
+// The end of the out-of-place ops (FQ:1178-1241): the decision, and the input copied over the quantized output when it
+// is the bf16 fallback
+__global__ __launch_bounds__(WG) void k_copy_if(const uint16_t* in, uint16_t* out, Finish fin, int64_t n, int64_t nvec) {
+    __shared__ float s_f[2 * WAVES];
+    __shared__ int s_i[WAVES];
+    if (finish_decision(fin, s_f, s_i) != 3) return;
     const int64_t stride = (int64_t)gridDim.x * WG;
     const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
     const uint4* in4 = reinterpret_cast<const uint4*>(in);
@@ -929,17 +944,17 @@ extern "C" size_t mor_workspace_bytes(int op, int64_t rows, int64_t cols, int64_
 
 template <bool E8, bool EMU, bool COL>
 static void launch_bs_quant(bool write, bool err, int grid, hipStream_t st, const uint16_t* in, uint16_t* out, uint32_t* ws,
-                            const float* scales, const int32_t* meta, int gate, const Shape& sh, int vec,
+                            const float* scales, const Finish& fin, int gate, int ss_mode, int npart1, const Shape& sh, int vec,
                             DivU32 d0, DivU32 d1, DivU32 d2, DivU32 d3) {
-    if (write && err) k_bs_quant<E8, EMU, COL, true, true><<<grid, WG, 0, st>>>(in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3);
-    else if (write) k_bs_quant<E8, EMU, COL, true, false><<<grid, WG, 0, st>>>(in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3);
-    else k_bs_quant<E8, EMU, COL, false, true><<<grid, WG, 0, st>>>(in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3);
+    if (write && err) k_bs_quant<E8, EMU, COL, true, true><<<grid, WG, 0, st>>>(in, out, ws, scales, fin, gate, ss_mode, npart1, sh, vec, d0, d1, d2, d3);
+    else if (write) k_bs_quant<E8, EMU, COL, true, false><<<grid, WG, 0, st>>>(in, out, ws, scales, fin, gate, ss_mode, npart1, sh, vec, d0, d1, d2, d3);
+    else k_bs_quant<E8, EMU, COL, false, true><<<grid, WG, 0, st>>>(in, out, ws, scales, fin, gate, ss_mode, npart1, sh, vec, d0, d1, d2, d3);
 }
 
 static void dispatch_bs_quant(bool e8, bool emu, bool col, bool write, bool err, int grid, hipStream_t st, const uint16_t* in,
-                              uint16_t* out, uint32_t* ws, const float* scales, const int32_t* meta, int gate, const Shape& sh,
-                              int vec, DivU32 d0, DivU32 d1, DivU32 d2, DivU32 d3) {
-#define BSQ(E8, EMU, COL) launch_bs_quant<E8, EMU, COL>(write, err, grid, st, in, out, ws, scales, meta, gate, sh, vec, d0, d1, d2, d3)
+                              uint16_t* out, uint32_t* ws, const float* scales, const Finish& fin, int gate, int ss_mode, int npart1,
+                              const Shape& sh, int vec, DivU32 d0, DivU32 d1, DivU32 d2, DivU32 d3) {
+#define BSQ(E8, EMU, COL) launch_bs_quant<E8, EMU, COL>(write, err, grid, st, in, out, ws, scales, fin, gate, ss_mode, npart1, sh, vec, d0, d1, d2, d3)
     if (e8) {
         if (emu) { if (col) BSQ(true, true, true); else BSQ(true, true, false); }
         else { if (col) BSQ(true, false, true); else BSQ(true, false, false); }
@@ -999,126 +1014,147 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
     const int vec = (aligned16(input) && aligned16(output) && cols % 8 == 0) ? 1 : 0;
     const bool col = (bcols == 1 && brows > 1);
 
+    // The launches: pass 1 (amax / non-zero partials, block amax), pass 2 (quantize, error partials), and the end of the
+    // op in the workgroups of the kernel that acts on the decision (out of place: the gated copy; in place: the gated
+    // write).  The grids of pass 1 and pass 2 are capped (PASS1_MAX / PASS2_MAX workgroups, grid-stride): every
+    // workgroup of the following kernel reduces their partials again.
+    Finish fin{ws, 0, 0, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error};
+    const int64_t n = rows * cols;
+    const int64_t nvec_all = vec ? n / 8 : 0;
+    auto gated_copy = [&]() { k_copy_if<<<grid_for(nvec_all > 0 ? nvec_all : n, 4), WG, 0, st>>>(in16, out16, fin, n, nvec_all); };
+
     // block-local scales: one pass out of place; in place one pass for the decision and one gated pass that writes
     const int64_t blk_chunks = (bcols % 8 == 0) ? brows * (bcols / 8) : 0;
     // (a decision pass that computes no output words and a write pass that computes no error terms; 128 x 128 blocks
     // in place at 8192^2: 83 us against 99 through the general three-pass path; blocks that fill less than a workgroup
     // take the general path)
-    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && blk_chunks >= WG && blk_chunks <= 8 * 1024
+    // The strategies that take the tensor amax (ss_mode 1 and 4) run the same kernels after a pass over the flat tensor
+    // that finds it: the blocks' own maxima come from the registers of the quantize pass, no per-block array is kept.
+    // ss_mode 4 needs no block maxima at all and takes the flat row kernel whatever the block shape is.
+    const bool global = (ss_mode == 1 || ss_mode == 4);
+    int npart1 = 0;
+    auto tensor_amax_pass = [&]() {
+        npart1 = (int)std::min<int64_t>(cdiv(n / 8, 8 * WG), PASS1_MAX);
+        k_bs_amax_flat<<<npart1, WG, 0, st>>>(static_cast<const uint4*>(input), ws, nullptr, n / 8, 1, 0);
+    };
+    const bool flat_ok = !emu && vec && n % 8 == 0;
+    if (flat_ok && !col && ss_mode != 4 && blk_chunks >= WG && blk_chunks <= 8 * 1024
         && brows * (cols / 8) < 0x7FFFFFFFll && (is_pow2(bcols / 8) || brows == 1)) {
+        if (global) tensor_amax_pass();
         const int cpr = (int)(bcols / 8);
         const int nv = (int)cdiv(blk_chunks, WG);
         const int NVc = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
         // up to 8 * 256 chunks: 256 threads; up to 32768 / 65536 elements: 8 vectors per lane of 512 / 1024 threads
         const int wgs = blk_chunks <= 8 * WG ? WG : blk_chunks <= 8 * 512 ? 512 : 1024;
         const bool full = blk_chunks == (int64_t)(wgs == WG ? NVc : 8) * wgs;
-        const int grid = (int)std::min<int64_t>(nb, 4096);      // partials: one per workgroup (the finalize kernel reads them all)
-        // tensors beyond the last-level cache: XCD bands of block columns (16384 x 14336, 128 x 128 blocks: 193 -> 185 us)
-        const bool bands = rows * cols > ((int64_t)128 << 20) && sh.gx % 8 == 0 && grid % 8 == 0 && nb % 8 == 0;
+        int grid = (int)std::min<int64_t>(nb, PASS2_MAX);      // partials: one per workgroup
+        // tensors that come from HBM: XCD bands of block columns (16384 x 14336, 128 x 128 blocks: 193 -> 185 us)
+        const bool bands = rows * cols >= ((int64_t)16 << 20) && sh.gx % 8 == 0 && nb % 8 == 0;
+        if (bands) grid &= ~7;
+        fin.nerr = grid;
+        fin.nstat = global ? npart1 : grid;
         // a one-row block is contiguous whatever its width: chunk k * 256 + tid is at that offset (shift 20: row 0 always)
         const int shift = (brows == 1 ? 20 : ilog2(cpr)) | (bands ? 256 : 0);
         const uint4* i4 = static_cast<const uint4*>(input);
         uint4* o4 = static_cast<uint4*>(output);
 #define MOR_BS_FUSED(E8, NV, PHASE) do { \
-        if (full) k_bs_fused<E8, NV, true><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); \
-        else k_bs_fused<E8, NV, false><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); } while (0)
+        if (full) k_bs_fused<E8, NV, true><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, fin, PHASE, npart1); \
+        else k_bs_fused<E8, NV, false><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, fin, PHASE, npart1); } while (0)
 #define MOR_BS_FUSED_W(E8, WGS_, PHASE) do { \
-        if (full) k_bs_fused<E8, 8, true, WGS_><<<grid, WGS_, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); \
-        else k_bs_fused<E8, 8, false, WGS_><<<grid, WGS_, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, meta, PHASE); } while (0)
+        if (full) k_bs_fused<E8, 8, true, WGS_><<<grid, WGS_, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, fin, PHASE, npart1); \
+        else k_bs_fused<E8, 8, false, WGS_><<<grid, WGS_, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, cpr, shift, nb, fin, PHASE, npart1); } while (0)
 #define MOR_BS_FUSED_ALL(PHASE) do { \
         if (wgs == 512) { if (ss_mode == 2) MOR_BS_FUSED_W(true, 512, PHASE); else MOR_BS_FUSED_W(false, 512, PHASE); } \
         else if (wgs == 1024) { if (ss_mode == 2) MOR_BS_FUSED_W(true, 1024, PHASE); else MOR_BS_FUSED_W(false, 1024, PHASE); } \
         else if (ss_mode == 2) { switch (NVc) { case 1: MOR_BS_FUSED(true, 1, PHASE); break; case 2: MOR_BS_FUSED(true, 2, PHASE); break; case 4: MOR_BS_FUSED(true, 4, PHASE); break; default: MOR_BS_FUSED(true, 8, PHASE); break; } } \
         else { switch (NVc) { case 1: MOR_BS_FUSED(false, 1, PHASE); break; case 2: MOR_BS_FUSED(false, 2, PHASE); break; case 4: MOR_BS_FUSED(false, 4, PHASE); break; default: MOR_BS_FUSED(false, 8, PHASE); break; } } } while (0)
         MOR_BS_FUSED_ALL(inplace ? 1 : 0);
-        k_bs_finalize<<<1, WG, 0, st>>>(ws, grid, grid, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
         if (inplace) MOR_BS_FUSED_ALL(2);
-        else {
-            const int64_t n_all = rows * cols;
-            k_copy_if<<<grid_for(n_all / 8, 4), WG, 0, st>>>(in16, out16, meta, 3, n_all, n_all / 8);
-        }
+        else gated_copy();
 #undef MOR_BS_FUSED_ALL
 #undef MOR_BS_FUSED_W
 #undef MOR_BS_FUSED
         return mor_check_launch("mor_block_scaling (single pass)");
     }
 
-    if (!emu && vec && !col && (ss_mode == 2 || ss_mode == 3) && brows == 1 && bcols % 8 == 0 && is_pow2(bcols / 8)
-        && bcols / 8 <= 64) {
+    if (flat_ok && (ss_mode == 4 || (!col && brows == 1 && bcols % 8 == 0 && is_pow2(bcols / 8) && bcols / 8 <= 64))) {
+        if (global) tensor_amax_pass();
         const int64_t nchunks = rows * cols / 8;
-        const int grid = (int)std::min<int64_t>(cdiv(nchunks, BS_ROWS_NV * WG), MAX_PARTIALS);
+        const int grid = (int)std::min<int64_t>(cdiv(nchunks, BS_ROWS_NV * WG), PASS2_MAX);
+        fin.nerr = grid;
+        fin.nstat = global ? npart1 : grid;
         const uint4* i4 = static_cast<const uint4*>(input);
         uint4* o4 = static_cast<uint4*>(output);
-        const int G = (int)(bcols / 8);
+        const int G = ss_mode == 4 ? 1 : (int)(bcols / 8);
         for (int phase = inplace ? 1 : 0; phase <= (inplace ? 2 : 0); ++phase) {
-            if (ss_mode == 2) k_bs_fused_rows<true><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, G, (int)ss_mode, meta, phase);
-            else k_bs_fused_rows<false><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, G, (int)ss_mode, meta, phase);
-            if (phase != 2) k_bs_finalize<<<1, WG, 0, st>>>(ws, grid, grid, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
+            if (ss_mode == 2) k_bs_fused_rows<true, 0><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, G, (int)ss_mode, fin, phase, npart1);
+            else if (ss_mode == 3) k_bs_fused_rows<false, 0><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, G, (int)ss_mode, fin, phase, npart1);
+            else if (ss_mode == 1) k_bs_fused_rows<false, 1><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, G, (int)ss_mode, fin, phase, npart1);
+            else k_bs_fused_rows<false, 2><<<grid, WG, 0, st>>>(i4, o4, ws, nchunks, G, (int)ss_mode, fin, phase, npart1);
         }
-        if (!inplace) k_copy_if<<<grid_for(nchunks, 4), WG, 0, st>>>(in16, out16, meta, 3, rows * cols, nchunks);
+        if (!inplace) gated_copy();
         return mor_check_launch("mor_block_scaling (single pass, row blocks)");
     }
 
-    // pass 1: per-block amax, per-workgroup partials of the tensor amax and the non-zero count
+    // pass 1: per-block amax (not for ss_mode 4, which only takes the tensor amax), per-workgroup partials of the tensor
+    // amax and the non-zero count
     const int64_t G = bcols / 8;
     int npart;
-    if (col) {
+    if (ss_mode == 4 && !col && vec && n % 8 == 0) {
+        npart = (int)std::min<int64_t>(cdiv(n / 8, 8 * WG), PASS1_MAX);
+        k_bs_amax_flat<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, nullptr, n / 8, 1, 0);
+    } else if (col) {
         k_zero_f32<<<grid_for(nb), WG, 0, st>>>(blocks, nb);
         const int rows_per_wg = (int)std::min<int64_t>(brows, 256);
         const unsigned gx = (unsigned)cdiv(cols, 256);
         const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
-        if ((int64_t)gx > MAX_PARTIALS) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many columns (%lld)", (long long)cols);
-        const unsigned gy = (unsigned)std::min<int64_t>(segs, std::max<int64_t>(MAX_PARTIALS / gx, 1));
+        if ((int64_t)gx > PASS1_MAX) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many columns (%lld)", (long long)cols);
+        const unsigned gy = (unsigned)std::min<int64_t>(segs, std::max<int64_t>(PASS1_MAX / gx, 1));
         npart = (int)(gx * gy);
         k_bs_amax_col<<<dim3(gx, gy), WG, 0, st>>>(in16, ws, blocks, sh, rows_per_wg, vec);
     } else if (vec && brows == 1 && bcols % 8 == 0 && is_pow2(G) && G <= 64) {
         const int64_t nchunks = rows * cols / 8;
-        npart = (int)std::min<int64_t>(cdiv(nchunks, 8 * WG), MAX_PARTIALS);
+        npart = (int)std::min<int64_t>(cdiv(nchunks, 8 * WG), PASS1_MAX);
         k_bs_amax_flat<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, blocks, nchunks, (int)G, ilog2(G));
     } else if (vec && bcols % 8 == 0 && brows * (bcols / 8) < WG && brows * (cols / 8) < 0x7FFFFFFFll) {
         const int nchb = (int)(brows * (bcols / 8));
         int logL = 0;
         while ((4 << logL) < nchb && logL < 6) ++logL;               // about four vectors per lane
         const int groups = WG >> logL;
-        npart = (int)std::min<int64_t>(cdiv(nb, groups), MAX_PARTIALS);
+        npart = (int)std::min<int64_t>(cdiv(nb, groups), PASS1_MAX);
         k_bs_amax_sub<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, blocks, sh, 1 << logL, logL, make_div((uint32_t)sh.gx),
                                             make_div((uint32_t)(bcols / 8)));
     } else {
         const int v1 = (vec && bcols % 8 == 0 && brows * (cols / 8) < 0x7FFFFFFFll) ? 1 : 0;
-        npart = (int)std::min<int64_t>(nb, MAX_PARTIALS);
+        npart = (int)std::min<int64_t>(nb, PASS1_MAX);
         k_bs_amax_block<<<npart, WG, 0, st>>>(in16, ws, blocks, sh, v1, make_div((uint32_t)sh.gx),
                                               make_div((uint32_t)std::max<int64_t>(bcols / 8, 1)));
     }
-    // pass 1.5: tensor amax and non-zero count into the header, block scales
-    k_bs_scales<<<(int)std::min<int64_t>(cdiv(nb, WG), 256), WG, 0, st>>>(ws, blocks, nb, (int)ss_mode, npart);
-    // pass 2: quantize (out of place: write now; in place: error only), error partials
-    // pass 3: decision and scalars
-    // pass 4: bf16 fallback (out of place: copy if meta == 3) or the quantized write (in place: only if meta == 1)
+    fin.nstat = npart;
+    // pass 2: quantize (out of place: write now; in place: error only), error partials; every workgroup first reduces
+    // the pass-1 partials to the tensor amax and computes its blocks' scales from it
+    // end: bf16 fallback (out of place: copy if meta == 3) or the quantized write (in place: only if meta == 1)
     const bool e8 = (ss_mode == 2);
-    const int64_t n = rows * cols;
     if (col && vec && !emu && !e8) {
         const int rows_per_wg = (int)std::min<int64_t>(brows, 16);
         const unsigned gx = (unsigned)cdiv(cdiv(cols, 8), WG);
         const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
-        const dim3 grid(gx, (unsigned)std::min<int64_t>(segs, std::max<int64_t>(MAX_PARTIALS / gx, 1)));
-        if (inplace) k_bs_quant_col<false, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 0, sh, rows_per_wg);
-        else k_bs_quant_col<true, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 0, sh, rows_per_wg);
-        k_bs_finalize<<<1, WG, 0, st>>>(ws, (int)(grid.x * grid.y), 0, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
-        if (inplace) k_bs_quant_col<true, false><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, meta, 1, sh, rows_per_wg);
+        const dim3 grid(gx, (unsigned)std::min<int64_t>(segs, std::max<int64_t>(PASS2_MAX / gx, 1)));
+        fin.nerr = (int)(grid.x * grid.y);
+        if (inplace) k_bs_quant_col<false, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 0, (int)ss_mode, npart, sh, rows_per_wg);
+        else k_bs_quant_col<true, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 0, (int)ss_mode, npart, sh, rows_per_wg);
+        if (inplace) k_bs_quant_col<true, false><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 1, (int)ss_mode, npart, sh, rows_per_wg);
     } else {
         const bool vec2 = vec && (col || bcols % 8 == 0) && n / 8 < 0xFFFFFFFFll;
         const int64_t work = vec2 ? n / 8 : n;
-        const int grid2 = (int)std::min<int64_t>(std::max<int64_t>(cdiv(work, WG), 1), MAX_PARTIALS);
+        const int grid2 = (int)std::min<int64_t>(std::max<int64_t>(cdiv(work, WG), 1), PASS2_MAX);
+        fin.nerr = grid2;
         DivU32 d0 = make_div((uint32_t)std::max<int64_t>(cols / 8, 1)), d1 = make_div((uint32_t)brows),
                d2 = make_div((uint32_t)std::max<int64_t>(bcols / 8, 1)), d3 = make_div((uint32_t)bcols);
-        dispatch_bs_quant(e8, emu, col, !inplace, true, grid2, st, in16, out16, ws, blocks, meta, 0, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
-        k_bs_finalize<<<1, WG, 0, st>>>(ws, grid2, 0, (float)e4m3_threshold, meta, global_amax, global_non_zero, global_error);
-        if (inplace) dispatch_bs_quant(e8, emu, col, true, false, grid2, st, in16, out16, ws, blocks, meta, 1, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
+        dispatch_bs_quant(e8, emu, col, !inplace, true, grid2, st, in16, out16, ws, blocks, fin, 0, (int)ss_mode, npart, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
+        if (inplace) dispatch_bs_quant(e8, emu, col, true, false, grid2, st, in16, out16, ws, blocks, fin, 1, (int)ss_mode, npart, sh, vec2 ? 1 : 0, d0, d1, d2, d3);
     }
-    if (!inplace) {
-        const int64_t nvec = vec ? n / 8 : 0;
-        k_copy_if<<<grid_for(nvec > 0 ? nvec : n, 4), WG, 0, st>>>(in16, out16, meta, 3, n, nvec);
-    }
+    if (!inplace) gated_copy();
     return mor_check_launch("mor_block_scaling");
 }
 
