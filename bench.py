@@ -327,6 +327,17 @@ def other_configs(torch, run, cabi, K, W):
             run.fake_quantize(xs, os_, ms_, 1, 32, 0.0, 2, 2)
     ms, wall = time_launches(torch, graph.replay, 20, 3)
     res["tiny_1x32"]["graph_replay_us_per_call"] = round(ms * 1e3 / 100, 2)
+    # 100 separate 1x32 tensors through the batch entry: two launches for all of them
+    from mor_amd.batch import BatchPlan
+    for mode, key in ((2, "batch_100_tensors_e4m3_us_per_tensor"), (1, "batch_100_tensors_mor_us_per_tensor")):
+        pool_x = torch.randn(100, 32, device="cuda").to(torch.bfloat16)
+        pool_o = torch.empty_like(pool_x)
+        pool_m = torch.empty((100, 1), dtype=torch.int32, device="cuda")
+        plan = BatchPlan([pool_x[i:i + 1] for i in range(100)], [pool_o[i:i + 1] for i in range(100)],
+                         [pool_m[i:i + 1] for i in range(100)], [(1, 32)] * 100, 1e-3, mode, 2)
+        ms, wall = time_launches(torch, plan.run, 200, 20)
+        res["tiny_1x32"][key] = round(ms * 1e3 / 100, 3)
+        res["tiny_1x32"][key.replace("_us_", "_wall_us_")] = round(wall * 1e3 / 100, 3)
     # the same call through the operator layer a user of the reference calls (allocations of out and meta included)
     import mor
     xg = xs.clone().requires_grad_(True)

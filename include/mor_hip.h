@@ -79,6 +79,24 @@ MOR_API int mor_fake_quantize(const void* input, void* output, int32_t* meta,
                       uint32_t flags, void* stream);
 
 /*
+ * fake_quantize on many tensors in one call: descs[i] holds the arguments of one mor_fake_quantize
+ * call (FQ:1839-1871; the reference's callers loop over their tensors, one launch each), and the
+ * result of every tensor is bit for bit that call's.  descs is host memory, read before the call
+ * returns.  Tensors of up to 2^18 elements share launches, 56 to a launch, one workgroup per block;
+ * larger ones are forwarded to mor_fake_quantize.  Every descriptor is validated before anything is
+ * launched; no device memory is allocated.
+ */
+typedef struct MorTensorDesc {
+    const void* input;
+    void* output;             /* may alias input */
+    int32_t* meta;
+    int64_t rows, cols, block_rows, block_cols;
+    double clamp_threshold;
+    int64_t mode, sf_type;
+} MorTensorDesc;
+MOR_API int mor_fake_quantize_batch(const MorTensorDesc* descs, int64_t n, uint32_t flags, void* stream);
+
+/*
  * Block fake quantization to one forced element format, scale fmax/amax per block as in
  * the block modes of FQ:801-823; MOR_FMT_E2M3 follows the E2M3 branch FQ:758-770
  * (software saturating cast).  The reference has no public op for a forced E2M3; this

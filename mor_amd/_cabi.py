@@ -22,6 +22,7 @@ SIGNATURES = {
     "mor_version": (C.c_char_p, []),
     "mor_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
     "mor_fake_quantize": (_int, [_vp, _vp, _i32p, _i64, _i64, _i64, _i64, _f64, _i64, _i64, _u32, _vp]),
+    "mor_fake_quantize_batch": (_int, [_vp, _i64, _u32, _vp]),
     "mor_block_format": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _i64, _u32, _vp]),
     "mor_block_scaling": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f64, _i64, _int, _vp, _sz, _u32, _vp]),
     "mor_block_scaling_static": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f64, _i64, _int, _u32, _vp]),

@@ -1136,7 +1136,7 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
     // end: bf16 fallback (out of place: copy if meta == 3) or the quantized write (in place: only if meta == 1)
     const bool e8 = (ss_mode == 2);
     if (col && vec && !emu && !e8) {
-        const int rows_per_wg = (int)std::min<int64_t>(brows, 16);
+        const int rows_per_wg = (int)std::min<int64_t>(brows, 32);
         const unsigned gx = (unsigned)cdiv(cdiv(cols, 8), WG);
         const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
         const dim3 grid(gx, (unsigned)std::min<int64_t>(segs, std::max<int64_t>(PASS2_MAX / gx, 1)));

@@ -44,3 +44,21 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert L.mor_block_scaling(1, 1, 1, 1, 1, 1, 256, 256, 128, 128, 0.045, 1, 0, None, 0, 0, None) == -2
     assert L.mor_e8mx(1, 1, 16, 16, 4, 4, 7, 1, 1, 64, 0, None) == -1
     assert L.mor_quant_dequant(1, 1, 16, 9, None) == -1
+
+
+def test_batch_entry_rejects_bad_arguments_without_a_gpu():
+    """argument checks run before any device call"""
+    from mor_amd import _cabi
+    from mor_amd.batch import TensorDesc
+    import ctypes as C
+    L = _cabi.lib()
+    assert L.mor_fake_quantize_batch(None, 3, 0, None) != 0
+    assert b"descriptor" in L.mor_last_error()
+    assert L.mor_fake_quantize_batch(None, -1, 0, None) != 0
+    assert L.mor_fake_quantize_batch(None, 0, 0, None) == 0            # an empty list is no work
+    d = (TensorDesc * 1)()
+    d[0].input, d[0].output, d[0].meta = 256, 256, 256                 # (never dereferenced: the shape is rejected first)
+    d[0].rows, d[0].cols, d[0].block_rows, d[0].block_cols = 4, 0, 1, 32
+    assert L.mor_fake_quantize_batch(d, 1, 0, None) != 0
+    assert b"positive" in L.mor_last_error()
+    assert C.sizeof(TensorDesc) == 80
