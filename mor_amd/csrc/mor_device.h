@@ -60,11 +60,13 @@ __device__ __forceinline__ void store16_rt(uint4* p, uint4 v, bool nt) {
 // cache: nothing of such a tensor is found there again (MX 1 x 32 on 16384 x 14336: 160 -> 150 us; at 8192^2 streaming
 // loads cost 39 -> 44 us).
 __device__ __forceinline__ bool streams_in(int64_t bf16_elements) { return bf16_elements > ((int64_t)128 << 20); }
-// The last (or only) read a kernel makes of a tensor of 32 MiB or more streams as well: nothing reads those lines again,
+// The last (or only) read a kernel makes of a tensor of 64 MiB or more streams as well: nothing reads those lines again,
 // and with streaming loads a tensor that comes from HBM does not push the caller's data out of the caches on its way
 // (8192^2 from HBM, 1 x 32 blocks: 45.5 -> 43 us; repeated launches on one buffer pair, which find part of their input in
 // the last-level cache only because the previous launch left it there, lose that: 39 -> 44 us).
-__device__ __forceinline__ bool streams_last_read(int64_t bf16_elements) { return bf16_elements >= ((int64_t)16 << 20); }
+// A tensor of 32 MiB and its image fit the 256 MB last-level cache with room to spare and keep the allocating loads
+// (4096^2 with the caller's scale: 10.0 against 12.5 us).
+__device__ __forceinline__ bool streams_last_read(int64_t bf16_elements) { return bf16_elements >= ((int64_t)32 << 20); }
 __device__ __forceinline__ uint4 load16_rt(const uint4* p, bool nt) { return nt ? load16<true>(p) : load16<false>(p); }
 
 // ---------------------------------------------------------------- bf16 <-> fp32

@@ -379,11 +379,11 @@ static void launch_rowgroup_f(const uint4* i4, uint4* o4, int32_t* meta, int64_t
         return;
     }
     // Few vectors per lane: many small workgroups interleave their loads and stores more finely than few large ones.
-    // Tensors of 32 MiB and more (they come from HBM) take one vector per lane: a plain copy of 8192^2 from HBM runs at
+    // Tensors of 64 MiB and more (they come from HBM) take one vector per lane: a plain copy of 8192^2 from HBM runs at
     // 0.79 of the peak rate with one, 0.76 with two, 0.73 with eight vectors per lane; at 16384 x 14336: 0.82 / 0.76 /
     // 0.73.  Smaller tensors take two (fewer workgroups to launch).
     // (the software casts of E2M3 / E3M2 cost more instructions per element and are better off with two: 49.6 -> 45.4 us)
-    const bool big = nchunks * 16 >= ((int64_t)32 << 20) && Fmt<F>::hw;
+    const bool big = nchunks * 16 >= ((int64_t)64 << 20) && Fmt<F>::hw;
     const bool nt_out = nchunks * 16 >= ((int64_t)4 << 20);
 #define MOR_ROWGROUP(NV) do { \
         if (nt_out && nchunks % ((int64_t)NV * WG) == 0 && (G == 4 || G == 16) && nchunks / ((int64_t)NV * WG) <= 0x7FFFFFFFll) { \
@@ -499,7 +499,11 @@ extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
             if (output != input) {
                 const int64_t n = rows * cols;
                 const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
-                k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(static_cast<const uint16_t*>(input), static_cast<uint16_t*>(output), n, nvec);
+                const uint16_t* i16 = static_cast<const uint16_t*>(input);
+                uint16_t* o16 = static_cast<uint16_t*>(output);
+                // (from HBM one vector per lane copies fastest, as in k_rowgroup)
+                if (nvec >= ((int64_t)4 << 20)) k_copy<1><<<(int)cdiv(nvec, (int64_t)WG), WG, 0, st>>>(i16, o16, n, nvec);
+                else k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(i16, o16, n, nvec);
             }
             k_fill_i32<<<grid_for(nblocks), WG, 0, st>>>(meta, nblocks, 3);
             return mor_check_launch("k_copy / k_fill_i32");

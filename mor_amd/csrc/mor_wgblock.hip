@@ -16,9 +16,10 @@ static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, i
                               const Shape& sh, const QuantArgs& qa, int cpr, int shift, hipStream_t st) {
     // Streaming stores for outputs that do not fit an L2 anyway (>= 4 MiB): the quantized tensor then does not evict
     // the input or the caller's data from the caches (measured at 8192^2: 42.7 -> 40.4 us, at 4096^2: 13.3 -> 10.3 us).
-    // Tensors of 32 MiB and more stream their loads as well (the block is read once).
+    // Tensors of 64 MiB and more stream their loads as well (the block is read once; a smaller tensor is likely to sit
+    // in the last-level cache, where its producer left it).
     const int64_t out_bytes = sh.rows * sh.cols * 2;
-    const int ntm = (out_bytes >= ((int64_t)32 << 20)) ? 1 : (out_bytes >= ((int64_t)4 << 20)) ? 2 : 0;
+    const int ntm = (out_bytes >= ((int64_t)64 << 20)) ? 1 : (out_bytes >= ((int64_t)4 << 20)) ? 2 : 0;
     // Large grids run 3 workgroups per CU (unused dynamic LDS caps the occupancy the registers would allow at 5):
     // fewer tiles in flight keep the memory system on fewer DRAM pages at a time (8192^2 from HBM, MoR 128 x 128:
     // 49.4 -> 47.5 us; 16384 x 14336: 161 -> 156 us), while a grid that fits the chip at once wants every slot
