@@ -347,11 +347,18 @@ __device__ __forceinline__ float bs_element(float x, const Scale& sc, float& err
     err += fabsf((dq - x) / x);
     return dq;
 }
+// acc + |q - a| / a for magnitudes a of a block whose scale is in the fast range, through the hardware reciprocal.
+// Both operands are taken times 2^16 first: the smallest bf16 denormal (2^-133) then has a reciprocal that fits the
+// format, and the largest element such a block can hold (448 * 2^100) does not overflow, so the term is right for
+// every finite element.  No selects: a zero element has q = 0 and its term is 0 * min(1 / 0, FLT_MAX) = 0.
+__device__ __forceinline__ float rel_err_fast(float q, float a, float acc) {
+    const float ac = a * 0x1p16f;
+    return fmaf(fabsf(fmaf(q, 0x1p16f, -ac)), fminf(__builtin_amdgcn_rcpf(ac), 0x1.fffffep127f), acc);
+}
 // Fast version on magnitudes for scales in the fast range: hardware convert; q = c / s by a reciprocal-multiply
 // with one exact-residual correction (r = 1 / s correctly rounded, the result is then the rounded quotient);
 // error term |q - x| / x through the hardware reciprocal (relative 1e-7, tolerance on the sum 1e-6).
-// No selects: a zero element has q = 0, so its term is 0 * min(1 / 0, FLT_MAX) = 0 and its magnitude bits are 0;
-// the sign of the input is kept for non-zero halves only (zero inputs come back as +0, FQ:1133-1134), through a
+// No selects: a zero element's magnitude bits are 0; the sign of the input is kept for non-zero halves only (zero inputs come back as +0, FQ:1133-1134), through a
 // packed 16-bit mask.
 // ERR / OUT: whether the error terms / the output word are wanted (the in-place phases need one of them each).
 template <bool E8, bool ERR = true, bool OUT = true>
@@ -371,9 +378,8 @@ __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, fl
         qb = div_by_scale(c.y, sc.s, rs);
     }
     if constexpr (ERR) {
-        const float ya = fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), yb = fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f);
-        err = fmaf(fabsf(qa - a), ya, err);
-        err = fmaf(fabsf(qb - b), yb, err);
+        err = rel_err_fast(qa, a, err);
+        err = rel_err_fast(qb, b, err);
     }
     if constexpr (!OUT) return 0u;
     const uint32_t nonzero = pk_min_u16(w & 0x7FFF7FFFu, 0x00010001u);        // 1 in each half that is not +-0
@@ -460,6 +466,50 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
     }
 }
 
+// One vector of 8 adjacent columns, each with the scale of its own column block (all in the fast range): the
+// arithmetic of bs_pair_fast with a scale per half of a word; a vector that holds a NaN takes the exact arithmetic.
+template <bool WRITE, bool ERR>
+__device__ __forceinline__ uint4 bs_cols_vec_fast(uint4 v, const Scale (&sc)[8], float& err) {
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    float row_err = 0.0f;
+    if (vec_has_nan(v)) {          // (rare)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float q0 = bs_element<false, false>(bf16_lo(w[j]), sc[2 * j], row_err);
+            float q1 = bs_element<false, false>(bf16_hi(w[j]), sc[2 * j + 1], row_err);
+            w[j] = store_pair<false>(q0, q1);
+        }
+    } else
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float a = fabsf(bf16_lo(w[j])), b = fabsf(bf16_hi(w[j]));
+        const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc[2 * j].s, b * sc[2 * j + 1].s));
+        const float qa = div_by_scale(c.x, sc[2 * j].s, sc[2 * j].r);
+        const float qb = div_by_scale(c.y, sc[2 * j + 1].s, sc[2 * j + 1].r);
+        if constexpr (ERR) {
+            row_err = rel_err_fast(qa, a, row_err);
+            row_err = rel_err_fast(qb, b, row_err);
+        }
+        if constexpr (WRITE) {
+            const uint32_t nonzero = pk_min_u16(w[j] & 0x7FFF7FFFu, 0x00010001u);
+            w[j] = store_pair<false>(qa, qb) | (w[j] & (nonzero << 15));
+        }
+    }
+    err += row_err;
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+// the same vector with the exact arithmetic (a scale outside the fast range)
+__device__ __forceinline__ uint4 bs_cols_vec_exact(uint4 v, const Scale (&sc)[8], float& err) {
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float q0 = bs_element<false, false>(bf16_lo(w[j]), sc[2 * j], err);
+        float q1 = bs_element<false, false>(bf16_hi(w[j]), sc[2 * j + 1], err);
+        w[j] = store_pair<false>(q0, q1);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // pass 2 / pass 4 for column blocks N x 1 with aligned rows (the geometry of k_bs_amax_col): a thread owns 8 adjacent
 // columns over a segment of rows, so its 8 scales and their reciprocals are computed once.  Threads whose scales are
 // not all in the fast range use the exact arithmetic.
@@ -485,10 +535,9 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
             const int64_t r_end = min(r_begin + rows_per_wg, (by + 1) * sh.brows);
             const int64_t sp = by * sh.cols + col0;
             Scale sc[8];
-            float rs[8];
             bool fast = true;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) { sc[j] = make_scale(block_scale(gamax, scales, sp + j, ss_mode)); rs[j] = sc[j].r; fast = fast && sc[j].fast; }
+            for (int j = 0; j < 8; ++j) { sc[j] = make_scale(block_scale(gamax, scales, sp + j, ss_mode)); fast = fast && sc[j].fast; }
             if (fast) {
 #pragma unroll 1
                 for (int64_t r = r_begin; r < r_end; r += 4) {
@@ -500,50 +549,17 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
                     }
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
-                        uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
-                        float row_err = 0.0f;
-                        if (vec_has_nan(v[k])) {          // a NaN among the 8 values: the exact arithmetic for this vector (rare)
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) {
-                                float q0 = bs_element<false, false>(bf16_lo(w[j]), sc[2 * j], row_err);
-                                float q1 = bs_element<false, false>(bf16_hi(w[j]), sc[2 * j + 1], row_err);
-                                w[j] = store_pair<false>(q0, q1);
-                            }
-                        } else
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            // as bs_pair_fast, with a scale of its own for each of the two columns of the word
-                            const float a = fabsf(bf16_lo(w[j])), b = fabsf(bf16_hi(w[j]));
-                            const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc[2 * j].s, b * sc[2 * j + 1].s));
-                            const float qa = div_by_scale(c.x, sc[2 * j].s, rs[2 * j]);
-                            const float qb = div_by_scale(c.y, sc[2 * j + 1].s, rs[2 * j + 1]);
-                            if constexpr (ERR) {
-                                row_err = fmaf(fabsf(qa - a), fminf(__builtin_amdgcn_rcpf(a), 0x1.fffffep127f), row_err);
-                                row_err = fmaf(fabsf(qb - b), fminf(__builtin_amdgcn_rcpf(b), 0x1.fffffep127f), row_err);
-                            }
-                            if constexpr (WRITE) {
-                                const uint32_t nonzero = pk_min_u16(w[j] & 0x7FFF7FFFu, 0x00010001u);
-                                w[j] = store_pair<false>(qa, qb) | (w[j] & (nonzero << 15));
-                            }
-                        }
-                        err += row_err;
+                        const uint4 q = bs_cols_vec_fast<WRITE, ERR>(v[k], sc, err);
                         if constexpr (WRITE) {
-                            if (r + k < r_end) store16_rt(out4 + (r + k) * row_stride + (col0 >> 3), make_uint4(w[0], w[1], w[2], w[3]), nt);
+                            if (r + k < r_end) store16_rt(out4 + (r + k) * row_stride + (col0 >> 3), q, nt);
                         }
                     }
                 }
             } else {
 #pragma unroll 1
                 for (int64_t r = r_begin; r < r_end; ++r) {
-                    const uint4 v = in4[r * row_stride + (col0 >> 3)];
-                    uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        float q0 = bs_element<false, false>(bf16_lo(w[j]), sc[2 * j], err);
-                        float q1 = bs_element<false, false>(bf16_hi(w[j]), sc[2 * j + 1], err);
-                        w[j] = store_pair<false>(q0, q1);
-                    }
-                    if constexpr (WRITE) out4[r * row_stride + (col0 >> 3)] = make_uint4(w[0], w[1], w[2], w[3]);
+                    const uint4 q = bs_cols_vec_exact(in4[r * row_stride + (col0 >> 3)], sc, err);
+                    if constexpr (WRITE) out4[r * row_stride + (col0 >> 3)] = q;
                 }
             }
         }

@@ -560,6 +560,13 @@ static inline float bs_element(float x, float sf, int64_t ss_mode, int flavour, 
     return dq;
 }
 
+/* The sum of the per-element error terms of the last mor_oracle_block_scaling call of this thread, added in double:
+ * the value the fp32 sums of the reference approach, whatever order they are added in.  (The reference's own result,
+ * global_error, carries the rounding of its order of additions: about sqrt(n) * 2^-24 relative for chains of n
+ * terms.) */
+static _Thread_local double g_last_exact_error;
+double mor_oracle_last_exact_error(void) { return g_last_exact_error; }
+
 int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
                              float* global_amax_o, int32_t* global_nnz_o, float* global_error_o,
                              int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
@@ -603,9 +610,10 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
     const int geom_block = !channel && (bcols % 64 == 0) && (brows % 32 == 0);
     const int geom_row = channel && brows == 1 && bcols >= 128 && (bcols % 128 == 0);
     const int geom_col = channel && bcols == 1 && brows == rows && (cols % 64 == 0) && (rows % 16 == 0);
+    double exact = 0.0;
     if (geom_col) {
         for (int64_t k = 0; k < nb; ++k) berr[k] = 0.0f;
-#pragma omp parallel for schedule(static)
+#pragma omp parallel for schedule(static) reduction(+:exact)
         for (int64_t tb = 0; tb < cols / 64; ++tb) {
             float partial[512];
             for (int ty = 0; ty < 16; ++ty)
@@ -619,8 +627,8 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
                         float x1 = mor_oracle_bf16_to_fp32(in[r * cols + c1]), x2 = mor_oracle_bf16_to_fp32(in[r * cols + c2]);
                         float q1 = bs_element(x1, sf1, ss_mode, flavour, &t1);
                         float q2 = bs_element(x2, sf2, ss_mode, flavour, &t2);
-                        if (x1 != 0.0f) e1 += t1;
-                        if (x2 != 0.0f) e2 += t2;
+                        if (x1 != 0.0f) { e1 += t1; exact += (double)t1; }
+                        if (x2 != 0.0f) { e2 += t2; exact += (double)t2; }
                         tmp[r * cols + c1] = (uint16_t)store_bf16(q1, flavour);
                         tmp[r * cols + c2] = (uint16_t)store_bf16(q2, flavour);
                     }
@@ -629,7 +637,7 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
             berr[tb * 64] = block_tree_sum(partial, 512);
         }
     } else {
-#pragma omp parallel for schedule(static)
+#pragma omp parallel for schedule(static) reduction(+:exact)
     for (int64_t k = 0; k < nb; ++k) {
         int64_t by = k / gx, bx = k % gx;
         float sf = mor_oracle_scaling_factor(gamax, bamax[k], (int)ss_mode);
@@ -647,8 +655,8 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
                             float x1 = mor_oracle_bf16_to_fp32(in[i1]), x2 = mor_oracle_bf16_to_fp32(in[i2]);
                             float q1 = bs_element(x1, sf, ss_mode, flavour, &e1);
                             float q2 = bs_element(x2, sf, ss_mode, flavour, &e2);
-                            if (x1 != 0.0f) acc += e1;
-                            if (x2 != 0.0f) acc += e2;
+                            if (x1 != 0.0f) { acc += e1; exact += (double)e1; }
+                            if (x2 != 0.0f) { acc += e2; exact += (double)e2; }
                             tmp[i1] = (uint16_t)store_bf16(q1, flavour);
                             tmp[i2] = (uint16_t)store_bf16(q2, flavour);
                         }
@@ -665,8 +673,8 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
                     float x1 = mor_oracle_bf16_to_fp32(in[i1]), x2 = mor_oracle_bf16_to_fp32(in[i2]);
                     float q1 = bs_element(x1, sf, ss_mode, flavour, &t1);
                     float q2 = bs_element(x2, sf, ss_mode, flavour, &t2);
-                    if (x1 != 0.0f) e1 += t1;
-                    if (x2 != 0.0f) e2 += t2;
+                    if (x1 != 0.0f) { e1 += t1; exact += (double)t1; }
+                    if (x2 != 0.0f) { e2 += t2; exact += (double)t2; }
                     tmp[i1] = (uint16_t)store_bf16(q1, flavour);
                     tmp[i2] = (uint16_t)store_bf16(q2, flavour);
                 }
@@ -684,6 +692,7 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
                     tmp[r * cols + c] = (uint16_t)store_bf16(q, flavour);
                 }
             berr[k] = (float)seq;
+            exact += seq;
         }
     }
     }
@@ -705,6 +714,7 @@ int mor_oracle_block_scaling(const uint16_t* in, uint16_t* out, int32_t* meta,
     *global_amax_o = gamax;
     *global_nnz_o = gnnz;
     *global_error_o = gerr;
+    g_last_exact_error = exact;
     if (use_bf16) {
         if (out != in) memcpy(out, in, sizeof(uint16_t) * (size_t)(rows * cols));
     } else {

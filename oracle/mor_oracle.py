@@ -48,6 +48,7 @@ def lib():
             "mor_oracle_fake_quantize": (C.c_int, [vp, vp, vp, i64, i64, i64, i64, f32, i64, i64, C.c_int, vp]),
             "mor_oracle_block_format": (C.c_int, [vp, vp, i64, i64, i64, i64, C.c_int, i64, C.c_int]),
             "mor_oracle_block_scaling": (C.c_int, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, f32, i64, C.c_int, C.c_int]),
+            "mor_oracle_last_exact_error": (C.c_double, []),
             "mor_oracle_e8mx": (C.c_int, [vp, vp, i64, i64, i64, i64, i64, i64, C.c_int]),
             "mor_oracle_quant_dequant": (None, [vp, vp, sz, C.c_int]),
             "mor_oracle_e4m3_with_e8_scale": (None, [vp, vp, sz, C.c_int]),
@@ -136,6 +137,12 @@ def block_scaling(a, block_x, block_y, e4m3_threshold, ss_mode, channel=False, f
     if rc:
         raise RuntimeError(f"mor_oracle_block_scaling failed: {rc}")
     return out, meta, gamax, gnnz, gerr
+
+
+def last_exact_error():
+    """The error terms of this thread's last block_scaling call added in float64 (global_error is the reference's fp32
+    sum in the reference's order of additions, rounding included)."""
+    return float(lib().mor_oracle_last_exact_error())
 
 
 def e8mx(a, block_x, block_y, quantize_type, scaling_strategy, flavour=KERNEL):
