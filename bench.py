@@ -274,6 +274,15 @@ def other_configs(torch, run, cabi, K, W):
     add("mor_256x256_8192x8192_normal", lambda: run.fake_quantize(x, out, meta, 256, 256, 1e-15, 1, 1), n * 4, n)
     add("per_row_e4m3_2048x32768", lambda: run.fake_quantize(x.view(2048, 32768), out.view(2048, 32768), meta, 1, 32768, 0.0, 2, 1), n * 4, n)
     add("per_row_e4m3_512x131072", lambda: run.fake_quantize(x.view(512, 131072), out.view(512, 131072), meta, 1, 131072, 0.0, 2, 1), n * 4, n)
+    # x and its transpose from one read, 128 x 128 tiles (one read + two writes: 6 B/element); the reference's callers
+    # run the op on x and on x.t().contiguous(): two launches and a transposing copy, 12 B/element
+    out_t = torch.empty_like(x)
+    meta_t = torch.empty_like(meta)
+    st_ = run.stream
+    for mode, key in ((1, "dual_tiles_mor_128x128_8192x8192"), (2, "dual_tiles_e4m3_128x128_8192x8192")):
+        add(key, lambda: cabi.check(run.L.mor_fake_quantize_dual_tiles(x.data_ptr(), out.data_ptr(), meta.data_ptr(), out_t.data_ptr(),
+                                                                         meta_t.data_ptr(), 8192, 8192, 1e-15, mode, 1, st_())), n * 6, n)
+    del out_t
     # C1: per-tensor E4M3, 4096x4096, scale from the tensor amax (the quantize pass only: 4 B/element)
     x1 = x[:4096, :4096].contiguous()
     o1 = torch.empty_like(x1)

@@ -228,6 +228,22 @@ MOR_API int mor_fake_quantize_dual(const void* input, void* output_rows, int32_t
                                    void* output_cols, int32_t* meta_cols, int64_t rows, int64_t cols,
                                    int64_t mode, int64_t sf_type, void* stream);
 
+/*
+ * The same for 128 x 128 tiles, with MoR (no counterpart in the reference either: its callers
+ * quantize x and x.t().contiguous() in two calls of fake_quantize, FQ:1839-1871):
+ *   output   [rows, cols], meta   [rows / 128, cols / 128] == mor_fake_quantize(x,   rows, cols, 128, 128, clamp, mode, sf_type)
+ *   output_t [cols, rows], meta_t [cols / 128, rows / 128] == mor_fake_quantize(x^T, cols, rows, 128, 128, clamp, mode, sf_type)
+ * for mode % 10 in 1 (MoR), 2 (E4M3), 3 (E5M2), mode / 100 as in mor_fake_quantize, default flavour.
+ * A tile and its transpose hold the same elements, so they share amax, scale and format: the tile is
+ * quantized once and stored twice.  (MoR compares two fp32 error sums; the call on x^T adds the same
+ * terms in another order, so a tile whose two sums agree to the last bits could come out in the other
+ * format there.  The decision taken here is that of the call on x.)
+ * rows and cols multiples of 128; three different 16-byte aligned tensors.
+ */
+MOR_API int mor_fake_quantize_dual_tiles(const void* input, void* output, int32_t* meta, void* output_t,
+                                         int32_t* meta_t, int64_t rows, int64_t cols, double clamp_threshold,
+                                         int64_t mode, int64_t sf_type, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

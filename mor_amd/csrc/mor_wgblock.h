@@ -14,11 +14,25 @@ namespace mor {
 // GATHER: the block's elements are read and written pair by pair (odd column counts, pointers or block widths that are
 // not multiples of 16 bytes): a lane's words are pairs of neighbouring elements of a row; every later step is
 // elementwise, so nothing else changes.
-template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false>
+// DUAL (whole 128 x 128 tiles, 256 threads): the quantized tile is also written transposed, to out_t [cols, rows]
+// (with its meta entry at meta_t [cols / 128, rows / 128]): every result vector goes to LDS as well as to `out`, and
+// the tile is read back from LDS column by column.  LDS layout: row r of the tile is 64 words (two columns each) at
+// r * 64, and the word of columns (2w, 2w + 1) sits at position w ^ ((r >> 3) << 1) of its row.  A vector of 8 columns
+// stays one aligned group of 4 words (in another order), so the writes are 16-byte writes; the 16 lanes that store one
+// transposed row read, for rows 8j .. 8j + 7 (j = 0 .. 15) of one column, words in 16 different banks, and the four
+// columns a wave handles at a time fill the other 16.
+template <class V> __device__ __forceinline__ void dual_tile_put(uint32_t* s_t, int r, int cc, V q) {
+    const int R = r >> 3;
+    const uint4 p = (R & 1) ? make_uint4(q.z, q.w, q.x, q.y) : make_uint4(q.x, q.y, q.z, q.w);
+    *reinterpret_cast<uint4*>(s_t + r * 64 + ((cc ^ (R >> 1)) << 2)) = p;
+}
+template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false, bool DUAL = false>
 __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                  float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift,
-                                                 int64_t first) {
+                                                 int64_t first, uint4* out_t, int32_t* __restrict__ meta_t) {
+    static_assert(!DUAL || (FULL && NV == 8 && WGS == 256 && !GATHER), "DUAL: whole 128 x 128 tiles");
     constexpr int NW = WGS / 64;
+    __shared__ __attribute__((aligned(16))) uint32_t s_t[DUAL ? 128 * 64 : 4];
     __shared__ float s_f[2][NW];
     __shared__ uint32_t s_u[NW];
     __shared__ float s_e[2][NW];           // the error sums have slots of their own: no barrier between pass 1's readers and pass 2's writers
@@ -102,6 +116,29 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
             }
         } else {
             store16<(NT != 0)>(bout + off[k], q);
+            if constexpr (DUAL) dual_tile_put(s_t, (k * WGS + tid) >> 4, tid & 15, q);
+        }
+    };
+    // DUAL: the tile in LDS -> out_t, a lane per 8 consecutive rows of one column; the tile's entry of meta_t
+    auto write_transposed = [&](int meta_val) {
+        if constexpr (DUAL) {
+            __syncthreads();
+            const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s_t);
+            const uint32_t row_stride_t = (uint32_t)(sh.rows >> 3);
+            uint4* tb = out_t + (c0 * row_stride_t + (r0 >> 3));
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const int ch = k * WGS + tid, c = ch >> 4, j = ch & 15;
+                uint32_t w[4];
+                const int at = 2 * ((c >> 1) ^ (j << 1)) + (c & 1);            // (rows 8j .. 8j + 7: the same position in each)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t lo = s16[(8 * j + 2 * i) * 128 + at], hi = s16[(8 * j + 2 * i + 1) * 128 + at];
+                    w[i] = lo | (hi << 16);
+                }
+                store16<(NT != 0)>(tb + (int64_t)c * row_stride_t + j, make_uint4(w[0], w[1], w[2], w[3]));
+            }
+            if (tid == 0 && meta_t && meta_val >= 0) meta_t[bx * sh.gy + by] = meta_val;
         }
     };
 
@@ -135,6 +172,17 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     if (amax_b > 0x7F800000u || (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast))) {           // uniform over the workgroup
         generic_block<false, false, WGS>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
                              sh, qa, E8, bid, s_f, s_u);
+        if constexpr (DUAL) {
+            // the tile as generic_block has just written it (this workgroup's own stores), through LDS to out_t
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                dual_tile_put(s_t, (k * WGS + tid) >> 4, tid & 15, bout[off[k]]);
+            }
+            int mv = qa.meta_val;
+            if constexpr (MOR) mv = meta[bid];                        // (thread 0 wrote it before the barrier above)
+            write_transposed(mv);
+        }
         return;
     }
 
@@ -193,6 +241,7 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     if (!out) return;
 
     // pass 3 (registers): quantize and store, FQ:733-851
+    auto pass3 = [&]() {
     if ((fmt < 0) || !(amax > 0.0f)) {
         if (out != in) {
 #pragma unroll
@@ -235,6 +284,9 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
             for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_fast<FMT_E2M3, E8>(v[k], sc));
             break;
     }
+    };
+    pass3();
+    write_transposed(meta_val);
 }
 
 

@@ -31,7 +31,7 @@ static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, i
     // last-level cache does not care).
     const int shift_arg = (grid >= 2048 && sh.gx % 8 == 0 && grid % 8 == 0) ? ((shift & 255) | 256) : shift;
 #define MOR_WGBLOCK(FULL, NT) for_slices(grid, [&](int64_t first, int count) { \
-        k_wgblock<MOR, E8, NV, FULL, NT, WGS><<<count, WGS, dyn_lds, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift_arg, first); })
+        k_wgblock<MOR, E8, NV, FULL, NT, WGS><<<count, WGS, dyn_lds, st>>>(i4, o4, meta, stats, sh, qa, cpr, shift_arg, first, nullptr, nullptr); })
     if (full) {
         if (ntm == 1) MOR_WGBLOCK(true, 1); else if (ntm == 2) MOR_WGBLOCK(true, 2); else MOR_WGBLOCK(true, 0);
     } else {
@@ -85,7 +85,7 @@ static void launch_wgblock_gather(const void* in, void* out, int32_t* meta, floa
     const uint4* i4 = static_cast<const uint4*>(in);
     uint4* o4 = static_cast<uint4*>(out);
 #define MOR_GATHER(NV) for_slices(grid, [&](int64_t first, int count) { \
-        k_wgblock<MOR, E8, NV, false, 0, WG, true><<<count, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, 1, 0, first); })
+        k_wgblock<MOR, E8, NV, false, 0, WG, true><<<count, WG, 0, st>>>(i4, o4, meta, stats, sh, qa, 1, 0, first, nullptr, nullptr); })
     if (nv <= 1) MOR_GATHER(1); else if (nv <= 2) MOR_GATHER(2); else if (nv <= 4) MOR_GATHER(4); else MOR_GATHER(8);
 #undef MOR_GATHER
 }

@@ -12,8 +12,7 @@ of quantization blocks whose mean relative error lies in [i * 0.005, (i + 1) * 0
 everything above.  The scalars are those of the block-scaling op (mor/csrc/cuda/fake_quantize.cu:1178-1241): the count
 of non-zero elements, the sum of |q / x - 1| over them, and their quotient.
 """
-import re
-from typing import Dict, List, Sequence
+from typing import List, Sequence
 
 import torch
 from torch import Tensor
@@ -28,31 +27,6 @@ def format_log_line(node_id: int, tensor_name: str, counter: int, step: int, row
     return (f"{node_id}: Tensor {tensor_name} at counter {counter} step {step} tensor dimension: {rows}x{cols} "
             f"global_non_zero: {global_non_zero} global_error: {global_error:.6f} relative_error: {rel:.8f} "
             f"histogram [{', '.join(str(int(h)) for h in histogram)}]")
-
-
-_FIELDS = {
-    "tensor": re.compile(r"Tensor\s+([\w\.]+)\s+at\s+counter\s+(\d+)\s+step\s+(\d+)"),
-    "dimension": re.compile(r"tensor dimension:\s+([\dx]+)"),
-    "non_zero": re.compile(r"global_non_zero:\s+(\d+)"),
-    "global_error": re.compile(r"global_error:\s+([\d\.]+)"),
-    "relative_error": re.compile(r"relative_error:\s+([\d\.]+)"),
-    "histogram": re.compile(r"histogram\s+\[([\d,\s]+)\]"),
-}
-
-
-def parse_log_line(line: str) -> Dict[str, object]:
-    """The fields of one line, found the way the reference's parser finds them (one search per field)."""
-    m = {k: p.search(line) for k, p in _FIELDS.items()}
-    if not all(m[k] for k in ("tensor", "non_zero", "global_error", "relative_error", "histogram")):
-        raise ValueError(f"not a tensor statistics line: {line!r}")
-    return {
-        "node_id": int(line.split(":")[0].strip()),
-        "tensor_name": m["tensor"].group(1), "counter": int(m["tensor"].group(2)), "step": int(m["tensor"].group(3)),
-        "tensor_dimension": m["dimension"].group(1) if m["dimension"] else None,
-        "global_non_zero": int(m["non_zero"].group(1)), "global_error": float(m["global_error"].group(1)),
-        "relative_error": float(m["relative_error"].group(1)),
-        "histogram": [int(v) for v in m["histogram"].group(1).split(",")],
-    }
 
 
 def block_error_histogram(x: Tensor, q: Tensor, block_rows: int, block_cols: int, bin_width: float = BIN_WIDTH,

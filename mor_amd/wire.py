@@ -89,3 +89,21 @@ def fake_quantize_mx_dual(x: Tensor, mode: int = 2, sf_type: int = 2) -> Tuple[T
         _cabi.check(_L.mor_fake_quantize_dual(x.data_ptr(), out.data_ptr(), meta.data_ptr(), out_t.data_ptr(), meta_t.data_ptr(),
                                               rows, cols, mode, sf_type, _stream(x)))
     return out, meta, out_t, meta_t
+
+
+def fake_quantize_tiles_dual(x: Tensor, clamp_threshold: float = 0.0, mode: int = 1, sf_type: int = 1) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """One read of x, 128 x 128 tiles: (out, meta) = mor.ops.fake_quantize(x, rows, cols, 128, 128, clamp_threshold,
+    mode, sf_type) and (out_t, meta_t) = the same op on x.t().contiguous(), without materialising the transpose.
+    mode % 10: 1 = MoR, 2 = E4M3, 3 = E5M2."""
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_cuda:
+        raise RuntimeError("mor: expected a 2-D bfloat16 GPU tensor")
+    rows, cols = x.shape
+    x = x.contiguous()
+    with torch.cuda.device(x.device):
+        out = torch.empty_like(x)
+        out_t = torch.empty((cols, rows), dtype=torch.bfloat16, device=x.device)
+        meta = torch.empty((max(rows // 128, 1), max(cols // 128, 1)), dtype=torch.int32, device=x.device)
+        meta_t = torch.empty((max(cols // 128, 1), max(rows // 128, 1)), dtype=torch.int32, device=x.device)
+        _cabi.check(_L.mor_fake_quantize_dual_tiles(x.data_ptr(), out.data_ptr(), meta.data_ptr(), out_t.data_ptr(), meta_t.data_ptr(),
+                                                    rows, cols, float(clamp_threshold), mode, sf_type, _stream(x)))
+    return out, meta, out_t, meta_t

@@ -18,7 +18,8 @@ def test_tensor_log_line_matches_oracle_scalars():
     a = xb.view(torch.int16).numpy().view(np.uint16).copy()
     print("stats line 512x768", flush=True)
     line = stats.tensor_log_line(3, "layers.0.attn.qkv.weight", 10, 2, xb.cuda())
-    p = stats.parse_log_line(line)
+    import log_line_fields
+    p = log_line_fields.parse(line)
     _, _, _, wnnz, werr = O.block_scaling(a, 128, 128, 1.0e30, 3)
     assert p["node_id"] == 3 and p["tensor_name"] == "layers.0.attn.qkv.weight" and p["counter"] == 10 and p["step"] == 2
     assert p["tensor_dimension"] == "512x768" and p["global_non_zero"] == int(wnnz[0]) == int((xb != 0).sum())

