@@ -117,7 +117,7 @@ def read_traffic(kernel):
     """-> (HBM bytes per launch of `kernel`, where the figure comes from).  Hardware counters cannot be read from inside
     the run: the figure is the one in the committed counter summary (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
     script, each scaled by the same counter's reading for the library's plain copy kernel); None when it holds none."""
-    rel = os.path.join("profiles", "hbm_traffic_counters.txt")
+    rel = os.path.join("profiles", "bench_step_mx_1x32_and_mor_128x128_8192x8192_hbm_traffic.txt")
     try:
         for line in open(os.path.join(ROOT, rel)):
             f = line.split()
