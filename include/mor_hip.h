@@ -184,6 +184,17 @@ MOR_API int mor_selftest_hw_cast(uint64_t* mismatches, void* stream);
 MOR_API int mor_selftest_hw_wire(uint64_t* mismatches, void* stream);
 
 /*
+ * The MX wire format as operands of the gfx950 scaled matrix instruction (no counterpart in the
+ * reference): out [16, 16] fp32 = A x B^T for two [16, 128] tensors given as mor_mx_quantize gives
+ * them (payload: 16 rows x 4 blocks of 32 codes, scales: 16 x 4 E8M0 bytes), computed by one
+ * V_MFMA_SCALE_F32_16X16X128_F8F6F4 whose lanes load a block of codes and its scale byte each, with
+ * no conversion in between.  Equals the product of the dequantized tensors up to the fp32
+ * accumulation.  fmt = MOR_FMT_*, the same for both operands; payloads 4-byte aligned.
+ */
+MOR_API int mor_selftest_mx_mfma(const void* payload_a, const void* scales_a, const void* payload_b,
+                                 const void* scales_b, int fmt, float* out, void* stream);
+
+/*
  * MX wire format: the quantized tensor itself instead of its dequantized bf16 image.
  *
  * No counterpart in the reference, whose ops all return bf16 (FQ:1839-1871).  For blocks of 32

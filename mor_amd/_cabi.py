@@ -33,6 +33,7 @@ SIGNATURES = {
     "mor_mor_stats": (_int, [_vp, _i64, _i64, _i64, _i64, _f64, _i64, _i64, _vp, _vp]),
     "mor_selftest_hw_cast": (_int, [_vp, _vp]),
     "mor_selftest_hw_wire": (_int, [_vp, _vp]),
+    "mor_selftest_mx_mfma": (_int, [_vp, _vp, _vp, _vp, _int, _vp, _vp]),
     "mor_mx_payload_bytes": (_sz, [_i64, _i64, _int]),
     "mor_mx_quantize": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
     "mor_mx_quantize_dual": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _vp]),

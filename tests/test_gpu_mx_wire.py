@@ -6,6 +6,7 @@ import torch
 
 from oracle import mor_oracle as O
 import data_gen
+import torch_emulation as E
 
 pytestmark = pytest.mark.gpu
 
@@ -174,3 +175,40 @@ def test_hw_scaled_converts_selftest(G):
     _cabi.check(L.mor_selftest_hw_wire(bad.data_ptr(), None))
     torch.cuda.synchronize()
     assert bad.tolist() == [0, 0, 0, 0]
+
+
+@pytest.mark.parametrize("fmt", [0, 1, 2, 3])
+def test_scaled_mfma_consumes_the_wire_format(G, fmt):
+    """Payload and scale bytes of mor_mx_quantize, loaded as they lie in memory, are the operands of the gfx950 scaled
+    matrix instruction: its 16 x 16 x 128 product equals the product of the dequantized tensors (exact in float64: the
+    operands are small dyadic numbers) up to the fp32 accumulation of 128 terms."""
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    rng = np.random.default_rng(40 + fmt)
+    for trial in range(6):
+        wide = trial % 2 == 0                # blocks with scales of their own (2^-20 .. 2^20) / one scale for all
+        mats = []
+        for _ in range(2):
+            x = rng.standard_normal((16, 128)).astype(np.float32)
+            if wide:
+                x *= np.exp2(rng.integers(-20, 20, (16, 4))).repeat(32, axis=1).astype(np.float32)
+            if trial == 3:
+                x[3, 32:64] = 0                                                                     # an all-zero block
+            mats.append(torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16).copy())
+        q = [G.mx_quantize(m, fmt) for m in mats]                    # (payload, scales) as numpy uint8
+        deq = [E.bits_to_bf16(G.mx_dequantize(p, s, fmt)).double().numpy() for p, s in q]
+        want = deq[0] @ deq[1].T
+        bound = np.abs(deq[0]) @ np.abs(deq[1]).T
+        dev = [[torch.from_numpy(np.ascontiguousarray(t)).to(G.dev()) for t in ps] for ps in q]
+        out = torch.zeros((16, 16), dtype=torch.float32, device=G.dev())
+        _cabi.check(L.mor_selftest_mx_mfma(dev[0][0].data_ptr(), dev[0][1].data_ptr(), dev[1][0].data_ptr(), dev[1][1].data_ptr(),
+                                           fmt, out.data_ptr(), G.stream_ptr()))
+        torch.cuda.synchronize()
+        got = out.cpu().double().numpy()
+        # the instruction aligns the products of a row to the largest before it adds them, so small ones lose bits
+        # (measured, as a fraction of the sum of magnitudes: 3e-5 with scales 2^40 apart, 7e-6 with one scale, 4e-8 for
+        # E3M2); a wrong layout would be wrong by the sum itself
+        tol = 1e-4 if wide else 2e-5
+        excess = np.max(np.abs(got - want) / (bound + 1e-300))
+        print(f"scaled mfma fmt {fmt} trial {trial}: max |error| / sum of magnitudes {excess:.3e}", flush=True)
+        assert excess <= tol, f"fmt {fmt} trial {trial}: {excess:.3e}"
