@@ -83,21 +83,6 @@ __global__ __launch_bounds__(WG) void k_batch(BatchArgs a, int fast_ok) {
 
 using namespace mor;
 
-// mode / sf_type -> what the kernels take (FQ:1773-1779, 1792-1834); false for the modes that copy
-static bool decode_mode(int64_t mode, double clamp, QuantArgs& qa) {
-    qa = QuantArgs{};
-    qa.clamp = (float)clamp;
-    qa.dyn_range = (mode / 100 > 0) ? 1 : 0;
-    switch ((int)(mode % 10)) {
-        case 1: qa.qmode = 1; qa.fmt = -1; qa.meta_val = -1; return true;
-        case 2: qa.qmode = 2; qa.fmt = FMT_E4M3; qa.meta_val = 1; return true;
-        case 3: qa.qmode = 2; qa.fmt = FMT_E5M2; qa.meta_val = 2; return true;
-        case 4: qa.qmode = 4; qa.fmt = FMT_E4M3; qa.meta_val = 1; return true;
-        case 5: qa.qmode = 4; qa.fmt = FMT_E5M2; qa.meta_val = 2; return true;
-        default: return false;
-    }
-}
-
 extern "C" int mor_fake_quantize_batch(const MorTensorDesc* descs, int64_t n, uint32_t flags, void* stream) {
     if (n < 0 || (n > 0 && !descs)) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "bad descriptor array");
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -127,7 +112,7 @@ extern "C" int mor_fake_quantize_batch(const MorTensorDesc* descs, int64_t n, ui
         }
         BatchItem& it = a.item[a.n];
         QuantArgs qa;
-        const bool quantizes = decode_mode(d.mode, d.clamp_threshold, qa);
+        const bool quantizes = mor_decode_mode(d.mode, d.clamp_threshold, qa);
         it = BatchItem{};
         it.in = static_cast<const uint16_t*>(d.input);
         it.out = static_cast<uint16_t*>(d.output);

@@ -71,7 +71,8 @@ template <int NW> __device__ __forceinline__ uint32_t lds_umin(const uint32_t* s
     return m;
 }
 template <int NW> __device__ __forceinline__ float lds_sum(const float* s) {
-    static_assert(NW == 4 || NW == 8 || NW == 16, "4, 8 or 16 waves");
+    static_assert(NW == 1 || NW == 4 || NW == 8 || NW == 16, "1, 4, 8 or 16 waves");
+    if constexpr (NW == 1) return s[0];
     float a = (s[0] + s[1]) + (s[2] + s[3]);
     if constexpr (NW >= 8) a += (s[4] + s[5]) + (s[6] + s[7]);
     if constexpr (NW == 16) a += ((s[8] + s[9]) + (s[10] + s[11])) + ((s[12] + s[13]) + (s[14] + s[15]));

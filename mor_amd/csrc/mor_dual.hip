@@ -40,15 +40,9 @@ extern "C" int mor_fake_quantize_dual_tiles(const void* input, void* output, int
         return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensors must be 16-byte aligned");
     if (input == output || input == output_t || output == output_t)
         return mor_fail(MOR_ERR_INVALID_ARGUMENT, "input and the two outputs must be three different tensors");
-    QuantArgs qa{};
-    qa.clamp = (float)clamp_threshold;
-    qa.dyn_range = (mode / 100 > 0) ? 1 : 0;            // FQ:1776-1779
-    switch ((int)(mode % 10)) {                         // FQ:1774, 1792-1834
-        case 1: qa.qmode = 1; qa.fmt = -1; qa.meta_val = -1; break;
-        case 2: qa.qmode = 2; qa.fmt = FMT_E4M3; qa.meta_val = 1; break;
-        case 3: qa.qmode = 2; qa.fmt = FMT_E5M2; qa.meta_val = 2; break;
-        default: return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mode %% 10 must be 1 (MoR), 2 (E4M3) or 3 (E5M2), got %lld", (long long)mode);
-    }
+    QuantArgs qa;
+    if (!mor_decode_mode(mode, clamp_threshold, qa) || qa.qmode == 4)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mode %% 10 must be 1 (MoR), 2 (E4M3) or 3 (E5M2), got %lld", (long long)mode);
     const Shape sh = make_shape(rows, cols, 128, 128);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint4* in = static_cast<const uint4*>(input);

@@ -37,6 +37,21 @@ __global__ __launch_bounds__(WG) void k_generic(const uint16_t* in, uint16_t* ou
     generic_block<EMU, true>(in, out, meta, stats, sh, qa, (e8 & 1) != 0, first + blockIdx.x, s_f, s_u, (e8 & 2) != 0);
 }
 
+// Small blocks (up to 512 elements) that no vector kernel serves, e.g. 1 x 32 blocks on a tensor with an odd column
+// count: a workgroup is one wave and takes `per_wave` consecutive blocks, so that 32 blocks are in flight per CU
+// instead of 8 and a workgroup's start-up is shared (4097 x 4095 in 1 x 32 blocks: 0.5 ms with a 256-thread
+// workgroup per block).
+template <bool EMU>
+__global__ __launch_bounds__(64) void k_generic_wave(const uint16_t* in, uint16_t* out, int32_t* __restrict__ meta,
+                                                     float* __restrict__ stats, Shape sh, QuantArgs qa, int e8, int64_t first,
+                                                     int64_t nblocks, int per_wave) {
+    __shared__ float s_f[2][1];
+    __shared__ uint32_t s_u[1];
+    const int64_t b0 = first + (int64_t)blockIdx.x * per_wave;
+    for (int i = 0; i < per_wave && b0 + i < nblocks; ++i)
+        generic_block<EMU, true, 64>(in, out, meta, stats, sh, qa, (e8 & 1) != 0, b0 + i, s_f, s_u, (e8 & 2) != 0);
+}
+
 // ------------------------------------------------------------------------------------------------
 // k_elementwise: modes 4 / 5 (FQ:825-842): every element uses the caller's scale; meta is a constant.
 // The host picks the fast kernel when the scale is in the fast range, else (or for the other flavours) the exact one.
@@ -462,12 +477,20 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
         mor_launch_bigblock(mor_mode, e8, input, output, meta, stats, sh, qa, st);
         return mor_check_launch("k_bigblock");
     }
+    // bit 0: power-of-two scale; bit 1: the few-instruction arithmetic (hardware converts) is allowed
+    const int gflags = (e8 ? 1 : 0) | (fast_ok ? 2 : 0);
+    if (brows * bcols <= 512) {
+        constexpr int PER_WAVE = 8;
+        for_slices(cdiv(nblocks, PER_WAVE), [&](int64_t first, int count) {
+            if (emu) k_generic_wave<true><<<count, 64, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags, first * PER_WAVE, nblocks, PER_WAVE);
+            else k_generic_wave<false><<<count, 64, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags, first * PER_WAVE, nblocks, PER_WAVE);
+        });
+        return mor_check_launch("k_generic_wave");
+    }
     if (fast_ok && brows * ((bcols + 1) / 2) <= 32 * WG && brows * cols < 0x7FFFFFFFll && nblocks <= 0x7FFFFFFFll) {
         mor_launch_wgblock(mor_mode, e8, true, input, output, meta, stats, sh, qa, st);
         return mor_check_launch("k_wgblock (element-wise)");
     }
-    // bit 0: power-of-two scale; bit 1: the few-instruction arithmetic (hardware converts) is allowed
-    const int gflags = (e8 ? 1 : 0) | (fast_ok ? 2 : 0);
     for_slices(nblocks, [&](int64_t first, int count) {
         if (emu) k_generic<true><<<count, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags, first);
         else k_generic<false><<<count, WG, 0, st>>>(in16, out16, meta, stats, sh, qa, gflags, first);
@@ -482,32 +505,22 @@ extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
     if (int rc = mor_validate_shape(input, rows, cols, brows, bcols)) return rc;
     if (!output || !meta) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output / meta is NULL");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int qmode = (int)(mode % 10);                 // FQ:1774
-    QuantArgs qa{};
-    qa.clamp = (float)clamp_threshold;
-    qa.dyn_range = (mode / 100 > 0) ? 1 : 0;            // FQ:1776-1779
+    QuantArgs qa;
     const bool e8 = (sf_type == 2);                     // FQ:1792, 1797
-    switch (qmode) {
-        case 1: qa.qmode = 1; qa.fmt = -1; qa.meta_val = -1; break;
-        case 2: qa.qmode = 2; qa.fmt = FMT_E4M3; qa.meta_val = 1; break;
-        case 3: qa.qmode = 2; qa.fmt = FMT_E5M2; qa.meta_val = 2; break;
-        case 4: qa.qmode = 4; qa.fmt = FMT_E4M3; qa.meta_val = 1; break;
-        case 5: qa.qmode = 4; qa.fmt = FMT_E5M2; qa.meta_val = 2; break;
-        default: {
-            // FQ:1831-1833, 727-729, 843: bf16 copy, meta 3
-            const int64_t nblocks = cdiv(rows, brows) * cdiv(cols, bcols);
-            if (output != input) {
-                const int64_t n = rows * cols;
-                const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
-                const uint16_t* i16 = static_cast<const uint16_t*>(input);
-                uint16_t* o16 = static_cast<uint16_t*>(output);
-                // (from HBM one vector per lane copies fastest, as in k_rowgroup)
-                if (nvec >= ((int64_t)4 << 20)) k_copy<1><<<(int)cdiv(nvec, (int64_t)WG), WG, 0, st>>>(i16, o16, n, nvec);
-                else k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(i16, o16, n, nvec);
-            }
-            k_fill_i32<<<grid_for(nblocks), WG, 0, st>>>(meta, nblocks, 3);
-            return mor_check_launch("k_copy / k_fill_i32");
+    if (!mor_decode_mode(mode, clamp_threshold, qa)) {
+        // FQ:1831-1833, 727-729, 843: bf16 copy, meta 3
+        const int64_t nblocks = cdiv(rows, brows) * cdiv(cols, bcols);
+        if (output != input) {
+            const int64_t n = rows * cols;
+            const int64_t nvec = (aligned16(input) && aligned16(output)) ? n / 8 : 0;
+            const uint16_t* i16 = static_cast<const uint16_t*>(input);
+            uint16_t* o16 = static_cast<uint16_t*>(output);
+            // (from HBM one vector per lane copies fastest, as in k_rowgroup)
+            if (nvec >= ((int64_t)4 << 20)) k_copy<1><<<(int)cdiv(nvec, (int64_t)WG), WG, 0, st>>>(i16, o16, n, nvec);
+            else k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(i16, o16, n, nvec);
         }
+        k_fill_i32<<<grid_for(nblocks), WG, 0, st>>>(meta, nblocks, 3);
+        return mor_check_launch("k_copy / k_fill_i32");
     }
     return run_quantize(input, output, meta, nullptr, rows, cols, brows, bcols, qa, e8, flags, st);
 }

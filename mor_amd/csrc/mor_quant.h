@@ -273,6 +273,23 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
 
 }  // namespace mor
 
+// mode / clamp_threshold of the fake_quantize ops -> what the kernels take (FQ:1773-1779, 1792-1834).  Returns false
+// for the mode digits that copy the tensor (meta 3).
+static inline bool mor_decode_mode(int64_t mode, double clamp_threshold, mor::QuantArgs& qa) {
+    qa = mor::QuantArgs{};
+    qa.clamp = (float)clamp_threshold;
+    qa.dyn_range = (mode / 100 > 0) ? 1 : 0;
+    switch ((int)(mode % 10)) {
+        case 1: qa.qmode = 1; qa.fmt = -1; qa.meta_val = -1; return true;
+        case 2: qa.qmode = 2; qa.fmt = mor::FMT_E4M3; qa.meta_val = 1; return true;
+        case 3: qa.qmode = 2; qa.fmt = mor::FMT_E5M2; qa.meta_val = 2; return true;
+        case 4: qa.qmode = 4; qa.fmt = mor::FMT_E4M3; qa.meta_val = 1; return true;
+        case 5: qa.qmode = 4; qa.fmt = mor::FMT_E5M2; qa.meta_val = 2; return true;
+        default: return false;
+    }
+}
+
+
 // A launch holds fewer than 2^32 threads per dimension (a larger grid wraps without an error): kernels that take one
 // workgroup per block are launched slice by slice, f(first block, blocks of the slice).
 constexpr int64_t LAUNCH_SLICE = (int64_t)1 << 22;
