@@ -281,8 +281,9 @@ def other_configs(torch, run, cabi, K, W):
 
     def add(name, fn, nbytes, nelem):
         ms, wall = time_launches(torch, fn, K, W)
-        if ms * K < 10.0:       # short bursts are noisy (clock ramp, refresh): time about 10 ms of back-to-back launches
-            ms, wall = time_launches(torch, fn, min(1000, int(10.0 / ms) + 1), W)
+        # short bursts after idle are not the sustained rate (clock ramp; the MoR kernels run 15 % slower between 2 and
+        # 8 ms into a burst): 30 ms of untimed launches, then about 10 ms of timed ones
+        ms, wall = time_launches(torch, fn, min(1000, max(K, int(10.0 / ms) + 1)), min(3000, int(30.0 / ms) + 1))
         res[name] = {"ms": round(ms, 5), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "elements_per_s": round(nelem / (ms * 1e-3), 0)}
 
@@ -310,6 +311,7 @@ def other_configs(torch, run, cabi, K, W):
         add(key, lambda: cabi.check(run.L.mor_fake_quantize_dual_tiles(x.data_ptr(), out.data_ptr(), meta.data_ptr(), out_t.data_ptr(),
                                                                          meta_t.data_ptr(), 8192, 8192, 1e-15, mode, 1, st_())), n * 6, n)
     del out_t
+    mor_tile_codes(torch, cabi, run, add, x, out, "8192x8192_normal")
     # C1: per-tensor E4M3, 4096x4096, scale from the tensor amax (the quantize pass only: 4 B/element)
     x1 = x[:4096, :4096].contiguous()
     o1 = torch.empty_like(x1)
@@ -342,6 +344,7 @@ def other_configs(torch, run, cabi, K, W):
     torch.cuda.synchronize()
     hist = torch.bincount(m4.flatten(), minlength=13).tolist()
     res["c4_mor_128x128_16384x14336_mixture"]["meta_histogram"] = {str(i): h for i, h in enumerate(hist) if h}
+    mor_tile_codes(torch, cabi, run, add, x4, o4, "16384x14336_mixture")
     del x4, o4
     res["flavour_differences"] = flavour_differences(torch, run, cabi)
     res["c5_llama3_8b_layer"] = c5_sweep(torch, run, max(3, K // 4), 2)
@@ -381,6 +384,29 @@ def other_configs(torch, run, cabi, K, W):
         ms, wall = time_launches(torch, lambda: mor.ops.fake_quantize(t, 1, 32, 1, 32, 0.0, 2, 2), 500, 50)
         res["tiny_1x32"][key] = round(wall * 1e3, 2)
     return res
+
+
+def mor_tile_codes(torch, cabi, run, add, x, out, label):
+    """MoR per 128 x 128 tile with the codes as the result (tag + fp32 scale + payload) and the decode back to bf16.
+    Bytes: the bf16 tensor on one side, on the other what the tiles' formats take (1 B/element for E4M3 / E5M2, 0.75 for
+    E2M3, 2 for BF16) plus 8 bytes of tag and scale per tile."""
+    from mor_amd.wire import TILE_PAYLOAD_BYTES, TILE_STORED_BF16
+    rows, cols = x.shape
+    gy, gx = rows // 128, cols // 128
+    payload = torch.empty((gy, gx, TILE_PAYLOAD_BYTES), dtype=torch.uint8, device="cuda")
+    tags = torch.empty((gy, gx), dtype=torch.int32, device="cuda")
+    scales = torch.empty((gy, gx), dtype=torch.float32, device="cuda")
+    L, st = run.L, run.stream
+    enc = lambda: cabi.check(L.mor_mor_quantize(x.data_ptr(), payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), rows, cols, 1e-15, 1, st()))
+    dec = lambda: cabi.check(L.mor_mor_dequantize(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, cols, st()))
+    enc()
+    torch.cuda.synchronize()
+    t = tags.flatten()
+    wide = ((t & TILE_STORED_BF16) != 0) | (t == 3)
+    code_bytes = int(wide.sum()) * 32768 + int(((t == 4) & ~wide).sum()) * 12288 + int((~wide & (t != 4)).sum()) * 16384
+    n = x.numel()
+    add("mor_tile_codes_quantize_" + label, enc, 2 * n + code_bytes + 8 * t.numel(), n)
+    add("mor_tile_codes_dequantize_" + label, dec, 2 * n + code_bytes + 8 * t.numel(), n)
 
 
 def flavour_differences(torch, run, cabi):

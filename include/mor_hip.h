@@ -255,6 +255,33 @@ MOR_API int mor_fake_quantize_dual_tiles(const void* input, void* output, int32_
                                          int32_t* meta_t, int64_t rows, int64_t cols, double clamp_threshold,
                                          int64_t mode, int64_t sf_type, void* stream);
 
+/*
+ * The MoR decision per 128 x 128 tile with the tile's codes as the result, and the way back (no
+ * counterpart in the reference, which only ever materialises the fake-quantized bf16 values,
+ * FQ:733-851; this is what a real low-precision GEMM after the MoR decision would read):
+ *   tags   [rows / 128, cols / 128] int32: the meta value mor_fake_quantize(input, rows, cols, 128, 128,
+ *          clamp_threshold, mode, 1) gives the tile (1 / 11 E4M3, 2 / 12 E5M2, 3 BF16, 4 E2M3).  A tile
+ *          whose scale is outside 2^-90 .. 2^90 or that holds a NaN has MOR_TILE_STORED_BF16 ORed in.
+ *   scales [rows / 128, cols / 128] float: the tile's fp32 scale fmax / amax (FQ:297-304); 1 for a
+ *          BF16 tile, a tile stored as bf16 and an all-zero tile.
+ *   payload: MOR_TILE_PAYLOAD_BYTES per tile, tile after tile in row-major tile order.  A tile
+ *          holds its 128 rows packed: E4M3 / E5M2 128 bytes per row (one code per element: the
+ *          OCP code of |x| * scale, the sign of x in bit 7); E2M3 96 bytes per row (6-bit codes,
+ *          dense little-endian, code k at bits 6k; a zero result has no sign, as the reference's
+ *          software cast gives +0); BF16 (and MOR_TILE_STORED_BF16) 256 bytes per row: the bf16
+ *          values mor_fake_quantize writes for the tile.  The rest of a tile's slot is not written.
+ * mor_mor_dequantize gives the output of that mor_fake_quantize call bit for bit: value of the code,
+ * divided by the scale (IEEE), rounded to bf16 half-up (FQ:312-316).
+ * mode % 10 must be 1, mode / 100 as in mor_fake_quantize; default flavour, fp32 scales.
+ * rows and cols multiples of 128; tensor and payload 16-byte aligned, different buffers.
+ */
+#define MOR_TILE_PAYLOAD_BYTES 32768
+#define MOR_TILE_STORED_BF16 0x100
+MOR_API int mor_mor_quantize(const void* input, void* payload, int32_t* tags, float* scales, int64_t rows,
+                             int64_t cols, double clamp_threshold, int64_t mode, void* stream);
+MOR_API int mor_mor_dequantize(const void* payload, const int32_t* tags, const float* scales, void* output,
+                               int64_t rows, int64_t cols, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

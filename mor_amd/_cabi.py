@@ -40,6 +40,8 @@ SIGNATURES = {
     "mor_mx_dequantize": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
     "mor_fake_quantize_dual": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "mor_fake_quantize_dual_tiles": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _i64, _i64, _vp]),
+    "mor_mor_quantize": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f64, _i64, _vp]),
+    "mor_mor_dequantize": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
 }
 
 _lib = None

@@ -15,9 +15,9 @@ from concurrent.futures import ThreadPoolExecutor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(_HERE, "csrc")
 _ROOT = os.path.dirname(_HERE)
-SOURCES = [os.path.join(_CSRC, n) for n in ("mor_kernels.hip", "mor_wgblock.hip", "mor_subblock.hip", "mor_scaling.hip", "mor_wire.hip", "mor_batch.hip", "mor_dual.hip", "mor_mfma_check.hip")]
+SOURCES = [os.path.join(_CSRC, n) for n in ("mor_kernels.hip", "mor_wgblock.hip", "mor_subblock.hip", "mor_scaling.hip", "mor_wire.hip", "mor_batch.hip", "mor_dual.hip", "mor_morwire.hip", "mor_mfma_check.hip")]
 SOURCES = [s for s in SOURCES if os.path.exists(s)]
-HEADERS = [os.path.join(_CSRC, n) for n in ("mor_device.h", "mor_common.h", "mor_quant.h", "mor_wgblock.h", "mor_host.h")] + [os.path.join(_ROOT, "include", "mor_hip.h")]
+HEADERS = [os.path.join(_CSRC, n) for n in ("mor_device.h", "mor_common.h", "mor_quant.h", "mor_wgblock.h", "mor_wirefmt.h", "mor_host.h")] + [os.path.join(_ROOT, "include", "mor_hip.h")]
 VERSION_SRC = os.path.join(_CSRC, "mor_version.cpp")
 OUT = os.path.join(_HERE, "lib", "libmor_hip.so")
 HASH_FILE = os.path.join(_HERE, "lib", "libmor_hip.srchash")           # the source hash libmor_hip.so was built from

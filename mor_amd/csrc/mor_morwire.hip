@@ -1,0 +1,146 @@
+// mor_mor_quantize / mor_mor_dequantize: the MoR decision per 128 x 128 tile with the tile's codes as the result
+// (format tag + fp32 scale + payload) instead of the fake-quantized bf16 values, and the way back.
+// The encoder is k_wgblock in its WIRE form (same passes 1 and 2, codes stored in pass 3); the decoder below repeats
+// the second half of the bf16 kernel's pass 3 (code -> value, division by the scale, bf16 store), so that
+// decode(encode(x)) is the output of mor_fake_quantize bit for bit.
+// "FQ" below is the reference file mor/csrc/cuda/fake_quantize.cu.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mor_wgblock.h"
+#include "mor_host.h"
+#include "../../include/mor_hip.h"
+
+using namespace mor;
+
+static_assert(TILE_PAYLOAD_BYTES == MOR_TILE_PAYLOAD_BYTES && TILE_STORED_BF16 == MOR_TILE_STORED_BF16, "header constants");
+
+namespace mor {
+
+// One workgroup per tile; lane (row r, chunk cc) of step k decodes 8 codes into one 16-byte vector of the output,
+// the mapping the encoder wrote them with.  The reads of a tile are one linear run of 16 / 12 / 32 KiB.
+template <int NT>
+__global__ __launch_bounds__(WG) void k_mor_decode(const uint8_t* __restrict__ payload, const int32_t* __restrict__ tags,
+                                                   const float* __restrict__ scales, uint4* __restrict__ out, Shape sh,
+                                                   int band, int64_t first) {
+    const int tid = threadIdx.x;
+    uint32_t bid = (uint32_t)(first + blockIdx.x);
+    if (band) bid = band_order(sh, bid);
+    uint32_t by, bx;
+    block_of(sh, bid, by, bx);
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3);
+    uint4* bout = out + ((int64_t)by * 128 * row_stride + (int64_t)bx * 16);
+    const uint8_t* tile = payload + (int64_t)bid * TILE_PAYLOAD_BYTES;
+    const int tag = tags[bid];
+    const int fmt = (tag & TILE_STORED_BF16) ? -1 : mor_fmt_of(tag);
+    const float s = scales[bid];
+    const float r = 1.0f / s;
+    // (the format is uniform over the workgroup: each case loads its 8 vectors first, then converts and stores)
+    auto put = [&](int k, uint4 q) {
+        const int ch = k * WG + tid;
+        store16<(NT != 0)>(bout + (uint32_t)(ch >> 4) * row_stride + (uint32_t)(ch & 15), q);
+    };
+    if (fmt < 0) {
+        uint4 c[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) c[k] = reinterpret_cast<const uint4*>(tile)[k * WG + tid];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) put(k, c[k]);
+    } else if (fmt == FMT_E4M3 || fmt == FMT_E5M2) {
+        uint2 c[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) c[k] = reinterpret_cast<const uint2*>(tile)[k * WG + tid];
+        auto decode = [&](auto unpack) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t c2[4] = {c[k].x & 0xFFFFu, c[k].x >> 16, c[k].y & 0xFFFFu, c[k].y >> 16};
+                uint32_t w[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const f32x2 d = unpack(c2[j] & 0x7F7Fu);
+                    const uint32_t sign = ((c2[j] & 0x80u) << 8) | ((c2[j] & 0x8000u) << 16);
+                    w[j] = store_pair<false>(div_by_scale(d.x, s, r), div_by_scale(d.y, s, r)) | sign;
+                }
+                put(k, make_uint4(w[0], w[1], w[2], w[3]));
+            }
+        };
+        if (fmt == FMT_E4M3) decode([](uint32_t m) { return hw_unpack2_low<FMT_E4M3>(m); });
+        else decode([](uint32_t m) { return hw_unpack2_low<FMT_E5M2>(m); });
+    } else {
+        uint16_t c[8][3];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint16_t* p = reinterpret_cast<const uint16_t*>(tile) + 3 * (k * WG + tid);
+            c[k][0] = p[0]; c[k][1] = p[1]; c[k][2] = p[2];
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint64_t bits = (uint64_t)c[k][0] | ((uint64_t)c[k][1] << 16) | ((uint64_t)c[k][2] << 32);
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t ca = (uint32_t)(bits >> (12 * j)) & 0x3Fu, cb = (uint32_t)(bits >> (12 * j + 6)) & 0x3Fu;
+                const float da = fp6_value<FMT_E2M3>(ca & 0x1Fu), db = fp6_value<FMT_E2M3>(cb & 0x1Fu);
+                const uint32_t sign = ((ca & 0x20u) << 10) | ((cb & 0x20u) << 26);
+                w[j] = store_pair<false>(div_by_scale(da, s, r), div_by_scale(db, s, r)) | sign;
+            }
+            put(k, make_uint4(w[0], w[1], w[2], w[3]));
+        }
+    }
+}
+
+}  // namespace mor
+
+static int check_tiles(const void* a, const void* b, const void* tags, const void* scales, int64_t rows, int64_t cols) {
+    if (int rc = mor_validate_shape(a, rows, cols, 128, 128)) return rc;
+    if (!b || !tags || !scales) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "NULL payload, tags or scales pointer");
+    if (rows % 128 || cols % 128)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "rows and cols must be multiples of 128 (got %lld x %lld)", (long long)rows, (long long)cols);
+    if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor and payload must be 16-byte aligned");
+    if (a == b) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor and payload must be different buffers");
+    return MOR_OK;
+}
+
+extern "C" int mor_mor_quantize(const void* input, void* payload, int32_t* tags, float* scales, int64_t rows, int64_t cols,
+                                double clamp_threshold, int64_t mode, void* stream) {
+    if (int rc = check_tiles(input, payload, tags, scales, rows, cols)) return rc;
+    QuantArgs qa;
+    if (!mor_decode_mode(mode, clamp_threshold, qa) || qa.qmode != 1)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mode %% 10 must be 1 (MoR), got %lld", (long long)mode);
+    const Shape sh = make_shape(rows, cols, 128, 128);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t nblocks = sh.gy * sh.gx;
+    // loads and XCD bands as for the bf16 kernel (launch_wgblock_nv)
+    const bool stream_loads = rows * cols * 2 >= ((int64_t)64 << 20);
+    const int shift = (nblocks >= 2048 && sh.gx % 8 == 0 && nblocks % 8 == 0) ? (4 | 256) : 4;
+    // four workgroups per CU on large grids (the bf16 kernel runs three: half the bytes are written here; 8192^2 from HBM:
+    // 42.0 us with three, 39.3 with four, 39.1 - 40.0 without a cap)
+    const size_t dl = nblocks >= 4096 ? 36000 : 0;
+    const uint4* in = static_cast<const uint4*>(input);
+    uint4* out = static_cast<uint4*>(payload);
+    for_slices(nblocks, [&](int64_t first, int count) {
+        if (stream_loads) k_wgblock<true, false, 8, true, 1, WG, false, false, true><<<count, WG, dl, st>>>(in, out, tags, scales, sh, qa, 16, shift, first, nullptr, nullptr);
+        else k_wgblock<true, false, 8, true, 0, WG, false, false, true><<<count, WG, dl, st>>>(in, out, tags, scales, sh, qa, 16, shift, first, nullptr, nullptr);
+    });
+    return mor_check_launch("k_wgblock (tile codes)");
+}
+
+extern "C" int mor_mor_dequantize(const void* payload, const int32_t* tags, const float* scales, void* output, int64_t rows,
+                                  int64_t cols, void* stream) {
+    if (int rc = check_tiles(output, payload, tags, scales, rows, cols)) return rc;
+    const Shape sh = make_shape(rows, cols, 128, 128);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t nblocks = sh.gy * sh.gx;
+    const int band = (nblocks >= 2048 && sh.gx % 8 == 0 && nblocks % 8 == 0) ? 1 : 0;
+    const bool nt = rows * cols * 2 >= ((int64_t)4 << 20);
+    const uint8_t* p = static_cast<const uint8_t*>(payload);
+    uint4* out = static_cast<uint4*>(output);
+    for_slices(nblocks, [&](int64_t first, int count) {
+        // (full occupancy: 8192^2 from HBM 37.4 us; capped at 4 / 3 workgroups per CU 43 / 53 us)
+        if (nt) k_mor_decode<1><<<count, WG, 0, st>>>(p, tags, scales, out, sh, band, first);
+        else k_mor_decode<0><<<count, WG, 0, st>>>(p, tags, scales, out, sh, band, first);
+    });
+    return mor_check_launch("k_mor_decode");
+}

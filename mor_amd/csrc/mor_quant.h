@@ -185,7 +185,9 @@ __device__ __forceinline__ void for_block_elements(int64_t bh, int64_t bw, int64
 template <bool EMU, bool FAST = false, int WGS = WG>
 __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out, int32_t* meta, float* stats,
                                               const Shape& sh, const QuantArgs& qa, bool e8, int64_t bid,
-                                              float (*s_f)[WGS / 64], uint32_t* s_u, bool allow_fast = false) {
+                                              float (*s_f)[WGS / 64], uint32_t* s_u, bool allow_fast = false,
+                                              uint16_t* packed_out = nullptr) {
+    // packed_out: the block's result goes there with the rows bh x bw packed (row pitch sh.bcols) instead of into `out`
     constexpr int NW = WGS / 64;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     uint32_t by32, bx32;
@@ -253,20 +255,26 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
         if (meta && meta_val >= 0) meta[bid] = meta_val;
         if (stats) { float* s = stats + 4 * (int64_t)bid; s[0] = amax; s[1] = amin; s[2] = e4; s[3] = e5; }
     }
-    if (!out) return;
+    if (!out && !packed_out) return;
     const bool copy = (fmt < 0) || !(amax > 0.0f);
-    if (copy && out == in) return;
+    if (copy && out == in && !packed_out) return;
     const Scale sc = make_scale(copy ? 1.0f : fmax_of(fmt) / amax);
     uint16_t* bout = out + r0 * sh.cols + c0;
+    // where the element at offset `at` of the block (row pitch sh.cols) goes
+    auto dst = [&](int64_t at) -> uint16_t* {
+        if (!packed_out) return bout + at;
+        const int64_t r = at / sh.cols;                 // (rare path: a division per element does not matter)
+        return packed_out + r * sh.bcols + (at - r * sh.cols);
+    };
     bool fast = false;
     if constexpr (FAST && !EMU) fast = allow_fast && !copy && sc.fast && sc.e8 >= -90 && sc.e8 <= 90;
     if (fast) {
-        for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { bout[at] = fq_one_fast(bin[at], fmt, e8, sc); });
+        for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { *dst(at) = fq_one_fast(bin[at], fmt, e8, sc); });
     } else {
         for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) {
             uint16_t h = bin[at];
             if (!copy) h = fq_one_exact<EMU>(h, fmt, e8, sc);
-            bout[at] = h;
+            *dst(at) = h;
         });
     }
 }

@@ -3,6 +3,7 @@
 #pragma once
 
 #include "mor_quant.h"
+#include "mor_wirefmt.h"
 
 namespace mor {
 
@@ -26,11 +27,19 @@ template <class V> __device__ __forceinline__ void dual_tile_put(uint32_t* s_t, 
     const uint4 p = (R & 1) ? make_uint4(q.z, q.w, q.x, q.y) : make_uint4(q.x, q.y, q.z, q.w);
     *reinterpret_cast<uint4*>(s_t + r * 64 + ((cc ^ (R >> 1)) << 2)) = p;
 }
-template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false, bool DUAL = false>
+// WIRE (whole 128 x 128 tiles, 256 threads, MoR, fp32 scale): instead of the fake-quantized bf16 tile the kernel writes
+// the tile's codes: `out` is the payload, MOR_TILE_PAYLOAD_BYTES (32768) per tile, tile after tile in block order, rows
+// packed (128 rows of 128 one-byte codes, of 96 bytes of 6-bit codes, or of 256 bytes of bf16); `meta` takes the
+// storage format of each tile and `stats` one float per tile, its scale.  A tile whose scale is outside the fast range
+// (or that holds a NaN) is stored as the bf16 image of its fake-quantized values, its format ORed with TILE_STORED_BF16.
+constexpr int TILE_PAYLOAD_BYTES = 32768;
+constexpr int TILE_STORED_BF16 = 0x100;
+template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false, bool DUAL = false, bool WIRE = false>
 __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                  float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift,
                                                  int64_t first, uint4* out_t, int32_t* __restrict__ meta_t) {
     static_assert(!DUAL || (FULL && NV == 8 && WGS == 256 && !GATHER), "DUAL: whole 128 x 128 tiles");
+    static_assert(!WIRE || (MOR && !E8 && FULL && NV == 8 && WGS == 256 && !GATHER && !DUAL), "WIRE: MoR on whole 128 x 128 tiles, fp32 scale");
     constexpr int NW = WGS / 64;
     __shared__ __attribute__((aligned(16))) uint32_t s_t[DUAL ? 128 * 64 : 4];
     __shared__ float s_f[2][NW];
@@ -170,6 +179,13 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     s5.e8 = s4.e8 + 7;
     // (a NaN in the block shows as amax_b above the bits of infinity: the exact path takes its maximum as the reference does)
     if (amax_b > 0x7F800000u || (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast))) {           // uniform over the workgroup
+        if constexpr (WIRE) {
+            // the exact path's decision and values; the tile is stored as their bf16 image
+            generic_block<false, false, WGS>(reinterpret_cast<const uint16_t*>(in), nullptr, meta, nullptr, sh, qa, E8, bid, s_f, s_u, false,
+                                             reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(out) + (int64_t)bid * TILE_PAYLOAD_BYTES));
+            if (tid == 0) { meta[bid] |= TILE_STORED_BF16; stats[bid] = 1.0f; }      // (thread 0 wrote the decision there)
+            return;
+        }
         generic_block<false, false, WGS>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
                              sh, qa, E8, bid, s_f, s_u);
         if constexpr (DUAL) {
@@ -233,6 +249,51 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
         }
         meta_val = qt;
         fmt = mor_fmt_of(qt);
+    }
+    if constexpr (WIRE) {
+        // codes instead of values: tile `bid` of the payload, rows packed; lane (row r, chunk cc) writes its 8 codes
+        uint8_t* tile = reinterpret_cast<uint8_t*>(out) + (int64_t)bid * TILE_PAYLOAD_BYTES;
+        const bool zero_tile = !(amax > 0.0f);               // (decided as E2M3, FQ:620-627: all codes are signed zeros)
+        const Scale sc = make_scale((fmt < 0 || zero_tile) ? 1.0f : fmax_of(fmt) / amax);
+        if (tid == 0) { meta[bid] = meta_val; stats[bid] = sc.s; }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int ch = k * WGS + tid, r = ch >> 4, cc = ch & 15;
+            const uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+            if (fmt < 0) {
+                *reinterpret_cast<uint4*>(tile + r * 256 + cc * 16) = v[k];
+            } else if (fmt == FMT_E4M3 || fmt == FMT_E5M2) {
+                // the magnitudes' codes as pass 3 of the bf16 kernel computes them, the sign of the input on top
+                uint32_t c2[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float a = fabsf(bf16_lo(w[j])) * sc.s, b = fabsf(bf16_hi(w[j])) * sc.s;
+                    const uint32_t p = (fmt == FMT_E4M3) ? hw_pack2_low<FMT_E4M3>(a, b) : hw_pack2_low<FMT_E5M2>(a, b);
+                    c2[j] = (p & 0xFFFFu) | ((w[j] >> 8) & 0x80u) | ((w[j] >> 16) & 0x8000u);
+                }
+                *reinterpret_cast<uint2*>(tile + r * 128 + cc * 8) = make_uint2(c2[0] | (c2[1] << 16), c2[2] | (c2[3] << 16));
+            } else {
+                // E2M3 (the reference's software cast: a zero result is +0): 8 codes of 6 bits = 3 half-words
+                uint64_t bits = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    uint32_t ca = 0, cb = 0;
+                    if (!zero_tile) {
+                        const float a = fminf(fabsf(bf16_lo(w[j])) * sc.s, Fmt<FMT_E2M3>::fmax), b = fminf(fabsf(bf16_hi(w[j])) * sc.s, Fmt<FMT_E2M3>::fmax);
+                        fp6_mag_codes<FMT_E2M3>(a, b, ca, cb);
+                        if (ca) ca |= (w[j] >> 10) & 0x20u;
+                        if (cb) cb |= (w[j] >> 26) & 0x20u;
+                    } else {
+                        ca = (w[j] >> 10) & 0x20u;           // (a zero tile is copied: its zeros keep their signs)
+                        cb = (w[j] >> 26) & 0x20u;
+                    }
+                    bits |= (uint64_t)(ca | (cb << 6)) << (12 * j);
+                }
+                uint16_t* d = reinterpret_cast<uint16_t*>(tile + r * 96 + cc * 6);
+                d[0] = (uint16_t)bits; d[1] = (uint16_t)(bits >> 16); d[2] = (uint16_t)(bits >> 32);
+            }
+        }
+        return;
     }
     if (tid == 0) {
         if (meta && meta_val >= 0) meta[bid] = meta_val;

@@ -17,18 +17,13 @@
 #include <stdint.h>
 #include <algorithm>
 
-#include "mor_device.h"
+#include "mor_wirefmt.h"
 #include "mor_host.h"
 #include "../../include/mor_hip.h"
 
 namespace mor {
 
 constexpr int WWG = 256;
-
-template <int F> struct Wire {
-    static constexpr int bits = Fmt<F>::hw ? 8 : 6;
-    static constexpr int bias = (F == FMT_E4M3) ? 7 : (F == FMT_E5M2) ? 15 : (F == FMT_E3M2) ? 3 : 1;
-};
 
 // Exponent of the block scale, limited to the finite E8M0 range.  The integer form needs a normal amax; the
 // division covers subnormal amax and the far ends of the exponent range.
@@ -40,35 +35,15 @@ template <int F> __device__ __forceinline__ int wire_e8(float amax) {
     return min(max(e8, -127), 127);
 }
 
-// value of a 5-bit magnitude code of F
-template <int F> __device__ __forceinline__ float fp6_value(uint32_t mag) {
-    constexpr int mb = Fmt<F>::mbits, bias = Wire<F>::bias;
-    const uint32_t e = mag >> mb, m = mag & ((1u << mb) - 1u);
-    const float sub = (float)m * (1.0f / (float)(1 << (mb + bias - 1)));
-    const float normal = u2f(((e + 127u - bias) << 23) | (m << (23 - mb)));
-    return e == 0 ? sub : normal;
-}
-
-// codes of the two elements of a packed word, in bits 0..bits-1 and bits..2*bits-1.
-// FP6 through the FP8 converts: E2M3 / E3M2 have the mantissa width of E4M3 / E5M2, so for a scaled magnitude a in
-// the normal range of the 6-bit format the 8-bit code differs from the 6-bit one by the bias difference only; below
-// that range the 6-bit grid is uniform (step = its subnormal step), which is the 8-bit grid of the binade
-// [norm_min, 2 norm_min): convert a + norm_min instead (the sum is exact whenever the rounding can depend on it).
+// codes of the two elements of a packed word, in bits 0..bits-1 and bits..2*bits-1 (FP6: fp6_mag_codes).
 template <int F> __device__ __forceinline__ uint32_t code_pair(uint32_t w, int e8) {
     if constexpr (Fmt<F>::hw) {
         return hw_pack2<F>(ldexpf(bf16_lo(w), e8), ldexpf(bf16_hi(w), e8)) & 0xFFFFu;
     } else {
-        constexpr int F8 = (F == FMT_E2M3) ? FMT_E4M3 : FMT_E5M2;
-        constexpr int mb = Fmt<F>::mbits;
-        constexpr float norm_min = (F == FMT_E2M3) ? 1.0f : 0.25f;
-        constexpr uint32_t off_normal = (uint32_t)(Wire<F8>::bias - Wire<F>::bias) << mb;
-        constexpr uint32_t off_sub = (uint32_t)(1 - Wire<F>::bias + Wire<F8>::bias) << mb;
         // (in a block scaled by its own e8 nothing exceeds fmax; the clamp is the cast's saturation for any other use)
         const float a = fminf(ldexpf(fabsf(bf16_lo(w)), e8), Fmt<F>::fmax), b = fminf(ldexpf(fabsf(bf16_hi(w)), e8), Fmt<F>::fmax);
-        const bool na = a >= norm_min, nb = b >= norm_min;
-        const uint32_t p = hw_pack2<F8>(na ? a : a + norm_min, nb ? b : b + norm_min);
-        const uint32_t ca = (p & 0xFFu) - (na ? off_normal : off_sub);
-        const uint32_t cb = ((p >> 8) & 0xFFu) - (nb ? off_normal : off_sub);
+        uint32_t ca, cb;
+        fp6_mag_codes<F>(a, b, ca, cb);
         return ca | ((w >> 10) & 0x20u) | ((cb | ((w >> 26) & 0x20u)) << 6);
     }
 }

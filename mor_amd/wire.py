@@ -107,3 +107,37 @@ def fake_quantize_tiles_dual(x: Tensor, clamp_threshold: float = 0.0, mode: int 
         _cabi.check(_L.mor_fake_quantize_dual_tiles(x.data_ptr(), out.data_ptr(), meta.data_ptr(), out_t.data_ptr(), meta_t.data_ptr(),
                                                     rows, cols, float(clamp_threshold), mode, sf_type, _stream(x)))
     return out, meta, out_t, meta_t
+
+
+TILE_PAYLOAD_BYTES = 32768     # MOR_TILE_PAYLOAD_BYTES
+TILE_STORED_BF16 = 0x100       # MOR_TILE_STORED_BF16
+
+
+def quantize_mor_tiles(x: Tensor, clamp_threshold: float = 0.0, mode: int = 1) -> Tuple[Tensor, Tensor, Tensor]:
+    """The MoR decision of mor.ops.fake_quantize(x, rows, cols, 128, 128, clamp_threshold, mode, 1) with each tile's
+    codes as the result: (payload uint8 [tiles_y, tiles_x, 32768], tags int32 [tiles_y, tiles_x], scales float32
+    [tiles_y, tiles_x]).  A tile's slot holds 128 packed rows of 128 (E4M3 / E5M2), 96 (E2M3) or 256 (BF16) bytes."""
+    rows, cols = _check(x, 128)
+    x = x.contiguous()
+    gy, gx = rows // 128, cols // 128
+    with torch.cuda.device(x.device):
+        payload = torch.empty((gy, gx, TILE_PAYLOAD_BYTES), dtype=torch.uint8, device=x.device)
+        tags = torch.empty((gy, gx), dtype=torch.int32, device=x.device)
+        scales = torch.empty((gy, gx), dtype=torch.float32, device=x.device)
+        _cabi.check(_L.mor_mor_quantize(x.data_ptr(), payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), rows, cols,
+                                        float(clamp_threshold), mode, _stream(x)))
+    return payload, tags, scales
+
+
+def dequantize_mor_tiles(payload: Tensor, tags: Tensor, scales: Tensor) -> Tensor:
+    """(payload, tags, scales) of quantize_mor_tiles -> the bf16 tensor mor.ops.fake_quantize returns for the input."""
+    if (payload.dtype != torch.uint8 or tags.dtype != torch.int32 or scales.dtype != torch.float32 or not payload.is_cuda
+            or tags.dim() != 2 or scales.shape != tags.shape or payload.numel() != tags.numel() * TILE_PAYLOAD_BYTES):
+        raise RuntimeError("mor: expected (uint8 payload, int32 tags, float32 scales) of one tile grid on the GPU")
+    payload, tags, scales = payload.contiguous(), tags.contiguous(), scales.contiguous()
+    rows, cols = tags.shape[0] * 128, tags.shape[1] * 128
+    with torch.cuda.device(payload.device):
+        out = torch.empty((rows, cols), dtype=torch.bfloat16, device=payload.device)
+        _cabi.check(_L.mor_mor_dequantize(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, cols,
+                                          _stream(payload)))
+    return out

@@ -1,0 +1,169 @@
+"""mor_mor_quantize / mor_mor_dequantize (MoR per 128 x 128 tile, codes + tag + fp32 scale): the tags are the oracle's
+meta values, the decoded tensor is the oracle's fake-quantized output, and the payload is decoded a second time on the
+host from the documented layout alone (float8 views, a table for E2M3, an IEEE division, a round-half-up bf16 store)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mor_oracle as O
+from test_gpu_dual_tiles import mixture
+
+pytestmark = pytest.mark.gpu
+
+TILE_BYTES = 32768
+STORED_BF16 = 0x100
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    assert torch.cuda.is_available()
+    return gpu_util
+
+
+def quantize(G, a, clamp, mode):
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    rows, cols = a.shape
+    gy, gx = rows // 128, cols // 128
+    x = G.to_dev_u16(a)
+    payload = torch.full((gy, gx, TILE_BYTES), 0xA5, dtype=torch.uint8, device=G.dev())
+    tags = torch.full((gy, gx), -7, dtype=torch.int32, device=G.dev())
+    scales = torch.full((gy, gx), -7.0, dtype=torch.float32, device=G.dev())
+    _cabi.check(L.mor_mor_quantize(x.data_ptr(), payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), rows, cols, float(clamp), mode,
+                                   G.stream_ptr()))
+    torch.cuda.synchronize()
+    return payload, tags, scales
+
+
+def dequantize(G, payload, tags, scales):
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    rows, cols = tags.shape[0] * 128, tags.shape[1] * 128
+    out = torch.full((rows, cols), 7.0, dtype=torch.bfloat16, device=G.dev())
+    _cabi.check(L.mor_mor_dequantize(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, cols, G.stream_ptr()))
+    torch.cuda.synchronize()
+    return G.to_host_u16(out)
+
+
+E2M3_VALUES = np.array([m / 8.0 for m in range(8)] + [(1 + m / 8.0) * 2.0 ** (e - 1) for e in range(1, 4) for m in range(8)], dtype=np.float32)
+
+
+def host_decode_tile(slot, tag, scale):
+    """one payload slot (uint8[32768]) -> uint16[128, 128] bf16 bits, from the documented layout"""
+    if tag & STORED_BF16 or tag == 3:
+        return slot[:128 * 256].view(np.uint16).reshape(128, 128).copy()
+    if tag in (1, 11, 2, 12):
+        codes = slot[:128 * 128].reshape(128, 128)
+        dt = torch.float8_e4m3fn if tag in (1, 11) else torch.float8_e5m2
+        mag = torch.from_numpy((codes & 0x7F).copy()).view(dt).to(torch.float32).numpy()
+        sign = (codes >> 7).astype(np.uint16)
+    else:
+        assert tag == 4, tag
+        b = slot[:128 * 96].reshape(128, 32, 3).astype(np.uint32)
+        w = b[..., 0] | (b[..., 1] << 8) | (b[..., 2] << 16)                      # 4 codes per 3 bytes, code k at bits 6k
+        codes = np.stack([(w >> (6 * k)) & 0x3F for k in range(4)], axis=-1).reshape(128, 128)
+        mag = E2M3_VALUES[codes & 0x1F]
+        sign = (codes >> 5).astype(np.uint16)
+    q = (mag / np.float32(scale)).astype(np.float32)                               # IEEE division
+    bits = ((q.view(np.uint32).astype(np.uint64) + 0x8000) >> 16).astype(np.uint16)  # bf16, half rounded up
+    return bits | (sign << 15)
+
+
+def tile_amax(a, by, bx):
+    t = a[by * 128:(by + 1) * 128, bx * 128:(bx + 1) * 128]
+    return (t & 0x7FFF).max()
+
+
+def bf16_bits_to_f32(b):
+    return np.array([int(b) << 16], dtype=np.uint32).view(np.float32)[0]
+
+
+@pytest.mark.parametrize("shape", [(128, 128), (256, 384), (1024, 512), (2048, 2048)])
+@pytest.mark.parametrize("mode", [1, 101])
+def test_tags_round_trip_and_host_decode(G, shape, mode):
+    rows, cols = shape
+    rng = np.random.default_rng(rows * 5 + cols + mode)
+    a = mixture(rng, rows, cols)
+    if rows > 128:
+        a[133, 7] = 0x7FC0              # a NaN and an infinity in tiles of their own
+        a[9, 131] = 0xFF80
+    clamp = 1e-3
+    print("mor wire", shape, mode, flush=True)
+    payload, tags, scales = quantize(G, a, clamp, mode)
+    got = dequantize(G, payload, tags, scales)
+    want, wmeta = O.fake_quantize(a, 128, 128, clamp, mode, 1)
+    t, s, p = tags.cpu().numpy(), scales.cpu().numpy(), payload.cpu().numpy()
+    assert np.array_equal(t & 0xFF, wmeta.reshape(t.shape)), "tags differ from the oracle's meta"
+    assert np.array_equal(got, want), "decoded tensor differs from the oracle's output"
+    seen = set()
+    for by in range(rows // 128):
+        for bx in range(cols // 128):
+            tag, amax_bits = int(t[by, bx]), int(tile_amax(a, by, bx))
+            amax = bf16_bits_to_f32(amax_bits)
+            # tiles stored as bf16 images: those with a NaN, and those whose scale 448 / amax leaves 2^-90 .. 2^90
+            with np.errstate(divide="ignore", over="ignore"):
+                s4 = np.float32(448.0) / amax if amax_bits <= 0x7F80 and amax_bits != 0 else np.float32(1.0)
+            s4_bits = int(np.array([s4], dtype=np.float32).view(np.uint32)[0])
+            expo = ((s4_bits >> 23) & 0xFF) - 127
+            outside = amax_bits > 0x7F80 or (amax_bits != 0 and (not (-90 <= expo <= 90) or s4_bits & 0x7FFFFF == 0x7FFFFF))
+            assert bool(tag & STORED_BF16) == bool(outside), (by, bx, tag, amax_bits)
+            fmax = {1: 448.0, 11: 448.0, 2: 57344.0, 12: 57344.0, 4: 7.5}.get(tag)
+            if fmax is not None and amax_bits != 0:
+                assert s[by, bx] == np.float32(fmax) / amax, (by, bx, tag, s[by, bx])
+            else:
+                assert s[by, bx] == 1.0, (by, bx, tag, s[by, bx])
+            dec = host_decode_tile(p[by, bx], tag, s[by, bx])
+            assert np.array_equal(dec, want[by * 128:(by + 1) * 128, bx * 128:(bx + 1) * 128]), ("host decode", by, bx, tag)
+            seen.add(tag)
+    if rows * cols >= 2048 * 2048:
+        assert len({x & 0xFF for x in seen}) >= 4 and any(x & STORED_BF16 for x in seen), seen
+
+
+def test_slot_bytes_beyond_the_tile_are_left_alone(G):
+    rng = np.random.default_rng(3)
+    a = mixture(rng, 512, 512)
+    payload, tags, scales = quantize(G, a, 1e-3, 1)
+    p, t = payload.cpu().numpy(), tags.cpu().numpy()
+    for by in range(4):
+        for bx in range(4):
+            tag = int(t[by, bx])
+            used = 128 * (256 if (tag & STORED_BF16 or tag == 3) else 96 if tag == 4 else 128)
+            assert (p[by, bx, used:] == 0xA5).all(), (by, bx, tag)
+
+
+def test_large_tensor_round_trip_equals_fake_quantize(G):
+    """8192 x 8192 (band order, streaming loads and stores): decode(encode(x)) is mor_fake_quantize's output, the tags its meta"""
+    import mor_amd
+    rows, cols = 8192, 8192
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn(rows, cols, device="cuda", generator=g)
+    x[:, :2048] *= torch.exp(3 * torch.randn(rows, 2048, device="cuda", generator=g))
+    x[:, 2048:3072] = 1.0 + 0.3 * torch.rand(rows, 1024, device="cuda", generator=g)
+    x[:1024, 4096:] *= 1e-34
+    x = x.to(torch.bfloat16)
+    for mode in (1, 101):
+        payload, tags, scales = mor_amd.wire.quantize_mor_tiles(x, 1e-15, mode)
+        back = mor_amd.wire.dequantize_mor_tiles(payload, tags, scales)
+        ref, rmeta = mor_amd.ops.fake_quantize(x, rows, cols, 128, 128, 1e-15, mode, 1)
+        assert torch.equal(tags & 0xFF, rmeta.view(tags.shape))
+        assert torch.equal(back.view(torch.int16), ref.view(torch.int16))
+        kinds = set((tags & 0xFF).unique().tolist())
+        assert len(kinds) >= 3 and bool((tags & STORED_BF16).any()), kinds
+
+
+def test_rejects_what_it_cannot_do(G):
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    x = torch.zeros((128, 256), dtype=torch.bfloat16, device=G.dev())
+    p = torch.zeros(2 * TILE_BYTES, dtype=torch.uint8, device=G.dev())
+    t = torch.zeros(2, dtype=torch.int32, device=G.dev())
+    s = torch.zeros(2, dtype=torch.float32, device=G.dev())
+    q = lambda r, c, mode, a=x, b=p: L.mor_mor_quantize(a.data_ptr(), b.data_ptr(), t.data_ptr(), s.data_ptr(), r, c, 0.0, mode, G.stream_ptr())
+    assert q(128, 200, 1) != 0 and b"multiples of 128" in L.mor_last_error()
+    assert q(128, 256, 2) != 0 and b"mode" in L.mor_last_error()
+    assert q(128, 256, 1, x, x) != 0 and b"different" in L.mor_last_error()
+    assert L.mor_mor_quantize(x.data_ptr(), p.data_ptr(), 0, s.data_ptr(), 128, 256, 0.0, 1, G.stream_ptr()) != 0
+    assert L.mor_mor_dequantize(p.data_ptr(), t.data_ptr(), s.data_ptr(), x.data_ptr(), 100, 256, G.stream_ptr()) != 0
+    assert q(128, 256, 1) == 0
+    torch.cuda.synchronize()
