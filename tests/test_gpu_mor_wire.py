@@ -49,22 +49,25 @@ def dequantize(G, payload, tags, scales):
 E2M3_VALUES = np.array([m / 8.0 for m in range(8)] + [(1 + m / 8.0) * 2.0 ** (e - 1) for e in range(1, 4) for m in range(8)], dtype=np.float32)
 
 
-def host_decode_tile(slot, tag, scale):
-    """one payload slot (uint8[32768]) -> uint16[128, 128] bf16 bits, from the documented layout"""
-    if tag & STORED_BF16 or tag == 3:
-        return slot[:128 * 256].view(np.uint16).reshape(128, 128).copy()
+def host_code_values(slot, tag):
+    """one payload slot of an FP8 / FP6 tile -> (magnitudes float32 [128, 128], sign bits uint16 [128, 128])"""
     if tag in (1, 11, 2, 12):
         codes = slot[:128 * 128].reshape(128, 128)
         dt = torch.float8_e4m3fn if tag in (1, 11) else torch.float8_e5m2
         mag = torch.from_numpy((codes & 0x7F).copy()).view(dt).to(torch.float32).numpy()
-        sign = (codes >> 7).astype(np.uint16)
-    else:
-        assert tag == 4, tag
-        b = slot[:128 * 96].reshape(128, 32, 3).astype(np.uint32)
-        w = b[..., 0] | (b[..., 1] << 8) | (b[..., 2] << 16)                      # 4 codes per 3 bytes, code k at bits 6k
-        codes = np.stack([(w >> (6 * k)) & 0x3F for k in range(4)], axis=-1).reshape(128, 128)
-        mag = E2M3_VALUES[codes & 0x1F]
-        sign = (codes >> 5).astype(np.uint16)
+        return mag, (codes >> 7).astype(np.uint16)
+    assert tag == 4, tag
+    b = slot[:128 * 96].reshape(128, 32, 3).astype(np.uint32)
+    w = b[..., 0] | (b[..., 1] << 8) | (b[..., 2] << 16)                      # 4 codes per 3 bytes, code k at bits 6k
+    codes = np.stack([(w >> (6 * k)) & 0x3F for k in range(4)], axis=-1).reshape(128, 128)
+    return E2M3_VALUES[codes & 0x1F], (codes >> 5).astype(np.uint16)
+
+
+def host_decode_tile(slot, tag, scale):
+    """one payload slot (uint8[32768]) -> uint16[128, 128] bf16 bits, from the documented layout"""
+    if tag & STORED_BF16 or tag == 3:
+        return slot[:128 * 256].view(np.uint16).reshape(128, 128).copy()
+    mag, sign = host_code_values(slot, tag)
     q = (mag / np.float32(scale)).astype(np.float32)                               # IEEE division
     bits = ((q.view(np.uint32).astype(np.uint64) + 0x8000) >> 16).astype(np.uint16)  # bf16, half rounded up
     return bits | (sign << 15)
@@ -167,3 +170,40 @@ def test_rejects_what_it_cannot_do(G):
     assert L.mor_mor_dequantize(p.data_ptr(), t.data_ptr(), s.data_ptr(), x.data_ptr(), 100, 256, G.stream_ptr()) != 0
     assert q(128, 256, 1) == 0
     torch.cuda.synchronize()
+
+
+def test_matrix_instruction_consumes_tile_rows(G):
+    """Rows of a tile's payload are operands of the gfx950 scaled matrix instruction as they lie in the slot (128 code
+    bytes per row for E4M3 / E5M2, 96 for E2M3: the row layout of the MX payload): 16 rows of one tile times 16 rows of
+    another with unit block scales, divided by the two tile scales, is the product of the decoded rows."""
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((128, 768)).astype(np.float32)
+    x[:, 128:256] *= 37.0                                                          # another scale, E4M3 as well
+    x[:, 256:384] = 1.0 + 0.3 * rng.random((128, 128))                             # E2M3
+    x[:, 384:512] = -(2.0 + 0.5 * rng.random((128, 128)))                          # E2M3
+    x[:, 512:768] = np.exp2(rng.uniform(-12.0, 8.0, (128, 256))) * rng.choice([-1.0, 1.0], (128, 256))   # range 2^20: E5M2 by the dynamic-range rule
+    a = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16).copy()
+    payload, tags, scales = quantize(G, a, 1e-3, 101)
+    t, s, p = tags.cpu().numpy()[0], scales.cpu().numpy()[0], payload.cpu().numpy()[0]
+    print("tile tags", t, flush=True)
+    assert t[0] in (1, 11) and t[1] in (1, 11) and t[2] == 4 and t[3] == 4 and t[4] in (2, 12) and t[5] in (2, 12), t
+    unit = torch.full((16, 4), 127, dtype=torch.uint8, device=G.dev())             # E8M0 bytes of 2^0
+    for ta, tb, fmt in ((0, 1, 0), (4, 5, 1), (2, 3, 3)):
+        out = torch.zeros((16, 16), dtype=torch.float32, device=G.dev())
+        pa, pb = payload[0, ta], payload[0, tb]                                     # rows 0..15 of each slot
+        _cabi.check(L.mor_selftest_mx_mfma(pa.data_ptr(), unit.data_ptr(), pb.data_ptr(), unit.data_ptr(), fmt, out.data_ptr(), G.stream_ptr()))
+        torch.cuda.synchronize()
+        got = out.cpu().double().numpy() / (float(s[ta]) * float(s[tb]))
+        rows = []
+        for k in (ta, tb):                                                          # value(code) / scale, from the documented layout
+            mag, sign = host_code_values(p[k], int(t[k]))
+            rows.append((mag[:16].astype(np.float64) * np.where(sign[:16] != 0, -1.0, 1.0)) / float(s[k]))
+        want = rows[0] @ rows[1].T
+        bound = np.abs(rows[0]) @ np.abs(rows[1]).T
+        excess = np.max(np.abs(got - want) / bound)
+        print(f"tile rows through the matrix instruction, format {fmt}: max |difference| / sum of magnitudes {excess:.3e}", flush=True)
+        # the instruction aligns the 128 products of a row to the largest before it adds them: 1e-5 of the sum of magnitudes
+        # for the narrow tiles, 1.3e-4 for the E5M2 rows whose products span 2^40; a wrong layout is wrong by the sum itself
+        assert excess <= (5e-4 if fmt == 1 else 2e-5), (fmt, excess)
