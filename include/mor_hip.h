@@ -272,7 +272,8 @@ MOR_API int mor_fake_quantize_dual_tiles(const void* input, void* output, int32_
  *          values mor_fake_quantize writes for the tile.  The rest of a tile's slot is not written.
  * mor_mor_dequantize gives the output of that mor_fake_quantize call bit for bit: value of the code,
  * divided by the scale (IEEE), rounded to bf16 half-up (FQ:312-316).
- * mode % 10 must be 1, mode / 100 as in mor_fake_quantize; default flavour, fp32 scales.
+ * mode % 10: 1 (MoR), or 2 / 3: every tile E4M3 / E5M2 with its own fp32 scale (block scaling in 128 x 128
+ * tiles: tags 1 / 2); mode / 100 as in mor_fake_quantize; default flavour, fp32 scales.
  * rows and cols multiples of 128; tensor and payload 16-byte aligned, different buffers.
  */
 #define MOR_TILE_PAYLOAD_BYTES 32768

@@ -1,4 +1,4 @@
-// mor_mor_quantize / mor_mor_dequantize: the MoR decision per 128 x 128 tile with the tile's codes as the result
+// mor_mor_quantize / mor_mor_dequantize: the MoR decision (or a forced FP8 format) per 128 x 128 tile with the tile's codes as the result
 // (format tag + fp32 scale + payload) instead of the fake-quantized bf16 values, and the way back.
 // The encoder is k_wgblock in its WIRE form (same passes 1 and 2, codes stored in pass 3); the decoder below repeats
 // the second half of the bf16 kernel's pass 3 (code -> value, division by the scale, bf16 store), so that
@@ -107,8 +107,8 @@ extern "C" int mor_mor_quantize(const void* input, void* payload, int32_t* tags,
                                 double clamp_threshold, int64_t mode, void* stream) {
     if (int rc = check_tiles(input, payload, tags, scales, rows, cols)) return rc;
     QuantArgs qa;
-    if (!mor_decode_mode(mode, clamp_threshold, qa) || qa.qmode != 1)
-        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mode %% 10 must be 1 (MoR), got %lld", (long long)mode);
+    if (!mor_decode_mode(mode, clamp_threshold, qa) || qa.qmode == 4)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "mode %% 10 must be 1 (MoR), 2 (E4M3) or 3 (E5M2), got %lld", (long long)mode);
     const Shape sh = make_shape(rows, cols, 128, 128);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t nblocks = sh.gy * sh.gx;
@@ -120,9 +120,12 @@ extern "C" int mor_mor_quantize(const void* input, void* payload, int32_t* tags,
     const size_t dl = nblocks >= 4096 ? 36000 : 0;
     const uint4* in = static_cast<const uint4*>(input);
     uint4* out = static_cast<uint4*>(payload);
+    const bool mor = qa.qmode == 1;
     for_slices(nblocks, [&](int64_t first, int count) {
-        if (stream_loads) k_wgblock<true, false, 8, true, 1, WG, false, false, true><<<count, WG, dl, st>>>(in, out, tags, scales, sh, qa, 16, shift, first, nullptr, nullptr);
-        else k_wgblock<true, false, 8, true, 0, WG, false, false, true><<<count, WG, dl, st>>>(in, out, tags, scales, sh, qa, 16, shift, first, nullptr, nullptr);
+#define MOR_TILE_CODES(MOR_, NT_) k_wgblock<MOR_, false, 8, true, NT_, WG, false, false, true><<<count, WG, dl, st>>>(in, out, tags, scales, sh, qa, 16, shift, first, nullptr, nullptr)
+        if (mor) { if (stream_loads) MOR_TILE_CODES(true, 1); else MOR_TILE_CODES(true, 0); }
+        else { if (stream_loads) MOR_TILE_CODES(false, 1); else MOR_TILE_CODES(false, 0); }
+#undef MOR_TILE_CODES
     });
     return mor_check_launch("k_wgblock (tile codes)");
 }

@@ -27,7 +27,7 @@ template <class V> __device__ __forceinline__ void dual_tile_put(uint32_t* s_t, 
     const uint4 p = (R & 1) ? make_uint4(q.z, q.w, q.x, q.y) : make_uint4(q.x, q.y, q.z, q.w);
     *reinterpret_cast<uint4*>(s_t + r * 64 + ((cc ^ (R >> 1)) << 2)) = p;
 }
-// WIRE (whole 128 x 128 tiles, 256 threads, MoR, fp32 scale): instead of the fake-quantized bf16 tile the kernel writes
+// WIRE (whole 128 x 128 tiles, 256 threads, fp32 scale; MoR or a forced format): instead of the fake-quantized bf16 tile the kernel writes
 // the tile's codes: `out` is the payload, MOR_TILE_PAYLOAD_BYTES (32768) per tile, tile after tile in block order, rows
 // packed (128 rows of 128 one-byte codes, of 96 bytes of 6-bit codes, or of 256 bytes of bf16); `meta` takes the
 // storage format of each tile and `stats` one float per tile, its scale.  A tile whose scale is outside the fast range
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
                                                  float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift,
                                                  int64_t first, uint4* out_t, int32_t* __restrict__ meta_t) {
     static_assert(!DUAL || (FULL && NV == 8 && WGS == 256 && !GATHER), "DUAL: whole 128 x 128 tiles");
-    static_assert(!WIRE || (MOR && !E8 && FULL && NV == 8 && WGS == 256 && !GATHER && !DUAL), "WIRE: MoR on whole 128 x 128 tiles, fp32 scale");
+    static_assert(!WIRE || (!E8 && FULL && NV == 8 && WGS == 256 && !GATHER && !DUAL), "WIRE: whole 128 x 128 tiles, fp32 scale");
     constexpr int NW = WGS / 64;
     __shared__ __attribute__((aligned(16))) uint32_t s_t[DUAL ? 128 * 64 : 4];
     __shared__ float s_f[2][NW];

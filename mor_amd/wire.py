@@ -116,7 +116,8 @@ TILE_STORED_BF16 = 0x100       # MOR_TILE_STORED_BF16
 def quantize_mor_tiles(x: Tensor, clamp_threshold: float = 0.0, mode: int = 1) -> Tuple[Tensor, Tensor, Tensor]:
     """The MoR decision of mor.ops.fake_quantize(x, rows, cols, 128, 128, clamp_threshold, mode, 1) with each tile's
     codes as the result: (payload uint8 [tiles_y, tiles_x, 32768], tags int32 [tiles_y, tiles_x], scales float32
-    [tiles_y, tiles_x]).  A tile's slot holds 128 packed rows of 128 (E4M3 / E5M2), 96 (E2M3) or 256 (BF16) bytes."""
+    [tiles_y, tiles_x]).  A tile's slot holds 128 packed rows of 128 (E4M3 / E5M2), 96 (E2M3) or 256 (BF16) bytes.
+    mode % 10: 1 = MoR, 2 / 3 = every tile E4M3 / E5M2 with its own fp32 scale."""
     rows, cols = _check(x, 128)
     x = x.contiguous()
     gy, gx = rows // 128, cols // 128

@@ -1,4 +1,4 @@
-"""mor_mor_quantize / mor_mor_dequantize (MoR per 128 x 128 tile, codes + tag + fp32 scale): the tags are the oracle's
+"""mor_mor_quantize / mor_mor_dequantize (MoR or a forced FP8 format per 128 x 128 tile, codes + tag + fp32 scale): the tags are the oracle's
 meta values, the decoded tensor is the oracle's fake-quantized output, and the payload is decoded a second time on the
 host from the documented layout alone (float8 views, a table for E2M3, an IEEE division, a round-half-up bf16 store)."""
 import numpy as np
@@ -83,7 +83,7 @@ def bf16_bits_to_f32(b):
 
 
 @pytest.mark.parametrize("shape", [(128, 128), (256, 384), (1024, 512), (2048, 2048)])
-@pytest.mark.parametrize("mode", [1, 101])
+@pytest.mark.parametrize("mode", [1, 101, 2, 3])
 def test_tags_round_trip_and_host_decode(G, shape, mode):
     rows, cols = shape
     rng = np.random.default_rng(rows * 5 + cols + mode)
@@ -119,7 +119,7 @@ def test_tags_round_trip_and_host_decode(G, shape, mode):
             dec = host_decode_tile(p[by, bx], tag, s[by, bx])
             assert np.array_equal(dec, want[by * 128:(by + 1) * 128, bx * 128:(bx + 1) * 128]), ("host decode", by, bx, tag)
             seen.add(tag)
-    if rows * cols >= 2048 * 2048:
+    if rows * cols >= 2048 * 2048 and mode % 10 == 1:
         assert len({x & 0xFF for x in seen}) >= 4 and any(x & STORED_BF16 for x in seen), seen
 
 
@@ -145,14 +145,14 @@ def test_large_tensor_round_trip_equals_fake_quantize(G):
     x[:, 2048:3072] = 1.0 + 0.3 * torch.rand(rows, 1024, device="cuda", generator=g)
     x[:1024, 4096:] *= 1e-34
     x = x.to(torch.bfloat16)
-    for mode in (1, 101):
+    for mode in (1, 101, 2):
         payload, tags, scales = mor_amd.wire.quantize_mor_tiles(x, 1e-15, mode)
         back = mor_amd.wire.dequantize_mor_tiles(payload, tags, scales)
         ref, rmeta = mor_amd.ops.fake_quantize(x, rows, cols, 128, 128, 1e-15, mode, 1)
         assert torch.equal(tags & 0xFF, rmeta.view(tags.shape))
         assert torch.equal(back.view(torch.int16), ref.view(torch.int16))
         kinds = set((tags & 0xFF).unique().tolist())
-        assert len(kinds) >= 3 and bool((tags & STORED_BF16).any()), kinds
+        assert (len(kinds) >= 3 or mode == 2) and bool((tags & STORED_BF16).any()), kinds
 
 
 def test_rejects_what_it_cannot_do(G):
@@ -164,7 +164,7 @@ def test_rejects_what_it_cannot_do(G):
     s = torch.zeros(2, dtype=torch.float32, device=G.dev())
     q = lambda r, c, mode, a=x, b=p: L.mor_mor_quantize(a.data_ptr(), b.data_ptr(), t.data_ptr(), s.data_ptr(), r, c, 0.0, mode, G.stream_ptr())
     assert q(128, 200, 1) != 0 and b"multiples of 128" in L.mor_last_error()
-    assert q(128, 256, 2) != 0 and b"mode" in L.mor_last_error()
+    assert q(128, 256, 4) != 0 and b"mode" in L.mor_last_error()
     assert q(128, 256, 1, x, x) != 0 and b"different" in L.mor_last_error()
     assert L.mor_mor_quantize(x.data_ptr(), p.data_ptr(), 0, s.data_ptr(), 128, 256, 0.0, 1, G.stream_ptr()) != 0
     assert L.mor_mor_dequantize(p.data_ptr(), t.data_ptr(), s.data_ptr(), x.data_ptr(), 100, 256, G.stream_ptr()) != 0
