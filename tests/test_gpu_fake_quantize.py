@@ -120,6 +120,13 @@ SHAPES = [
     (5, 28672, 1, 28672),             # ... one long row per block
     (3, 131072, 1, 131072),
     (131, 2056, 129, 2048),           # ... an odd row count per block
+    # blocks 128 columns wide on rows that do not start on 16-byte boundaries
+    (259, 383, 128, 128),             # odd width: every shift 0 .. 7, last block column 127 wide, last block row 3 rows
+    (140, 644, 128, 128),             # rows 8-byte aligned (shifts 0 and 4), last block column 4 wide
+    (70, 1026, 64, 128),              # rows 4-byte aligned, 4 vectors per lane, last block column 2 wide
+    (40, 301, 16, 128),               # one vector per lane, last block column 45 wide (a partial vector in the middle of the row)
+    (33, 129, 1, 128),                # one-row blocks, last block column 1 wide
+    (129, 127, 128, 128),             # a tensor narrower than the block
 ]
 
 
@@ -267,3 +274,33 @@ def test_nan_and_inf_elements_stay_inside_their_block(G, br, bc, mode, sf):
     mask = np.repeat(np.repeat(clean, br, 0), bc, 1)
     assert np.array_equal(out[mask], want[mask])
     assert np.array_equal(meta[clean], wmeta[clean])
+
+
+@pytest.mark.parametrize("offset", [1, 3, 4, 7])
+@pytest.mark.parametrize("inplace", [False, True])
+def test_tensor_that_does_not_start_on_a_vector_boundary(G, offset, inplace):
+    """A tensor `offset` elements into an allocation (128-wide blocks, column count a multiple of 8): input and output
+    rows start `offset` elements past 16-byte boundaries; what lies before and after the tensor stays as it was."""
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    rows, cols = 150, 264
+    a = data_gen.c2_student_t(rows, cols, seed=90 + offset)
+    a[3, 5] = 0x7FC0                                           # a NaN: its block takes the exact path
+    pad = 24
+    buf = torch.full((offset + rows * cols + pad,), 3.0, dtype=torch.bfloat16, device=G.dev())
+    x = buf[offset:offset + rows * cols]
+    x.copy_(G.to_dev_u16(a).flatten())
+    obuf = buf if inplace else torch.full_like(buf, 5.0)
+    o = obuf[offset:offset + rows * cols]
+    meta = torch.full((2, 3), -7, dtype=torch.int32, device=G.dev())
+    for mode in (1, 2):
+        if inplace:
+            x.copy_(G.to_dev_u16(a).flatten())
+        print("offset tensor", offset, inplace, mode, flush=True)
+        _cabi.check(L.mor_fake_quantize(x.data_ptr(), o.data_ptr(), meta.data_ptr(), rows, cols, 128, 128, 1e-15, mode, 1, 0, G.stream_ptr()))
+        torch.cuda.synchronize()
+        want, wmeta = O.fake_quantize(a, 128, 128, 1e-15, mode, 1)
+        assert np.array_equal(meta.cpu().numpy(), wmeta)
+        assert_same(G.to_host_u16(o).reshape(rows, cols), want, f"offset {offset} mode {mode}")
+        fill = 3.0 if inplace else 5.0
+        assert bool((obuf[:offset] == fill).all()) and bool((obuf[offset + rows * cols:] == fill).all()), "wrote outside the tensor"
