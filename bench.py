@@ -377,6 +377,25 @@ def other_configs(torch, run, cabi, K, W):
         ms, wall = time_launches(torch, plan.run, 200, 20)
         res["tiny_1x32"][key] = round(ms * 1e3 / 100, 3)
         res["tiny_1x32"][key.replace("_us_", "_wall_us_")] = round(wall * 1e3 / 100, 3)
+    # the seven weight matrices of a Llama-3-8B layer (q, k, v, o, gate, up, down: 872 MB of traffic) in one call: their
+    # 128 x 128 tiles run as grids of one tile kernel (tensors of one streaming class share a launch)
+    wshapes = [(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096), (4096, 14336)]
+    gw = torch.Generator(device="cuda").manual_seed(1005)
+    wx = [(torch.randn(r, c, device="cuda", generator=gw) * 0.02).to(torch.bfloat16) for r, c in wshapes]
+    wo = [torch.empty_like(t) for t in wx]
+    wm = [torch.empty((r // 128, c // 128), dtype=torch.int32, device="cuda") for r, c in wshapes]
+    wbytes = sum(t.numel() for t in wx) * 4
+    res["llama3_8b_weights_one_call"] = {"bytes": wbytes}
+    for mode, key in ((1, "mor_128x128"), (2, "block_e4m3_128x128")):
+        plan = BatchPlan(wx, wo, wm, [(128, 128)] * 7, 1e-15, mode, 1)
+        ms, wall = time_launches(torch, plan.run, 60, 200)
+        one = 0.0
+        for t, o, m in zip(wx, wo, wm):
+            ms1, _ = time_launches(torch, lambda: run.fake_quantize(t, o, m, 128, 128, 1e-15, mode, 1), 100, 300)
+            one += ms1
+        res["llama3_8b_weights_one_call"][key] = {"ms": round(ms, 5), "GBps": round(wbytes / (ms * 1e-3) / 1e9, 1), "frac": round(wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                                  "seven_calls_ms": round(one, 5)}
+    del wx, wo
     # the same call through the operator layer a user of the reference calls (allocations of out and meta included)
     import mor
     xg = xs.clone().requires_grad_(True)

@@ -34,10 +34,13 @@ template <class V> __device__ __forceinline__ void dual_tile_put(uint32_t* s_t, 
 // (or that holds a NaN) is stored as the bf16 image of its fake-quantized values, its format ORed with TILE_STORED_BF16.
 constexpr int TILE_PAYLOAD_BYTES = 32768;
 constexpr int TILE_STORED_BF16 = 0x100;
+// The work of one workgroup on block `bid` (k_wgblock below is its kernel; the batch entry runs it on the blocks of
+// several tensors in one launch).  cpr_shift: log2 of the chunk count per block row, negative when that is not a power
+// of two.
 template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false, bool DUAL = false, bool WIRE = false>
-__global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
-                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift,
-                                                 int64_t first, uint4* out_t, int32_t* __restrict__ meta_t) {
+__device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_t* __restrict__ meta, float* __restrict__ stats,
+                                             const Shape& sh, const QuantArgs& qa, int cpr, int cpr_shift, uint32_t bid,
+                                             uint4* out_t, int32_t* __restrict__ meta_t) {
     static_assert(!DUAL || (FULL && NV == 8 && WGS == 256 && !GATHER), "DUAL: whole 128 x 128 tiles");
     static_assert(!WIRE || (!E8 && FULL && NV == 8 && WGS == 256 && !GATHER && !DUAL), "WIRE: whole 128 x 128 tiles, fp32 scale");
     constexpr int NW = WGS / 64;
@@ -46,14 +49,6 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     __shared__ uint32_t s_u[NW];
     __shared__ float s_e[2][NW];           // the error sums have slots of their own: no barrier between pass 1's readers and pass 2's writers
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // Workgroup -> block.  cpr_shift bit 8 (large tensors whose block grid is a multiple of 8 wide): consecutive
-    // workgroup ids go round the 8 XCDs, and each XCD takes a band of gx / 8 block columns, walking it row by row.
-    uint32_t bid = (uint32_t)(first + blockIdx.x);       // (a launch holds a slice of the blocks, see for_slices; fewer than 2^31 blocks)
-    if (cpr_shift >= 256) {            // (a negative cpr_shift means a chunk count per row that is not a power of two)
-        bid = band_order(sh, bid);
-        cpr_shift &= 255;
-        if (cpr_shift == 255) cpr_shift = -1;
-    }
     uint32_t by32, bx32;
     block_of(sh, bid, by32, bx32);
     const int64_t by = by32, bx = bx32;
@@ -348,6 +343,21 @@ __global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, in
     };
     pass3();
     write_transposed(meta_val);
+}
+
+template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false, bool DUAL = false, bool WIRE = false>
+__global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
+                                                 float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift,
+                                                 int64_t first, uint4* out_t, int32_t* __restrict__ meta_t) {
+    // Workgroup -> block.  cpr_shift bit 8 (large tensors whose block grid is a multiple of 8 wide): consecutive
+    // workgroup ids go round the 8 XCDs, and each XCD takes a band of gx / 8 block columns, walking it row by row.
+    uint32_t bid = (uint32_t)(first + blockIdx.x);       // (a launch holds a slice of the blocks, see for_slices; fewer than 2^31 blocks)
+    if (cpr_shift >= 256) {            // (a negative cpr_shift means a chunk count per row that is not a power of two)
+        bid = band_order(sh, bid);
+        cpr_shift &= 255;
+        if (cpr_shift == 255) cpr_shift = -1;
+    }
+    wgblock_body<MOR, E8, NV, FULL, NT, WGS, GATHER, DUAL, WIRE>(in, out, meta, stats, sh, qa, cpr, cpr_shift, bid, out_t, meta_t);
 }
 
 

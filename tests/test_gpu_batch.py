@@ -139,3 +139,34 @@ def test_a_bad_descriptor_stops_the_call_before_any_launch(G):
     assert b"block dims" in L.mor_last_error()
     torch.cuda.synchronize()
     assert (m.cpu().numpy() == -7).all() and float(y.float().abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("mode,sf", [(1, 1), (1, 2), (101, 1), (2, 1), (2, 2), (3, 1)])
+@pytest.mark.parametrize("inplace", [False, True])
+def test_tensors_in_whole_tiles_share_launches(G, mode, sf, inplace):
+    """Tensors in whole 128 x 128 tiles beyond the small-tensor limit: their tiles run as one grid of the tile kernel
+    (several streaming classes, grids with and without the band order, a tensor that is not in whole tiles and a small
+    one in between); every tensor must come out as the oracle gives it."""
+    rng = np.random.default_rng(1300 + mode * 3 + sf)
+    shapes = [(512, 1024), (1024, 256), (2048, 1024), (640, 896), (4096, 1024), (384, 768), (1000, 520), (128, 128),
+              (1024, 2048), (2304, 2176)]
+    arrays = [bits(rng, r, c, i % 3) for i, (r, c) in enumerate(shapes)]
+    arrays[2][:128, :128] = 0                                      # a zero tile
+    arrays[4][130, 5] = 0x7FC0                                     # a NaN: its tile takes the exact path
+    arrays[0][:128, 128:256] = bits(rng, 128, 128, 0) & 0x807F     # a tile of tiny values: scale outside the fast range
+    blocks = [(128, 128)] * len(shapes)
+    got = run_batch(G, arrays, blocks, 1e-3, mode, sf, inplace=inplace)
+    check_against_oracle(arrays, blocks, 1e-3, mode, sf, got)
+
+
+def test_fifty_tile_tensors_take_two_launches(G):
+    """more tensors than one launch of the tile kernel holds (48), every one as from a call of its own"""
+    rng = np.random.default_rng(77)
+    shapes = [(512, 640)] * 25 + [(768, 512)] * 25
+    arrays = [bits(rng, r, c, i % 3) for i, (r, c) in enumerate(shapes)]
+    blocks = [(128, 128)] * len(shapes)
+    got = run_batch(G, arrays, blocks, 1e-3, 1, 1)
+    singles = [G.fake_quantize(a, 128, 128, 1e-3, 1, 1) for a in arrays]
+    for i, ((out, meta), (want, wmeta)) in enumerate(zip(got, singles)):
+        assert np.array_equal(meta, wmeta) and np.array_equal(out, want), i
+    check_against_oracle(arrays[:4], blocks[:4], 1e-3, 1, 1, got[:4])
