@@ -156,3 +156,41 @@ def test_wire_sweep(G, case):
             w, _ = O.fake_quantize(a, 1, 32, 0.0, mode, sf)
             wt, _ = O.fake_quantize(np.ascontiguousarray(a.T), 1, 32, 0.0, mode, sf)
             assert np.array_equal(o, w) and np.array_equal(ot, wt), (case, sf)
+
+
+def tile_cases():
+    rng = np.random.default_rng(20257)
+    return [(i, 128 * int(rng.integers(1, 7)), 128 * int(rng.integers(1, 9)), int(rng.choice([1, 101, 2, 3])), int(rng.integers(4)))
+            for i in range(24)]
+
+
+@pytest.mark.parametrize("case", tile_cases(), ids=lambda c: "tiles%d_%dx%d_m%d_k%d" % c)
+def test_tile_entries_sweep(G, case):
+    """128 x 128 tiles through the three entries that work on them besides mor_fake_quantize: the tile codes and their
+    decode, both orientations from one read, and a batch call; all against the oracle."""
+    import mor_amd
+    from test_gpu_batch import run_batch
+    i, rows, cols, mode, kind = case
+    rng = np.random.default_rng(5000 + i)
+    a = make_data(rng, rows, cols, kind)
+    if kind == 2:
+        a[:128, :128] = (a[:128, :128] & 0x8000) | 0x0080 | (a[:128, :128] & 0x007F)        # a tile of values near 2^-126: scale outside the fast range
+    print("sweep", case, flush=True)
+    clamp = 1e-3
+    want, wmeta = O.fake_quantize(a, 128, 128, clamp, mode, 1)
+    x = G.to_dev_u16(a)
+    payload, tags, scales = mor_amd.wire.quantize_mor_tiles(x, clamp, mode)
+    back = mor_amd.wire.dequantize_mor_tiles(payload, tags, scales)
+    assert np.array_equal((tags & 0xFF).cpu().numpy(), wmeta), case
+    assert np.array_equal(G.to_host_u16(back), want), case
+    out, meta, out_t, meta_t = mor_amd.wire.fake_quantize_tiles_dual(x, clamp, mode, 1)
+    want_t, wmeta_t = O.fake_quantize(np.ascontiguousarray(a.T), 128, 128, clamp, mode, 1)
+    assert np.array_equal(meta.cpu().numpy(), wmeta) and np.array_equal(G.to_host_u16(out), want), case
+    assert np.array_equal(meta_t.cpu().numpy(), wmeta_t) and np.array_equal(G.to_host_u16(out_t), want_t), case
+    # the same tensor three times in a batch (large enough for the tile path when rows * cols > 2^18), next to a small one
+    small = make_data(rng, 64, 96, kind)
+    got = run_batch(G, [a, small, a, a], [(128, 128), (16, 32), (128, 128), (128, 128)], clamp, mode, 1)
+    for k in (0, 2, 3):
+        assert np.array_equal(got[k][1], wmeta) and np.array_equal(got[k][0], want), (case, k)
+    ws, wsm = O.fake_quantize(small, 16, 32, clamp, mode, 1)
+    assert np.array_equal(got[1][1], wsm) and np.array_equal(got[1][0], ws), case
