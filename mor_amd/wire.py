@@ -118,7 +118,11 @@ def quantize_mor_tiles(x: Tensor, clamp_threshold: float = 0.0, mode: int = 1) -
     codes as the result: (payload uint8 [tiles_y, tiles_x, 32768], tags int32 [tiles_y, tiles_x], scales float32
     [tiles_y, tiles_x]).  A tile's slot holds 128 packed rows of 128 (E4M3 / E5M2), 96 (E2M3) or 256 (BF16) bytes.
     mode % 10: 1 = MoR, 2 / 3 = every tile E4M3 / E5M2 with its own fp32 scale."""
-    rows, cols = _check(x, 128)
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_cuda:
+        raise RuntimeError("mor: expected a 2-D bfloat16 GPU tensor")
+    rows, cols = x.shape
+    if rows % 128 or cols % 128:
+        raise RuntimeError(f"mor: tile codes need rows and cols that are multiples of 128, got {tuple(x.shape)}")
     x = x.contiguous()
     gy, gx = rows // 128, cols // 128
     with torch.cuda.device(x.device):

@@ -62,3 +62,16 @@ def test_batch_entry_rejects_bad_arguments_without_a_gpu():
     assert L.mor_fake_quantize_batch(d, 1, 0, None) != 0
     assert b"positive" in L.mor_last_error()
     assert C.sizeof(TensorDesc) == 80
+
+
+def test_tile_code_entries_reject_bad_arguments_without_a_gpu():
+    """argument checks of mor_mor_quantize / mor_mor_dequantize run before any device call"""
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    assert L.mor_mor_quantize(256, 512, 768, 1024, 128, 200, 0.0, 1, None) == -1 and b"multiples of 128" in L.mor_last_error()
+    assert L.mor_mor_quantize(256, 512, 768, 1024, 128, 256, 0.0, 4, None) == -1 and b"mode" in L.mor_last_error()
+    assert L.mor_mor_quantize(256, 256, 768, 1024, 128, 256, 0.0, 1, None) == -1 and b"different" in L.mor_last_error()
+    assert L.mor_mor_quantize(256, 520, 768, 1024, 128, 256, 0.0, 1, None) == -1 and b"aligned" in L.mor_last_error()
+    assert L.mor_mor_quantize(256, 512, None, 1024, 128, 256, 0.0, 1, None) == -1
+    assert L.mor_mor_dequantize(512, 768, 1024, 256, 100, 256, None) == -1
+    assert L.mor_mor_dequantize(512, None, 1024, 256, 128, 256, None) == -1
