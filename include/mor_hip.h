@@ -83,8 +83,10 @@ MOR_API int mor_fake_quantize(const void* input, void* output, int32_t* meta,
  * call (FQ:1839-1871; the reference's callers loop over their tensors, one launch each), and the
  * result of every tensor is bit for bit that call's.  descs is host memory, read before the call
  * returns.  Tensors of up to 2^18 elements share launches, 56 to a launch, one workgroup per block;
- * larger ones in whole 128 x 128 tiles (MoR or a forced format, default flavour, 16-byte aligned)
- * share launches of the tile kernel, 48 to a launch; the rest are forwarded to mor_fake_quantize.
+ * larger ones in whole blocks of 2048, 4096, 8192 or 16384 elements (128 x 128 tiles, rows of 4096
+ * elements, ...; a forced format, or MoR on blocks of 16384 elements; default flavour, 16-byte
+ * aligned) share launches of the kernel that holds a block in registers, 48 tensors to a launch; the
+ * rest are forwarded to mor_fake_quantize.
  * Every descriptor is validated before anything is launched; no device memory is allocated.
  */
 typedef struct MorTensorDesc {

@@ -79,47 +79,49 @@ __global__ __launch_bounds__(WG) void k_batch(BatchArgs a, int fast_ok) {
     else elementwise_block<EMU>(it, sh, qa, bid);
 }
 
-// Tensors in whole 128 x 128 tiles (MoR or a forced format) that are too large for the records above: the tiles of up
-// to 48 such tensors as one grid of the register-resident tile kernel (wgblock_body), so that a tensor of a few MiB does
-// not pay a launch of its own and the tail of one tensor's grid overlaps the head of the next.  A tensor's workgroups
-// start at a multiple of 8 (the XCD band order counts on workgroup id mod 8); the padding workgroups leave at once.
-constexpr int TILE_BATCH_MAX = 48;
-struct TileItem {                                    // 72 bytes
+// Tensors that are too large for the records above and whose blocks a workgroup holds in registers: whole blocks of
+// 2048 x NV elements, NV = 1, 2, 4 or 8 (128 x 128 tiles, rows of 4096 elements, ...), MoR for NV = 8 or a forced
+// format.  The blocks of up to 48 such tensors run as one grid of the register-resident block kernel (wgblock_body), so
+// that a tensor of a few MiB does not pay a launch of its own and the tail of one tensor's grid overlaps the head of the
+// next.  A tensor's workgroups start at a multiple of 8 (the XCD band order counts on workgroup id mod 8); the padding
+// workgroups leave at once.
+constexpr int BLOCK_BATCH_MAX = 48;
+struct BlockItem {                                   // 80 bytes
     const uint4* in;
     uint4* out;
     int32_t* meta;
-    int32_t rows, cols;
+    int32_t rows, cols, brows, bcols;
     DivU32 d_gx, d_band;
     float clamp;
     int8_t qmode, fmt, meta_val, dyn_range;
-    int8_t band, pad[7];
+    int8_t band, shift, pad[6];                      // shift: log2 of the chunks per block row (20 for one-row blocks: row 0 always)
 };
-static_assert(sizeof(TileItem) == 72, "record size");
-struct TileArgs {
+static_assert(sizeof(BlockItem) == 80, "record size");
+struct BlockArgs {
     int n;
-    uint32_t first[TILE_BATCH_MAX + 1];
-    TileItem item[TILE_BATCH_MAX];
+    uint32_t first[BLOCK_BATCH_MAX + 1];
+    BlockItem item[BLOCK_BATCH_MAX];
 };
-static_assert(sizeof(TileArgs) <= 4096 - 16, "kernel argument size");
+static_assert(sizeof(BlockArgs) <= 4096 - 16, "kernel argument size");
 
-template <bool MOR, bool E8, int NT>
-__global__ __launch_bounds__(WG) void k_batch_tiles(TileArgs a) {
+template <bool MOR, bool E8, int NV, int NT>
+__global__ __launch_bounds__(WG) void k_batch_blocks(BlockArgs a) {
     int lo = 0, hi = a.n - 1;
     while (lo < hi) {
         const int mid = (lo + hi + 1) >> 1;
         if (blockIdx.x >= a.first[mid]) lo = mid; else hi = mid - 1;
     }
-    const TileItem& it = a.item[lo];
+    const BlockItem& it = a.item[lo];
     const uint32_t local = blockIdx.x - a.first[lo];
     Shape sh{};
-    sh.rows = it.rows; sh.cols = it.cols; sh.brows = 128; sh.bcols = 128;
-    sh.gy = it.rows >> 7; sh.gx = it.cols >> 7;
+    sh.rows = it.rows; sh.cols = it.cols; sh.brows = it.brows; sh.bcols = it.bcols;
+    sh.gx = it.d_gx.d; sh.gy = it.rows / it.brows;
     sh.d_gx = it.d_gx; sh.d_band = it.d_band;
     if (local >= (uint32_t)(sh.gy * sh.gx)) return;                  // padding up to the next multiple of 8
     QuantArgs qa{};
     qa.qmode = it.qmode; qa.fmt = it.fmt; qa.meta_val = it.meta_val; qa.dyn_range = it.dyn_range; qa.clamp = it.clamp;
     const uint32_t bid = it.band ? band_order(sh, local) : local;
-    wgblock_body<MOR, E8, 8, true, NT>(it.in, it.out, it.meta, nullptr, sh, qa, 16, 4, bid, nullptr, nullptr);
+    wgblock_body<MOR, E8, NV, true, NT>(it.in, it.out, it.meta, nullptr, sh, qa, it.bcols >> 3, it.shift, bid, nullptr, nullptr);
 }
 
 }  // namespace mor
@@ -127,15 +129,26 @@ __global__ __launch_bounds__(WG) void k_batch_tiles(TileArgs a) {
 using namespace mor;
 
 // streaming class of a tensor's loads and stores, as launch_wgblock_nv chooses it
-static int tile_nt_class(int64_t bytes) { return bytes >= ((int64_t)64 << 20) ? 1 : bytes >= ((int64_t)4 << 20) ? 2 : 0; }
+static int block_nt_class(int64_t bytes) { return bytes >= ((int64_t)64 << 20) ? 1 : bytes >= ((int64_t)4 << 20) ? 2 : 0; }
 
-template <bool MOR, bool E8>
-static void launch_batch_tiles(const TileArgs& a, int nt, hipStream_t st) {
+template <bool MOR, bool E8, int NV>
+static void launch_batch_blocks_nv(const BlockArgs& a, int nt, hipStream_t st) {
     const uint32_t grid = a.first[a.n];
-    const size_t dyn_lds = grid >= 4096 ? 53000 : 0;                 // three workgroups per CU on large grids (launch_wgblock_nv)
-    if (nt == 1) k_batch_tiles<MOR, E8, 1><<<grid, WG, dyn_lds, st>>>(a);
-    else if (nt == 2) k_batch_tiles<MOR, E8, 2><<<grid, WG, dyn_lds, st>>>(a);
-    else k_batch_tiles<MOR, E8, 0><<<grid, WG, dyn_lds, st>>>(a);
+    const size_t dyn_lds = (NV == 8 && grid >= 4096) ? 53000 : 0;    // three workgroups per CU on large grids (launch_wgblock_nv)
+    if (nt == 1) k_batch_blocks<MOR, E8, NV, 1><<<grid, WG, dyn_lds, st>>>(a);
+    else if (nt == 2) k_batch_blocks<MOR, E8, NV, 2><<<grid, WG, dyn_lds, st>>>(a);
+    else k_batch_blocks<MOR, E8, NV, 0><<<grid, WG, dyn_lds, st>>>(a);
+}
+// (MoR only with NV = 8: the caller sends other MoR tensors to mor_fake_quantize)
+template <bool E8>
+static void launch_batch_blocks(const BlockArgs& a, bool mor, int nv, int nt, hipStream_t st) {
+    if (mor) { launch_batch_blocks_nv<true, E8, 8>(a, nt, st); return; }
+    switch (nv) {
+        case 1: launch_batch_blocks_nv<false, E8, 1>(a, nt, st); break;
+        case 2: launch_batch_blocks_nv<false, E8, 2>(a, nt, st); break;
+        case 4: launch_batch_blocks_nv<false, E8, 4>(a, nt, st); break;
+        default: launch_batch_blocks_nv<false, E8, 8>(a, nt, st); break;
+    }
 }
 
 extern "C" int mor_fake_quantize_batch(const MorTensorDesc* descs, int64_t n, uint32_t flags, void* stream) {
@@ -149,15 +162,16 @@ extern "C" int mor_fake_quantize_batch(const MorTensorDesc* descs, int64_t n, ui
         if (int rc = mor_validate_shape(d.input, d.rows, d.cols, d.block_rows, d.block_cols)) return rc;
         if (!d.output || !d.meta) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output / meta of tensor %lld is NULL", (long long)i);
     }
-    // tensors in whole 128 x 128 tiles share launches of the tile kernel (same mode class, scale type and streaming class)
-    TileArgs ta{};
-    int ta_mor = 0, ta_e8 = 0, ta_nt = 0;
-    auto flush_tiles = [&]() -> int {
+    // tensors in whole register-resident blocks share launches of the block kernel (same mode class, scale type, block
+    // size class and streaming class)
+    BlockArgs ta{};
+    int ta_mor = 0, ta_e8 = 0, ta_nv = 0, ta_nt = 0;
+    auto flush_blocks = [&]() -> int {
         if (ta.n == 0) return MOR_OK;
-        if (ta_mor) { if (ta_e8) launch_batch_tiles<true, true>(ta, ta_nt, st); else launch_batch_tiles<true, false>(ta, ta_nt, st); }
-        else { if (ta_e8) launch_batch_tiles<false, true>(ta, ta_nt, st); else launch_batch_tiles<false, false>(ta, ta_nt, st); }
+        if (ta_e8) launch_batch_blocks<true>(ta, ta_mor != 0, ta_nv, ta_nt, st);
+        else launch_batch_blocks<false>(ta, ta_mor != 0, ta_nv, ta_nt, st);
         ta.n = 0;
-        return mor_check_launch("k_batch_tiles");
+        return mor_check_launch("k_batch_blocks");
     };
     BatchArgs a{};
     auto flush = [&]() -> int {
@@ -172,30 +186,37 @@ extern "C" int mor_fake_quantize_batch(const MorTensorDesc* descs, int64_t n, ui
         const int64_t nblocks = cdiv(d.rows, d.block_rows) * cdiv(d.cols, d.block_cols);
         if (d.rows * d.cols > BATCH_SMALL || nblocks > (1 << 16)) {
             QuantArgs tq;
-            const bool tiles = fast_ok && d.block_rows == 128 && d.block_cols == 128 && d.rows % 128 == 0 && d.cols % 128 == 0
-                               && nblocks <= (1 << 20) && d.rows * (d.cols / 8) < 0x7FFFFFFFll
-                               && ((reinterpret_cast<uintptr_t>(d.input) | reinterpret_cast<uintptr_t>(d.output)) & 15u) == 0
-                               && (d.sf_type == 1 || d.sf_type == 2) && mor_decode_mode(d.mode, d.clamp_threshold, tq) && tq.qmode != 4;
-            if (tiles) {
-                const int is_mor = tq.qmode == 1, is_e8 = d.sf_type == 2, nt = tile_nt_class(d.rows * d.cols * 2);
-                if (ta.n && (is_mor != ta_mor || is_e8 != ta_e8 || nt != ta_nt || ta.n == TILE_BATCH_MAX
+            const int64_t nch = (d.block_cols % 8 == 0) ? d.block_rows * (d.block_cols / 8) : 0;     // 16-byte chunks per block
+            const int64_t cpr = d.block_cols / 8;
+            bool blocks = fast_ok && (nch == WG || nch == 2 * WG || nch == 4 * WG || nch == 8 * WG)
+                          && d.rows % d.block_rows == 0 && d.cols % d.block_cols == 0 && (d.block_rows == 1 || is_pow2(cpr))
+                          && nblocks <= (1 << 20) && d.block_rows * (d.cols / 8) < 0x7FFFFFFFll
+                          && ((reinterpret_cast<uintptr_t>(d.input) | reinterpret_cast<uintptr_t>(d.output)) & 15u) == 0
+                          && (d.sf_type == 1 || d.sf_type == 2) && mor_decode_mode(d.mode, d.clamp_threshold, tq) && tq.qmode != 4;
+            if (blocks && tq.qmode == 1 && nch != 8 * WG) blocks = false;
+            if (blocks) {
+                const int is_mor = tq.qmode == 1, is_e8 = d.sf_type == 2, nv = (int)(nch / WG), nt = block_nt_class(d.rows * d.cols * 2);
+                if (ta.n && (is_mor != ta_mor || is_e8 != ta_e8 || nv != ta_nv || nt != ta_nt || ta.n == BLOCK_BATCH_MAX
                              || (uint64_t)ta.first[ta.n] + (uint64_t)nblocks + 8 > (1u << 22))) {
-                    if (int rc = flush_tiles()) return rc;
+                    if (int rc = flush_blocks()) return rc;
                 }
-                ta_mor = is_mor; ta_e8 = is_e8; ta_nt = nt;
-                TileItem& it = ta.item[ta.n];
-                it = TileItem{};
+                ta_mor = is_mor; ta_e8 = is_e8; ta_nv = nv; ta_nt = nt;
+                BlockItem& it = ta.item[ta.n];
+                it = BlockItem{};
                 it.in = static_cast<const uint4*>(d.input);
                 it.out = static_cast<uint4*>(d.output);
                 it.meta = d.meta;
                 it.rows = (int32_t)d.rows;
                 it.cols = (int32_t)d.cols;
-                const int64_t gx = d.cols / 128;
+                it.brows = (int32_t)d.block_rows;
+                it.bcols = (int32_t)d.block_cols;
+                const int64_t gx = d.cols / d.block_cols;
                 it.d_gx = make_div((uint32_t)gx);
                 it.d_band = make_div((uint32_t)std::max<int64_t>(gx >> 3, 1));
                 it.clamp = tq.clamp;
                 it.qmode = (int8_t)tq.qmode; it.fmt = (int8_t)tq.fmt; it.meta_val = (int8_t)tq.meta_val; it.dyn_range = (int8_t)tq.dyn_range;
                 it.band = (nblocks >= 2048 && gx % 8 == 0 && nblocks % 8 == 0) ? 1 : 0;
+                it.shift = (int8_t)(d.block_rows == 1 ? 20 : ilog2((int)cpr));
                 ta.first[ta.n + 1] = ta.first[ta.n] + (uint32_t)((nblocks + 7) & ~(int64_t)7);
                 ++ta.n;
                 continue;
@@ -223,6 +244,6 @@ extern "C" int mor_fake_quantize_batch(const MorTensorDesc* descs, int64_t n, ui
         a.first[a.n + 1] = a.first[a.n] + (uint32_t)nblocks;
         if (++a.n == BATCH_MAX) { if (int rc = flush()) return rc; }
     }
-    if (int rc = flush_tiles()) return rc;
+    if (int rc = flush_blocks()) return rc;
     return flush();
 }

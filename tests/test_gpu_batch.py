@@ -170,3 +170,20 @@ def test_fifty_tile_tensors_take_two_launches(G):
     for i, ((out, meta), (want, wmeta)) in enumerate(zip(got, singles)):
         assert np.array_equal(meta, wmeta) and np.array_equal(out, want), i
     check_against_oracle(arrays[:4], blocks[:4], 1e-3, 1, 1, got[:4])
+
+
+@pytest.mark.parametrize("mode,sf", [(2, 1), (3, 2), (1, 1), (101, 2)])
+def test_register_resident_blocks_of_every_size_share_launches(G, mode, sf):
+    """Tensors beyond the small-tensor limit in whole blocks of 2048, 4096, 8192 and 16384 elements (rows, tiles of
+    several shapes): a launch per size class, every tensor as the oracle gives it.  (MoR shares launches for blocks of
+    16384 elements only; the other MoR tensors go through calls of their own.)"""
+    rng = np.random.default_rng(1700 + mode * 3 + sf)
+    cases = [((512, 4096), (1, 4096)), ((1024, 2048), (1, 2048)), ((768, 4096), (1, 4096)), ((512, 1024), (64, 64)),
+             ((640, 768), (32, 64)), ((96, 16384), (1, 16384)), ((1024, 1024), (128, 128)), ((512, 2048), (64, 256)),
+             ((300, 8192), (1, 8192)), ((1024, 512), (256, 64)), ((2048, 4096), (1, 4096)), ((512, 1024), (128, 64))]
+    arrays = [bits(rng, r, c, i % 3) for i, ((r, c), _) in enumerate(cases)]
+    arrays[0][3] = 0                                               # a zero row
+    arrays[2][5, 7] = 0x7FC0                                       # a NaN
+    blocks = [b for _, b in cases]
+    got = run_batch(G, arrays, blocks, 1e-3, mode, sf)
+    check_against_oracle(arrays, blocks, 1e-3, mode, sf, got)
