@@ -102,6 +102,22 @@ template <int F> __device__ __forceinline__ uint4 fq_vec_div(uint4 v, float s, f
     return o;
 }
 
+// the same through a table of the block's 128 dequantized magnitudes (bf16 bits of code / s, in LDS): |x| * s, hardware
+// convert, two lookups, sign
+template <int F> __device__ __forceinline__ uint32_t fq_pair_tab(uint32_t w, float s, const uint16_t* tab, uint32_t& codes) {
+    codes = hw_pack2_low_keep<F>(fabsf(bf16_lo(w)) * s, fabsf(bf16_hi(w)) * s, codes);
+    const uint32_t qa = tab[codes & 0xFFu], qb = tab[(codes >> 8) & 0xFFu];
+    return qa | (qb << 16) | (w & 0x80008000u);
+}
+template <int F> __device__ __forceinline__ uint4 fq_vec_tab(uint4 v, float s, const uint16_t* tab, uint32_t& codes) {
+    uint4 o;
+    o.x = fq_pair_tab<F>(v.x, s, tab, codes);
+    o.y = fq_pair_tab<F>(v.y, s, tab, codes);
+    o.z = fq_pair_tab<F>(v.z, s, tab, codes);
+    o.w = fq_pair_tab<F>(v.w, s, tab, codes);
+    return o;
+}
+
 // The two error terms of one packed word (FQ:504-542) on magnitudes; s5 = 128 * s4 exactly.
 // The reference computes |q / x - 1| with q = c / s.  E8 scale: |q - x| * (1 / x), q - x exact.  FP32 scale:
 // with y = x * s the same quantity is |c - y| / y (c - y is exact: c is within a factor 2 of y, or 0), which needs

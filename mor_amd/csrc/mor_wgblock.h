@@ -48,6 +48,7 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
     __shared__ float s_f[2][NW];
     __shared__ uint32_t s_u[NW];
     __shared__ float s_e[2][NW];           // the error sums have slots of their own: no barrier between pass 1's readers and pass 2's writers
+    __shared__ uint16_t s_q[128];          // pass 3, fp32 scale: the dequantized bf16 value of every 7-bit magnitude code
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     uint32_t by32, bx32;
     block_of(sh, bid, by32, bx32);
@@ -307,14 +308,21 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
     }
     if constexpr (!E8) {
         if (fmt == FMT_E4M3 || fmt == FMT_E5M2) {
+            // An FP8 format has 127 magnitudes, a block one scale: code / scale, rounded to bf16, is computed once per
+            // code (a thread each) and looked up per element, which leaves a multiply, the convert and the sign per element.
             const float r4 = s4.r;                    // 1 / s5 = r4 / 128 exactly
+            if (tid < 128) {
+                const float c = (fmt == FMT_E4M3) ? hw_unpack2_low<FMT_E4M3>((uint32_t)tid).x : hw_unpack2_low<FMT_E5M2>((uint32_t)tid).x;
+                s_q[tid] = store_bf16<false>((fmt == FMT_E4M3) ? div_by_scale(c, s4.s, r4) : div_by_scale(c, s5.s, r4 * 0.0078125f));
+            }
+            __syncthreads();
             uint32_t codes = 0;                       // (the converts write half of this register: carried from word to word)
             if (fmt == FMT_E4M3) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_div<FMT_E4M3>(v[k], s4.s, r4, codes));
+                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_tab<FMT_E4M3>(v[k], s4.s, s_q, codes));
             } else {
 #pragma unroll
-                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_div<FMT_E5M2>(v[k], s5.s, r4 * 0.0078125f, codes));
+                for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_tab<FMT_E5M2>(v[k], s5.s, s_q, codes));
             }
             return;
         }
