@@ -265,7 +265,7 @@ def main():
                                f"{ROT} buffer pairs in rotation",
                    "arithmetic": "bf16 tensors, fp32 / integer arithmetic, gfx950 fp8 / fp6 converts",
                    "preheat": f"{preheat_steps} untimed steps ({args.preheat_ms:g} ms) before the {W} warmup steps: the first 15 ms of load after idle are "
-                              f"a transient of the MoR kernel (48 -> 57 -> 48 us per launch); the first 20 steps after idle took "
+                              f"a transient of the MoR kernel (up to a fifth slower between 2 and 8 ms); the first 20 steps after idle took "
                               f"{first_wall:.5f} ms each (per kernel: first_20_steps_after_idle), the timed steps are the sustained rate",
                    "elements_per_s": round(4 * nelem / (ms_per_step * 1e-3), 0), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": roofline,
