@@ -114,6 +114,16 @@ def test_c4_mor_16384x14336(G):
     st = G.mor_stats(a, 128, 128, 1e-15, 1, 1)
     assert np.array_equal(st[..., :2], stats[..., :2])
     np.testing.assert_allclose(st[..., 2:], stats[..., 2:], rtol=1e-6, atol=0)
+    # the same decisions and values through the tile codes and their decode, and through a batch call
+    import mor_amd
+    x = G.to_dev_u16(a)
+    payload, tags, scales = mor_amd.wire.quantize_mor_tiles(x, 1e-15, 1)
+    assert np.array_equal((tags & 0xFF).cpu().numpy(), wmeta), "C4 tile codes: tags"
+    same(G.to_host_u16(mor_amd.wire.dequantize_mor_tiles(payload, tags, scales)), want, "C4 tile codes decoded")
+    del payload
+    (bout, bmeta), = mor_amd.batch.fake_quantize_batch([x], [(128, 128)], 1e-15, 1, 1)
+    assert np.array_equal(bmeta.cpu().numpy(), wmeta), "C4 batch call: meta"
+    same(G.to_host_u16(bout), want, "C4 batch call")
 
 
 C5_SHAPES = [
