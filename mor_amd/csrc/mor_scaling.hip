@@ -512,16 +512,19 @@ __device__ __forceinline__ uint4 bs_cols_vec_exact(uint4 v, const Scale (&sc)[8]
 
 // pass 2 / pass 4 for column blocks N x 1 with aligned rows (the geometry of k_bs_amax_col): a thread owns 8 adjacent
 // columns over a segment of rows, so its 8 scales and their reciprocals are computed once.  Threads whose scales are
-// not all in the fast range use the exact arithmetic.
+// not all in the fast range use the exact arithmetic.  A workgroup is 2^cg_log column groups wide and 256 >> cg_log row
+// lanes deep (a tensor of fewer than 2048 columns still fills it); row lane l takes the rows l, l + lanes, ... of a segment.
 template <bool WRITE, bool ERR>
 __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_t* out, uint32_t* ws, const float* scales,
-                                                     Finish fin, int gate, int ss_mode, int npart1, Shape sh, int rows_per_wg) {
+                                                     Finish fin, int gate, int ss_mode, int npart1, Shape sh, int rows_per_wg,
+                                                     int cg_log) {
     __shared__ float s_f[2 * WAVES];
     __shared__ int s_i[WAVES];
     if (gate > 0 && finish_decision(fin, s_f, s_i) != gate) return;
     const float gamax = reduce_partial_amax(ws, npart1, s_f);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t col0 = ((int64_t)blockIdx.x * WG + threadIdx.x) * 8;
+    const int row_lane = (int)threadIdx.x >> cg_log, row_lanes = WG >> cg_log;
+    const int64_t col0 = (((int64_t)blockIdx.x << cg_log) + (threadIdx.x & ((1 << cg_log) - 1))) * 8;
     const int64_t segs_per_block = (sh.brows + rows_per_wg - 1) / rows_per_wg;
     const int64_t row_stride = sh.cols >> 3;
     const uint4* in4 = reinterpret_cast<const uint4*>(in);
@@ -540,24 +543,24 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_
             for (int j = 0; j < 8; ++j) { sc[j] = make_scale(block_scale(gamax, scales, sp + j, ss_mode)); fast = fast && sc[j].fast; }
             if (fast) {
 #pragma unroll 1
-                for (int64_t r = r_begin; r < r_end; r += 4) {
+                for (int64_t r = r_begin + row_lane; r < r_end; r += 4 * row_lanes) {
                     uint4 v[4];
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         v[k] = make_uint4(0, 0, 0, 0);
-                        if (r + k < r_end) v[k] = load16_rt(in4 + (r + k) * row_stride + (col0 >> 3), streams_last_read(sh.rows * sh.cols));
+                        if (r + k * row_lanes < r_end) v[k] = load16_rt(in4 + (r + k * row_lanes) * row_stride + (col0 >> 3), streams_last_read(sh.rows * sh.cols));
                     }
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         const uint4 q = bs_cols_vec_fast<WRITE, ERR>(v[k], sc, err);
                         if constexpr (WRITE) {
-                            if (r + k < r_end) store16_rt(out4 + (r + k) * row_stride + (col0 >> 3), q, nt);
+                            if (r + k * row_lanes < r_end) store16_rt(out4 + (r + k * row_lanes) * row_stride + (col0 >> 3), q, nt);
                         }
                     }
                 }
             } else {
 #pragma unroll 1
-                for (int64_t r = r_begin; r < r_end; ++r) {
+                for (int64_t r = r_begin + row_lane; r < r_end; r += row_lanes) {
                     const uint4 q = bs_cols_vec_exact(in4[r * row_stride + (col0 >> 3)], sc, err);
                     if constexpr (WRITE) out4[r * row_stride + (col0 >> 3)] = q;
                 }
@@ -1152,14 +1155,17 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
     // end: bf16 fallback (out of place: copy if meta == 3) or the quantized write (in place: only if meta == 1)
     const bool e8 = (ss_mode == 2);
     if (col && vec && !emu && !e8) {
-        const int rows_per_wg = (int)std::min<int64_t>(brows, 32);
-        const unsigned gx = (unsigned)cdiv(cdiv(cols, 8), WG);
+        // a workgroup is min(256, column groups) lanes wide (a power of two) and the rest of its threads deep: 32 rows per
+        // thread and segment (16384 x 1024: 128 lanes x 2 row lanes instead of half-empty workgroups, the op 41.5 -> 34.4 us)
+        const int cg_log = std::min(8, ilog2(cdiv(cols, 8)));
+        const int rows_per_wg = (int)std::min<int64_t>(brows, 32 * (WG >> cg_log));
+        const unsigned gx = (unsigned)cdiv(cdiv(cols, 8), (int64_t)1 << cg_log);
         const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
         const dim3 grid(gx, (unsigned)std::min<int64_t>(segs, std::max<int64_t>(PASS2_MAX / gx, 1)));
         fin.nerr = (int)(grid.x * grid.y);
-        if (inplace) k_bs_quant_col<false, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 0, (int)ss_mode, npart, sh, rows_per_wg);
-        else k_bs_quant_col<true, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 0, (int)ss_mode, npart, sh, rows_per_wg);
-        if (inplace) k_bs_quant_col<true, false><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 1, (int)ss_mode, npart, sh, rows_per_wg);
+        if (inplace) k_bs_quant_col<false, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 0, (int)ss_mode, npart, sh, rows_per_wg, cg_log);
+        else k_bs_quant_col<true, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 0, (int)ss_mode, npart, sh, rows_per_wg, cg_log);
+        if (inplace) k_bs_quant_col<true, false><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 1, (int)ss_mode, npart, sh, rows_per_wg, cg_log);
     } else {
         const bool vec2 = vec && (col || bcols % 8 == 0) && n / 8 < 0xFFFFFFFFll;
         const int64_t work = vec2 ? n / 8 : n;
