@@ -97,10 +97,12 @@ __global__ __launch_bounds__(WG) void k_fill_i32(int32_t* p, int64_t n, int32_t 
 }
 
 // bf16 copy (mode 7 and the unused mode digits, FQ:1831-1833): 16-byte vectors and a scalar tail
+// (meta: the blocks' entries, all 3, written by the same launch; may be NULL)
 template <int EW_NV>
-__global__ __launch_bounds__(WG) void k_copy(const uint16_t* in, uint16_t* out, int64_t n, int64_t nvec) {
+__global__ __launch_bounds__(WG) void k_copy(const uint16_t* in, uint16_t* out, int64_t n, int64_t nvec, int32_t* meta, int64_t nblocks) {
     const int64_t stride = (int64_t)gridDim.x * WG;
     const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
+    if (meta) for (int64_t i = gtid; i < nblocks; i += stride) meta[i] = 3;
     const uint4* in4 = reinterpret_cast<const uint4*>(in);
     uint4* out4 = reinterpret_cast<uint4*>(out);
     const int64_t base = (int64_t)blockIdx.x * (EW_NV * WG) + threadIdx.x;
@@ -516,10 +518,12 @@ extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
             const uint16_t* i16 = static_cast<const uint16_t*>(input);
             uint16_t* o16 = static_cast<uint16_t*>(output);
             // (from HBM one vector per lane copies fastest, as in k_rowgroup)
-            if (nvec >= ((int64_t)4 << 20)) k_copy<1><<<(int)cdiv(nvec, (int64_t)WG), WG, 0, st>>>(i16, o16, n, nvec);
-            else k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(i16, o16, n, nvec);
+            // (the meta entries leave with the same launch: a launch of their own costs 2 us of the 45 at 8192^2)
+            if (nvec >= ((int64_t)4 << 20)) k_copy<1><<<(int)cdiv(nvec, (int64_t)WG), WG, 0, st>>>(i16, o16, n, nvec, meta, nblocks);
+            else k_copy<2><<<nvec > 0 ? (int)cdiv(nvec, 2ll * WG) : grid_for(n, 16), WG, 0, st>>>(i16, o16, n, nvec, meta, nblocks);
+        } else {
+            k_fill_i32<<<grid_for(nblocks), WG, 0, st>>>(meta, nblocks, 3);
         }
-        k_fill_i32<<<grid_for(nblocks), WG, 0, st>>>(meta, nblocks, 3);
         return mor_check_launch("k_copy / k_fill_i32");
     }
     return run_quantize(input, output, meta, nullptr, rows, cols, brows, bcols, qa, e8, flags, st);
