@@ -187,3 +187,16 @@ def test_register_resident_blocks_of_every_size_share_launches(G, mode, sf):
     blocks = [b for _, b in cases]
     got = run_batch(G, arrays, blocks, 1e-3, mode, sf)
     check_against_oracle(arrays, blocks, 1e-3, mode, sf, got)
+
+
+@pytest.mark.parametrize("flags,flavour", [(1, "EMU"), (2, "KERNEL")])
+def test_other_flavours_do_not_take_the_shared_launches(G, flags, flavour):
+    """With the torch-emulation flavour or the software casts, large tensors in whole tiles are forwarded to calls of
+    their own (the shared launches run the default arithmetic only); the results are the flavour's."""
+    rng = np.random.default_rng(2100 + flags)
+    shapes = [(1024, 1024), (512, 640), (64, 64)]
+    arrays = [bits(rng, r, c, i % 3) for i, (r, c) in enumerate(shapes)]
+    blocks = [(128, 128), (128, 128), (16, 32)]
+    for mode, sf in ((1, 1), (2, 2)):
+        got = run_batch(G, arrays, blocks, 1e-3, mode, sf, flags=flags)
+        check_against_oracle(arrays, blocks, 1e-3, mode, sf, got, flavour=getattr(O, flavour))
