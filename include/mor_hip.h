@@ -271,7 +271,8 @@ MOR_API int mor_fake_quantize_dual_tiles(const void* input, void* output, int32_
  *          holds its 128 rows packed: E4M3 / E5M2 128 bytes per row (one code per element: the
  *          OCP code of |x| * scale, the sign of x in bit 7); E2M3 96 bytes per row (6-bit codes,
  *          dense little-endian, code k at bits 6k; a zero result has no sign, as the reference's
- *          software cast gives +0); BF16 (and MOR_TILE_STORED_BF16) 256 bytes per row: the bf16
+ *          software cast gives +0 -- except in an all-zero tile, which the reference copies: its
+ *          zeros keep their signs); BF16 (and MOR_TILE_STORED_BF16) 256 bytes per row: the bf16
  *          values mor_fake_quantize writes for the tile.  The rest of a tile's slot is not written.
  * mor_mor_dequantize gives the output of that mor_fake_quantize call bit for bit: value of the code,
  * divided by the scale (IEEE), rounded to bf16 half-up (FQ:312-316).

@@ -1,5 +1,5 @@
-// mor_mor_quantize / mor_mor_dequantize: the MoR decision (or a forced FP8 format) per 128 x 128 tile with the tile's codes as the result
-// (format tag + fp32 scale + payload) instead of the fake-quantized bf16 values, and the way back.
+// mor_mor_quantize / mor_mor_dequantize: the MoR decision (or a forced FP8 format) per 128 x 128 tile with the tile's
+// codes as the result (format tag + fp32 scale + payload) instead of the fake-quantized bf16 values, and the way back.
 // The encoder is k_wgblock in its WIRE form (same passes 1 and 2, codes stored in pass 3); the decoder below repeats
 // the second half of the bf16 kernel's pass 3 (code -> value, division by the scale, bf16 store), so that
 // decode(encode(x)) is the output of mor_fake_quantize bit for bit.
