@@ -91,6 +91,7 @@ def test_tags_round_trip_and_host_decode(G, shape, mode):
     if rows > 128:
         a[133, 7] = 0x7FC0              # a NaN and an infinity in tiles of their own
         a[9, 131] = 0xFF80
+        a[128:256, 128:256] = np.where(rng.random((128, 128)) < 0.5, 0x8000, 0).astype(np.uint16)    # zeros of both signs
     clamp = 1e-3
     print("mor wire", shape, mode, flush=True)
     payload, tags, scales = quantize(G, a, clamp, mode)
