@@ -50,3 +50,28 @@ def c4_mixture(rows=16384, cols=14336, seed=1004, tile=128, as_tensor=False):
     sign = torch.where(torch.rand(rows, cols, generator=g) < 0.5, -1.0, 1.0)
     t = torch.where(kind_e == 1, torch.exp(3 * t) * sign, torch.where(kind_e == 2, t * 1e-4, t))
     return t.to(torch.bfloat16) if as_tensor else _bits(t)
+
+
+def tile_mixture(rng, rows, cols):
+    """tiles of every kind MoR tells apart: narrow range, moderate, wide, outliers, tiny, zero, out of the fast range"""
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    kinds = rng.integers(0, 8, (rows // 128, cols // 128))
+    for by in range(rows // 128):
+        for bx in range(cols // 128):
+            t = x[by * 128:(by + 1) * 128, bx * 128:(bx + 1) * 128]
+            k = kinds[by, bx]
+            if k == 0:
+                t[:] = 1.0 + 0.3 * rng.random((128, 128))                       # range <= 7.5: E2M3
+            elif k == 1:
+                t *= np.exp(4 * rng.standard_normal((128, 128)))               # wide: the error sums decide
+            elif k == 2:
+                t[rng.random((128, 128)) < 0.01] *= 3000                      # outliers
+            elif k == 3:
+                t *= 1e-5
+            elif k == 4:
+                t[:] = 0
+            elif k == 5:
+                t *= 1e-33                                                    # scale outside the fast range
+            elif k == 6:
+                t[rng.random((128, 128)) < 0.3] = 0
+    return torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16).copy()

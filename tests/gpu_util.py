@@ -179,3 +179,21 @@ def fake_quantize_dual(a_u16, mode, sf_type, want_meta=True):
                                          mt.data_ptr() if want_meta else None, rows, cols, mode, sf_type, stream_ptr()))
     torch.cuda.synchronize()
     return to_host_u16(o), m.cpu().numpy(), to_host_u16(ot), mt.cpu().numpy()
+
+
+def fake_quantize_batch(arrays, blocks, clamp, mode, sf, flags=0, inplace=False):
+    """-> [(out bits, meta)] through mor_fake_quantize_batch, every tensor with the same clamp / mode / sf_type"""
+    from mor_amd.batch import TensorDesc
+    L = _cabi.lib()
+    xs = [to_dev_u16(a) for a in arrays]
+    outs = xs if inplace else [torch.full_like(x, 7.0) for x in xs]
+    metas = [torch.full((cdiv(a.shape[0], br), cdiv(a.shape[1], bc)), -7, dtype=torch.int32, device=dev())
+             for a, (br, bc) in zip(arrays, blocks)]
+    descs = (TensorDesc * len(xs))()
+    for d, x, y, m, (br, bc) in zip(descs, xs, outs, metas, blocks):
+        d.input, d.output, d.meta = x.data_ptr(), y.data_ptr(), m.data_ptr()
+        d.rows, d.cols, d.block_rows, d.block_cols = x.shape[0], x.shape[1], br, bc
+        d.clamp_threshold, d.mode, d.sf_type = clamp, mode, sf
+    _cabi.check(L.mor_fake_quantize_batch(descs, len(xs), flags, stream_ptr()))
+    torch.cuda.synchronize()
+    return [(to_host_u16(y), m.cpu().numpy()) for y, m in zip(outs, metas)]

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import mor_oracle as O
-from test_gpu_dual_tiles import mixture
+from data_gen import tile_mixture as mixture
 
 pytestmark = pytest.mark.gpu
 

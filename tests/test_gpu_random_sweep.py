@@ -169,7 +169,6 @@ def test_tile_entries_sweep(G, case):
     """128 x 128 tiles through the three entries that work on them besides mor_fake_quantize: the tile codes and their
     decode, both orientations from one read, and a batch call; all against the oracle."""
     import mor_amd
-    from test_gpu_batch import run_batch
     i, rows, cols, mode, kind = case
     rng = np.random.default_rng(5000 + i)
     a = make_data(rng, rows, cols, kind)
@@ -189,7 +188,7 @@ def test_tile_entries_sweep(G, case):
     assert np.array_equal(meta_t.cpu().numpy(), wmeta_t) and np.array_equal(G.to_host_u16(out_t), want_t), case
     # the same tensor three times in a batch (large enough for the tile path when rows * cols > 2^18), next to a small one
     small = make_data(rng, 64, 96, kind)
-    got = run_batch(G, [a, small, a, a], [(128, 128), (16, 32), (128, 128), (128, 128)], clamp, mode, 1)
+    got = G.fake_quantize_batch([a, small, a, a], [(128, 128), (16, 32), (128, 128), (128, 128)], clamp, mode, 1)
     for k in (0, 2, 3):
         assert np.array_equal(got[k][1], wmeta) and np.array_equal(got[k][0], want), (case, k)
     ws, wsm = O.fake_quantize(small, 16, 32, clamp, mode, 1)
