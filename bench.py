@@ -426,6 +426,11 @@ def mor_tile_codes(torch, cabi, run, add, x, out, label):
     n = x.numel()
     add("mor_tile_codes_quantize_" + label, enc, 2 * n + code_bytes + 8 * t.numel(), n)
     add("mor_tile_codes_dequantize_" + label, dec, 2 * n + code_bytes + 8 * t.numel(), n)
+    # the codes of the transposed tensor from the codes (tile by tile through LDS): the codes are read once and written once
+    payload_t, tags_t, scales_t = torch.empty_like(payload).view(gx, gy, TILE_PAYLOAD_BYTES), torch.empty((gx, gy), dtype=torch.int32, device="cuda"), torch.empty((gx, gy), dtype=torch.float32, device="cuda")
+    tr = lambda: cabi.check(L.mor_mor_transpose(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), payload_t.data_ptr(), tags_t.data_ptr(),
+                                                scales_t.data_ptr(), gy, gx, st()))
+    add("mor_tile_codes_transpose_" + label, tr, 2 * code_bytes + 16 * t.numel(), n)
 
 
 def flavour_differences(torch, run, cabi):

@@ -287,6 +287,17 @@ MOR_API int mor_mor_quantize(const void* input, void* payload, int32_t* tags, fl
 MOR_API int mor_mor_dequantize(const void* payload, const int32_t* tags, const float* scales, void* output,
                                int64_t rows, int64_t cols, void* stream);
 
+/*
+ * The tile codes of the transposed tensor from the tile codes of the tensor (no counterpart in the
+ * reference, whose callers quantize x.t().contiguous() in a call of its own): tile (i, j) of
+ * [tile_rows, tile_cols] tiles becomes tile (j, i) of [tile_cols, tile_rows] tiles with its codes
+ * transposed; tags and scales move with it (a tile and its transpose hold the same elements, so they
+ * share format and scale).  mor_mor_dequantize of the result is the transpose of mor_mor_dequantize of
+ * the source, bit for bit.  Source and destination are different buffers; payloads 16-byte aligned.
+ */
+MOR_API int mor_mor_transpose(const void* payload, const int32_t* tags, const float* scales, void* payload_t,
+                              int32_t* tags_t, float* scales_t, int64_t tile_rows, int64_t tile_cols, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,7 @@ SIGNATURES = {
     "mor_fake_quantize_dual_tiles": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _i64, _i64, _vp]),
     "mor_mor_quantize": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f64, _i64, _vp]),
     "mor_mor_dequantize": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "mor_mor_transpose": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
 }
 
 _lib = None

@@ -90,6 +90,105 @@ __global__ __launch_bounds__(WG) void k_mor_decode(const uint8_t* __restrict__ p
     }
 }
 
+// The codes of a tile, transposed: one workgroup per tile reads its slot, turns the tile through LDS and writes the
+// slot of the transposed tensor's tile (the same format, scale and tag: a tile and its transpose hold the same
+// elements).  8-bit codes travel as a 128 x 128 byte tile, 6-bit codes are unpacked to bytes on the way in and packed on
+// the way out, bf16 tiles go in two halves through the word layout of the two-output kernel.  Byte tile in LDS: row r
+// is 32 words, and word w of row r sits at position w ^ (r >> 3): the 16 lanes that collect, for one column, the bytes
+// of rows 8 j .. 8 j + 7 (j = 0 .. 15) read 16 different banks, and the four columns a wave handles at a time share
+// their words.
+__global__ __launch_bounds__(WG) void k_mor_transpose(const uint8_t* __restrict__ payload, const int32_t* __restrict__ tags,
+                                                      const float* __restrict__ scales, uint8_t* __restrict__ payload_t,
+                                                      int32_t* __restrict__ tags_t, float* __restrict__ scales_t, int gy, int gx,
+                                                      int64_t first) {
+    __shared__ __attribute__((aligned(16))) uint32_t s_t[128 * 32];            // 16 KiB: a byte tile, or half a bf16 tile
+    const int tid = threadIdx.x;
+    const int64_t bid = first + blockIdx.x;
+    const int by = (int)(bid / gx), bx = (int)(bid - (int64_t)by * gx);
+    const int64_t tid_t = (int64_t)bx * gy + by;
+    const uint8_t* slot = payload + bid * TILE_PAYLOAD_BYTES;
+    uint8_t* slot_t = payload_t + tid_t * TILE_PAYLOAD_BYTES;
+    const int tag = tags[bid];
+    const int fmt = (tag & TILE_STORED_BF16) ? -1 : mor_fmt_of(tag);
+    if (tid == 0) { tags_t[tid_t] = tag; scales_t[tid_t] = scales[bid]; }
+    if (fmt < 0) {
+        // bf16, the left and the right half of the tile in turn (64 columns = 32 words per row): vectors of 8 columns in,
+        // vectors of 8 rows out.  The word of columns (2 w, 2 w + 1) of row r sits at position w ^ ((r >> 3) << 1) of its
+        // row, as in the two-output kernel: a vector stays one aligned group of 4 words, in another order.
+        const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s_t);
+#pragma unroll 1
+        for (int h = 0; h < 2; ++h) {
+            if (h) __syncthreads();                                            // the first half has been read out
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int ch = k * WG + tid, r = ch >> 3, c8 = ch & 7, R = r >> 3;
+                const uint4 q = reinterpret_cast<const uint4*>(slot)[r * 16 + h * 8 + c8];
+                const uint4 p = (R & 1) ? make_uint4(q.z, q.w, q.x, q.y) : q;
+                *reinterpret_cast<uint4*>(s_t + r * 32 + ((c8 ^ (R >> 1)) << 2)) = p;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int ch = k * WG + tid, c = ch >> 4, j = ch & 15;       // column c of the half, rows 8 j .. 8 j + 7
+                const int at = 2 * ((c >> 1) ^ (j << 1)) + (c & 1);
+                uint32_t w[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t lo = s16[(8 * j + 2 * i) * 64 + at], hi = s16[(8 * j + 2 * i + 1) * 64 + at];
+                    w[i] = lo | (hi << 16);
+                }
+                reinterpret_cast<uint4*>(slot_t)[(h * 64 + c) * 16 + j] = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+        return;
+    }
+    const bool six = fmt == FMT_E2M3;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int ch = k * WG + tid, r = ch >> 4, cc = ch & 15, j = r >> 3;
+        uint2 v;
+        if (six) {
+            const uint16_t* p = reinterpret_cast<const uint16_t*>(slot) + 3 * ch;
+            const uint64_t bits = (uint64_t)p[0] | ((uint64_t)p[1] << 16) | ((uint64_t)p[2] << 32);
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                lo |= ((uint32_t)(bits >> (6 * i)) & 0x3Fu) << (8 * i);
+                hi |= ((uint32_t)(bits >> (6 * (i + 4))) & 0x3Fu) << (8 * i);
+            }
+            v = make_uint2(lo, hi);
+        } else {
+            v = reinterpret_cast<const uint2*>(slot)[ch];
+        }
+        // words 2 cc, 2 cc + 1 of row r at positions (2 cc) ^ j, (2 cc + 1) ^ j: one aligned pair, halves swapped for odd j
+        *reinterpret_cast<uint2*>(s_t + r * 32 + 2 * (cc ^ (j >> 1))) = (j & 1) ? make_uint2(v.y, v.x) : v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int ch = k * WG + tid, c = ch >> 4, j = ch & 15;             // column c of the tile, rows 8 j .. 8 j + 7
+        const int at = (c >> 2) ^ j, sh8 = 8 * (c & 3);
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            lo |= ((s_t[(8 * j + i) * 32 + at] >> sh8) & 0xFFu) << (8 * i);
+            hi |= ((s_t[(8 * j + 4 + i) * 32 + at] >> sh8) & 0xFFu) << (8 * i);
+        }
+        if (six) {
+            uint64_t bits = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                bits |= (uint64_t)((lo >> (8 * i)) & 0x3Fu) << (6 * i);
+                bits |= (uint64_t)((hi >> (8 * i)) & 0x3Fu) << (6 * (i + 4));
+            }
+            uint16_t* d = reinterpret_cast<uint16_t*>(slot_t) + 3 * ch;
+            d[0] = (uint16_t)bits; d[1] = (uint16_t)(bits >> 16); d[2] = (uint16_t)(bits >> 32);
+        } else {
+            reinterpret_cast<uint2*>(slot_t)[ch] = make_uint2(lo, hi);
+        }
+    }
+}
+
 }  // namespace mor
 
 static int check_tiles(const void* a, const void* b, const void* tags, const void* scales, int64_t rows, int64_t cols) {
@@ -146,4 +245,21 @@ extern "C" int mor_mor_dequantize(const void* payload, const int32_t* tags, cons
         else k_mor_decode<0><<<count, WG, 0, st>>>(p, tags, scales, out, sh, band, first);
     });
     return mor_check_launch("k_mor_decode");
+}
+
+extern "C" int mor_mor_transpose(const void* payload, const int32_t* tags, const float* scales, void* payload_t, int32_t* tags_t,
+                                 float* scales_t, int64_t tile_rows, int64_t tile_cols, void* stream) {
+    if (tile_rows <= 0 || tile_cols <= 0 || tile_rows > (1 << 20) || tile_cols > (1 << 20) || tile_rows * tile_cols > ((int64_t)1 << 30))
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "bad tile grid %lld x %lld", (long long)tile_rows, (long long)tile_cols);
+    if (!payload || !tags || !scales || !payload_t || !tags_t || !scales_t) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "NULL pointer");
+    if ((reinterpret_cast<uintptr_t>(payload) | reinterpret_cast<uintptr_t>(payload_t)) & 15u)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "payloads must be 16-byte aligned");
+    if (payload == payload_t || tags == tags_t || scales == scales_t)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "source and destination must be different buffers");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    for_slices(tile_rows * tile_cols, [&](int64_t first, int count) {
+        k_mor_transpose<<<count, WG, 0, st>>>(static_cast<const uint8_t*>(payload), tags, scales, static_cast<uint8_t*>(payload_t), tags_t, scales_t,
+                                              (int)tile_rows, (int)tile_cols, first);
+    });
+    return mor_check_launch("k_mor_transpose");
 }

@@ -146,3 +146,20 @@ def dequantize_mor_tiles(payload: Tensor, tags: Tensor, scales: Tensor) -> Tenso
         _cabi.check(_L.mor_mor_dequantize(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, cols,
                                           _stream(payload)))
     return out
+
+
+def transpose_mor_tiles(payload: Tensor, tags: Tensor, scales: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+    """(payload, tags, scales) of a tensor -> those of its transpose (tile (i, j) becomes tile (j, i), its codes
+    transposed): the operand of the GEMM that reduces over the other dimension, without quantizing x.t() again."""
+    if (payload.dtype != torch.uint8 or tags.dtype != torch.int32 or scales.dtype != torch.float32 or not payload.is_cuda
+            or tags.dim() != 2 or scales.shape != tags.shape or payload.numel() != tags.numel() * TILE_PAYLOAD_BYTES):
+        raise RuntimeError("mor: expected (uint8 payload, int32 tags, float32 scales) of one tile grid on the GPU")
+    payload, tags, scales = payload.contiguous(), tags.contiguous(), scales.contiguous()
+    gy, gx = tags.shape
+    with torch.cuda.device(payload.device):
+        payload_t = torch.empty((gx, gy, TILE_PAYLOAD_BYTES), dtype=torch.uint8, device=payload.device)
+        tags_t = torch.empty((gx, gy), dtype=torch.int32, device=payload.device)
+        scales_t = torch.empty((gx, gy), dtype=torch.float32, device=payload.device)
+        _cabi.check(_L.mor_mor_transpose(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), payload_t.data_ptr(), tags_t.data_ptr(),
+                                         scales_t.data_ptr(), gy, gx, _stream(payload)))
+    return payload_t, tags_t, scales_t

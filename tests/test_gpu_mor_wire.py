@@ -269,3 +269,75 @@ def test_tile_entries_replay_in_a_hip_graph(G):
             assert torch.equal(cap[k].view(torch.int32) if cap[k].dtype == torch.float32 else cap[k], eager[k].view(torch.int32) if eager[k].dtype == torch.float32 else eager[k]), (rep, k)
         assert np.array_equal(G.to_host_u16(cap["back"]), ref) and np.array_equal(G.to_host_u16(cap["bout"]), ref), rep
         assert np.array_equal(cap["bmeta"].cpu().numpy(), rmeta), rep
+
+
+def host_transpose_slot(slot, tag):
+    """the slot of the transposed tile, from the documented layout"""
+    out = np.full(TILE_BYTES, 0xA5, dtype=np.uint8)
+    if tag & STORED_BF16 or tag == 3:
+        out[:128 * 256] = np.ascontiguousarray(slot[:128 * 256].view(np.uint16).reshape(128, 128).T).view(np.uint8).ravel()
+    elif tag in (1, 11, 2, 12):
+        out[:128 * 128] = np.ascontiguousarray(slot[:128 * 128].reshape(128, 128).T).ravel()
+    else:
+        b = slot[:128 * 96].reshape(128, 32, 3).astype(np.uint32)
+        w = b[..., 0] | (b[..., 1] << 8) | (b[..., 2] << 16)
+        codes = np.stack([(w >> (6 * k)) & 0x3F for k in range(4)], axis=-1).reshape(128, 128).T.reshape(128, 32, 4)
+        w = codes[..., 0] | (codes[..., 1] << 6) | (codes[..., 2] << 12) | (codes[..., 3] << 18)
+        out[:128 * 96] = np.stack([w & 0xFF, (w >> 8) & 0xFF, (w >> 16) & 0xFF], axis=-1).astype(np.uint8).ravel()
+    return out
+
+
+@pytest.mark.parametrize("shape", [(128, 128), (256, 640), (1024, 512), (384, 2048)])
+def test_transposed_tile_codes(G, shape):
+    """mor_mor_transpose: every slot is the transposed tile in the same packing, tags and scales move with their tiles,
+    and the result decodes to the transpose of what the source decodes to."""
+    import mor_amd
+    rows, cols = shape
+    rng = np.random.default_rng(rows * 11 + cols)
+    a = mixture(rng, rows, cols)
+    if rows > 128:
+        a[133, 7] = 0x7FC0
+    payload, tags, scales = quantize(G, a, 1e-3, 1)
+    gy, gx = tags.shape
+    payload_t = torch.full((gx, gy, TILE_BYTES), 0xA5, dtype=torch.uint8, device=G.dev())
+    tags_t = torch.full((gx, gy), -7, dtype=torch.int32, device=G.dev())
+    scales_t = torch.full((gx, gy), -7.0, dtype=torch.float32, device=G.dev())
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    _cabi.check(L.mor_mor_transpose(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), payload_t.data_ptr(), tags_t.data_ptr(),
+                                    scales_t.data_ptr(), gy, gx, G.stream_ptr()))
+    torch.cuda.synchronize()
+    assert torch.equal(tags_t, tags.t()) and torch.equal(scales_t, scales.t())
+    p, pt, t = payload.cpu().numpy(), payload_t.cpu().numpy(), tags.cpu().numpy()
+    seen = set()
+    for by in range(gy):
+        for bx in range(gx):
+            assert np.array_equal(pt[bx, by], host_transpose_slot(p[by, bx], int(t[by, bx]))), (by, bx, int(t[by, bx]))
+            seen.add(int(t[by, bx]))
+    back = dequantize(G, payload, tags, scales)
+    back_t = dequantize(G, payload_t, tags_t, scales_t)
+    assert np.array_equal(back_t, np.ascontiguousarray(back.T))
+    if rows * cols >= 1024 * 512:
+        assert len({x & 0xFF for x in seen}) >= 3 and any(x & STORED_BF16 for x in seen), seen
+    # the Python helper
+    pt2, tt2, st2 = mor_amd.wire.transpose_mor_tiles(payload, tags, scales)
+    assert torch.equal(tt2, tags_t) and torch.equal(st2, scales_t)
+    assert np.array_equal(G.to_host_u16(mor_amd.wire.dequantize_mor_tiles(pt2, tt2, st2)), back_t)
+
+
+def test_transposed_tile_codes_equal_the_codes_of_the_transpose(G):
+    """On tiles whose decision does not hang on the order of the error sums, transposing the codes equals quantizing the
+    transposed tensor (the same elements, the same amax, scale and format)."""
+    import mor_amd
+    rows, cols = 1024, 768
+    g = torch.Generator(device="cuda").manual_seed(23)
+    x = torch.randn(rows, cols, device="cuda", generator=g)
+    x[:, :256] = 1.0 + 0.3 * torch.rand(rows, 256, device="cuda", generator=g)
+    x = x.to(torch.bfloat16)
+    for mode in (101, 2):                                        # (dynamic-range rule and a forced format: no error sums)
+        p, t, s = mor_amd.wire.quantize_mor_tiles(x, 1e-3, mode)
+        pt, tt, st = mor_amd.wire.transpose_mor_tiles(p, t, s)
+        q, u, v = mor_amd.wire.quantize_mor_tiles(x.t().contiguous(), 1e-3, mode)
+        assert torch.equal(tt, u) and torch.equal(st, v)
+        used = torch.where((u == 4)[..., None], torch.arange(TILE_BYTES, device="cuda") < 128 * 96, torch.arange(TILE_BYTES, device="cuda") < 128 * 128)
+        assert torch.equal(pt[used], q[used])
