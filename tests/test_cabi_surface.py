@@ -75,3 +75,7 @@ def test_tile_code_entries_reject_bad_arguments_without_a_gpu():
     assert L.mor_mor_quantize(256, 512, None, 1024, 128, 256, 0.0, 1, None) == -1
     assert L.mor_mor_dequantize(512, 768, 1024, 256, 100, 256, None) == -1
     assert L.mor_mor_dequantize(512, None, 1024, 256, 128, 256, None) == -1
+    assert L.mor_mor_transpose(512, 768, 1024, 1536, 2048, 2560, 0, 4, None) == -1 and b"tile grid" in L.mor_last_error()
+    assert L.mor_mor_transpose(512, 768, 1024, 512, 2048, 2560, 2, 4, None) == -1 and b"different" in L.mor_last_error()
+    assert L.mor_mor_transpose(512, 768, 1024, 1544, 2048, 2560, 2, 4, None) == -1 and b"aligned" in L.mor_last_error()
+    assert L.mor_mor_transpose(512, None, 1024, 1536, 2048, 2560, 2, 4, None) == -1
