@@ -190,7 +190,7 @@ extern "C" int mor_fake_quantize_batch(const MorTensorDesc* descs, int64_t n, ui
             const int64_t cpr = d.block_cols / 8;
             bool blocks = fast_ok && (nch == WG || nch == 2 * WG || nch == 4 * WG || nch == 8 * WG)
                           && d.rows % d.block_rows == 0 && d.cols % d.block_cols == 0 && (d.block_rows == 1 || is_pow2(cpr))
-                          && nblocks <= (1 << 20) && d.block_rows * (d.cols / 8) < 0x7FFFFFFFll
+                          && nblocks <= (1 << 20) && d.rows <= 0x7FFFFFFFll && d.cols <= 0x7FFFFFFFll && d.block_rows * (d.cols / 8) < 0x7FFFFFFFll
                           && ((reinterpret_cast<uintptr_t>(d.input) | reinterpret_cast<uintptr_t>(d.output)) & 15u) == 0
                           && (d.sf_type == 1 || d.sf_type == 2) && mor_decode_mode(d.mode, d.clamp_threshold, tq) && tq.qmode != 4;
             if (blocks && tq.qmode == 1 && nch != 8 * WG) blocks = false;
