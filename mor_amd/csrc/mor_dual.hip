@@ -38,6 +38,8 @@ extern "C" int mor_fake_quantize_dual_tiles(const void* input, void* output, int
         return mor_fail(MOR_ERR_INVALID_ARGUMENT, "rows and cols must be multiples of 128 (got %lld x %lld)", (long long)rows, (long long)cols);
     if ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(output) | reinterpret_cast<uintptr_t>(output_t)) & 15u)
         return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensors must be 16-byte aligned");
+    if (cols >= ((int64_t)1 << 27) || rows >= ((int64_t)1 << 27))              // (a tile row's chunk offsets are 32-bit, in both tensors)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "more than 2^27 rows or columns (%lld x %lld)", (long long)rows, (long long)cols);
     if (input == output || input == output_t || output == output_t)
         return mor_fail(MOR_ERR_INVALID_ARGUMENT, "input and the two outputs must be three different tensors");
     QuantArgs qa;

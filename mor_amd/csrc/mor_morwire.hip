@@ -199,6 +199,8 @@ static int check_tiles(const void* a, const void* b, const void* tags, const voi
     if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u)
         return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor and payload must be 16-byte aligned");
     if (a == b) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor and payload must be different buffers");
+    if (cols >= ((int64_t)1 << 27))                  // (a tile row's chunk offsets are 32-bit)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "more than 2^27 columns (%lld)", (long long)cols);
     return MOR_OK;
 }
 

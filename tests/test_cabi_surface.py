@@ -79,3 +79,6 @@ def test_tile_code_entries_reject_bad_arguments_without_a_gpu():
     assert L.mor_mor_transpose(512, 768, 1024, 512, 2048, 2560, 2, 4, None) == -1 and b"different" in L.mor_last_error()
     assert L.mor_mor_transpose(512, 768, 1024, 1544, 2048, 2560, 2, 4, None) == -1 and b"aligned" in L.mor_last_error()
     assert L.mor_mor_transpose(512, None, 1024, 1536, 2048, 2560, 2, 4, None) == -1
+    # a tile row's chunk offsets are 32-bit: tensors of 2^27 columns and more are refused
+    assert L.mor_mor_quantize(256, 512, 768, 1024, 128, 1 << 27, 0.0, 1, None) == -1 and b"columns" in L.mor_last_error()
+    assert L.mor_fake_quantize_dual_tiles(256, 512, 768, 1024, 1280, 128, 1 << 27, 0.0, 1, 1, None) == -1 and b"2^27" in L.mor_last_error()
