@@ -163,3 +163,11 @@ def transpose_mor_tiles(payload: Tensor, tags: Tensor, scales: Tensor) -> Tuple[
         _cabi.check(_L.mor_mor_transpose(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), payload_t.data_ptr(), tags_t.data_ptr(),
                                          scales_t.data_ptr(), gy, gx, _stream(payload)))
     return payload_t, tags_t, scales_t
+
+
+def quantize_mor_tiles_dual(x: Tensor, clamp_threshold: float = 0.0, mode: int = 1):
+    """Tile codes of x and of x.t() (the operands of the two GEMMs that reduce over either dimension of x) from one
+    decision per tile: quantize_mor_tiles(x), then transpose_mor_tiles of the result.
+    -> ((payload, tags, scales), (payload_t, tags_t, scales_t))"""
+    codes = quantize_mor_tiles(x, clamp_threshold, mode)
+    return codes, transpose_mor_tiles(*codes)

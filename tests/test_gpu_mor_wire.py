@@ -319,7 +319,10 @@ def test_transposed_tile_codes(G, shape):
     assert np.array_equal(back_t, np.ascontiguousarray(back.T))
     if rows * cols >= 1024 * 512:
         assert len({x & 0xFF for x in seen}) >= 3 and any(x & STORED_BF16 for x in seen), seen
-    # the Python helper
+    # the Python helpers
+    (p3, t3, s3), (pt3, tt3, st3) = mor_amd.wire.quantize_mor_tiles_dual(G.to_dev_u16(a), 1e-3, 1)
+    assert torch.equal(t3, tags) and torch.equal(tt3, tags_t) and torch.equal(st3, scales_t)
+    assert np.array_equal(G.to_host_u16(mor_amd.wire.dequantize_mor_tiles(pt3, tt3, st3)), back_t)
     pt2, tt2, st2 = mor_amd.wire.transpose_mor_tiles(payload, tags, scales)
     assert torch.equal(tt2, tags_t) and torch.equal(st2, scales_t)
     assert np.array_equal(G.to_host_u16(mor_amd.wire.dequantize_mor_tiles(pt2, tt2, st2)), back_t)
