@@ -431,6 +431,10 @@ def mor_tile_codes(torch, cabi, run, add, x, out, label):
     tr = lambda: cabi.check(L.mor_mor_transpose(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), payload_t.data_ptr(), tags_t.data_ptr(),
                                                 scales_t.data_ptr(), gy, gx, st()))
     add("mor_tile_codes_transpose_" + label, tr, 2 * code_bytes + 16 * t.numel(), n)
+    # both in one call (two launches)
+    both = lambda: cabi.check(L.mor_mor_quantize_dual(x.data_ptr(), payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), payload_t.data_ptr(),
+                                                      tags_t.data_ptr(), scales_t.data_ptr(), rows, cols, 1e-15, 1, st()))
+    add("mor_tile_codes_quantize_dual_" + label, both, 2 * n + 2 * code_bytes + 16 * t.numel(), n)
 
 
 def flavour_differences(torch, run, cabi):

@@ -298,6 +298,15 @@ MOR_API int mor_mor_dequantize(const void* payload, const int32_t* tags, const f
 MOR_API int mor_mor_transpose(const void* payload, const int32_t* tags, const float* scales, void* payload_t,
                               int32_t* tags_t, float* scales_t, int64_t tile_rows, int64_t tile_cols, void* stream);
 
+/*
+ * mor_mor_quantize and mor_mor_transpose of its result in one call (no counterpart in the
+ * reference): payload / tags / scales as mor_mor_quantize writes them, payload_t / tags_t / scales_t
+ * as mor_mor_transpose writes them.  Every output its own buffer.
+ */
+MOR_API int mor_mor_quantize_dual(const void* input, void* payload, int32_t* tags, float* scales, void* payload_t,
+                                  int32_t* tags_t, float* scales_t, int64_t rows, int64_t cols,
+                                  double clamp_threshold, int64_t mode, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

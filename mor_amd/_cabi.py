@@ -43,6 +43,7 @@ SIGNATURES = {
     "mor_mor_quantize": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f64, _i64, _vp]),
     "mor_mor_dequantize": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "mor_mor_transpose": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "mor_mor_quantize_dual": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _i64, _vp]),
 }
 
 _lib = None

@@ -265,3 +265,16 @@ extern "C" int mor_mor_transpose(const void* payload, const int32_t* tags, const
     });
     return mor_check_launch("k_mor_transpose");
 }
+
+// Both orientations in one call: the codes of the tensor, then the codes of its transpose from them (two launches; a
+// kernel that wrote both from one read of the tensor was built and measured no faster: 63.4 against 61.6 us at 8192^2 from
+// HBM, the transposition through LDS and the second slot lengthen every workgroup by what the second launch costs).
+extern "C" int mor_mor_quantize_dual(const void* input, void* payload, int32_t* tags, float* scales, void* payload_t, int32_t* tags_t,
+                                     float* scales_t, int64_t rows, int64_t cols, double clamp_threshold, int64_t mode, void* stream) {
+    if (!payload_t || !tags_t || !scales_t) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "NULL pointer of the transposed tensor");
+    if (payload_t == input || payload_t == payload || tags_t == tags || scales_t == scales)
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "the outputs of the two orientations must be different buffers");
+    if (reinterpret_cast<uintptr_t>(payload_t) & 15u) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "payloads must be 16-byte aligned");
+    if (int rc = mor_mor_quantize(input, payload, tags, scales, rows, cols, clamp_threshold, mode, stream)) return rc;
+    return mor_mor_transpose(payload, tags, scales, payload_t, tags_t, scales_t, rows / 128, cols / 128, stream);
+}

@@ -167,7 +167,20 @@ def transpose_mor_tiles(payload: Tensor, tags: Tensor, scales: Tensor) -> Tuple[
 
 def quantize_mor_tiles_dual(x: Tensor, clamp_threshold: float = 0.0, mode: int = 1):
     """Tile codes of x and of x.t() (the operands of the two GEMMs that reduce over either dimension of x) from one
-    decision per tile: quantize_mor_tiles(x), then transpose_mor_tiles of the result.
+    decision per tile: what quantize_mor_tiles(x) and transpose_mor_tiles of it return, in one call.
     -> ((payload, tags, scales), (payload_t, tags_t, scales_t))"""
-    codes = quantize_mor_tiles(x, clamp_threshold, mode)
-    return codes, transpose_mor_tiles(*codes)
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_cuda:
+        raise RuntimeError("mor: expected a 2-D bfloat16 GPU tensor")
+    rows, cols = x.shape
+    if rows % 128 or cols % 128:
+        raise RuntimeError(f"mor: tile codes need rows and cols that are multiples of 128, got {tuple(x.shape)}")
+    x = x.contiguous()
+    gy, gx = rows // 128, cols // 128
+    with torch.cuda.device(x.device):
+        mk = lambda a, b: (torch.empty((a, b, TILE_PAYLOAD_BYTES), dtype=torch.uint8, device=x.device),
+                           torch.empty((a, b), dtype=torch.int32, device=x.device), torch.empty((a, b), dtype=torch.float32, device=x.device))
+        p, t, s = mk(gy, gx)
+        pt, tt, st = mk(gx, gy)
+        _cabi.check(_L.mor_mor_quantize_dual(x.data_ptr(), p.data_ptr(), t.data_ptr(), s.data_ptr(), pt.data_ptr(), tt.data_ptr(), st.data_ptr(),
+                                             rows, cols, float(clamp_threshold), mode, _stream(x)))
+    return (p, t, s), (pt, tt, st)

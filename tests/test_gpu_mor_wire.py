@@ -344,3 +344,38 @@ def test_transposed_tile_codes_equal_the_codes_of_the_transpose(G):
         assert torch.equal(tt, u) and torch.equal(st, v)
         used = torch.where((u == 4)[..., None], torch.arange(TILE_BYTES, device="cuda") < 128 * 96, torch.arange(TILE_BYTES, device="cuda") < 128 * 128)
         assert torch.equal(pt[used], q[used])
+
+
+@pytest.mark.parametrize("shape", [(128, 128), (256, 640), (1024, 512), (2048, 2048)])
+@pytest.mark.parametrize("mode", [1, 101, 2])
+def test_both_orientations_in_one_call(G, shape, mode):
+    """mor_mor_quantize_dual writes, byte for byte (slot tails untouched), what mor_mor_quantize and mor_mor_transpose
+    of its result write."""
+    from mor_amd import _cabi
+    L = _cabi.lib()
+    rows, cols = shape
+    rng = np.random.default_rng(rows * 13 + cols + mode)
+    a = mixture(rng, rows, cols)
+    if rows > 128:
+        a[133, 7] = 0x7FC0
+        a[128:256, 128:256] = np.where(rng.random((128, 128)) < 0.5, 0x8000, 0).astype(np.uint16)
+    print("tile codes, both orientations", shape, mode, flush=True)
+    payload, tags, scales = quantize(G, a, 1e-3, mode)
+    gy, gx = tags.shape
+
+    def fresh(y, x):
+        return (torch.full((y, x, TILE_BYTES), 0xA5, dtype=torch.uint8, device=G.dev()), torch.full((y, x), -7, dtype=torch.int32, device=G.dev()),
+                torch.full((y, x), -7.0, dtype=torch.float32, device=G.dev()))
+
+    pt, tt, st = fresh(gx, gy)
+    _cabi.check(L.mor_mor_transpose(payload.data_ptr(), tags.data_ptr(), scales.data_ptr(), pt.data_ptr(), tt.data_ptr(), st.data_ptr(), gy, gx, G.stream_ptr()))
+    p2, t2, s2 = fresh(gy, gx)
+    pt2, tt2, st2 = fresh(gx, gy)
+    x = G.to_dev_u16(a)
+    _cabi.check(L.mor_mor_quantize_dual(x.data_ptr(), p2.data_ptr(), t2.data_ptr(), s2.data_ptr(), pt2.data_ptr(), tt2.data_ptr(), st2.data_ptr(),
+                                        rows, cols, 1e-3, mode, G.stream_ptr()))
+    torch.cuda.synchronize()
+    assert torch.equal(t2, tags) and torch.equal(s2.view(torch.int32), scales.view(torch.int32)) and torch.equal(p2, payload)
+    assert torch.equal(tt2, tt) and torch.equal(st2.view(torch.int32), st.view(torch.int32)) and torch.equal(pt2, pt)
+    assert L.mor_mor_quantize_dual(x.data_ptr(), p2.data_ptr(), t2.data_ptr(), s2.data_ptr(), p2.data_ptr(), tt2.data_ptr(), st2.data_ptr(),
+                                   rows, cols, 1e-3, mode, G.stream_ptr()) != 0 and b"different" in L.mor_last_error()
