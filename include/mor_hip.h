@@ -43,6 +43,11 @@ extern "C" {
 #define MOR_FLAG_TORCH_EMULATION 1u
 /* Do not use the gfx950 FP8 convert instructions; cast in integer/float software. */
 #define MOR_FLAG_SOFTWARE_CAST 2u
+/* MoR (FQ:487-584, 661): compute the two error sums of every block that needs them with the reference's
+ * divisions and in the order of the reference's additions (its thread layout and shuffle trees), which
+ * is what the kernels otherwise do only for blocks whose two sums are within 1e-5 of each other.  The
+ * results are the same either way; the flag exists so that tests can compare the sums bit for bit. */
+#define MOR_FLAG_REFERENCE_ORDER_SUMS 4u
 
 /* element formats for mor_block_format / mor_quant_dequant */
 #define MOR_FMT_E4M3 0
@@ -162,9 +167,11 @@ MOR_API int mor_block_stats(const void* input, int64_t rows, int64_t cols, int64
                     float fmax, float* amax, float* scale, int32_t* e8m0, void* stream);
 
 /* Per block {amax, min non-zero |x|, E4M3 error sum, E5M2 error sum} of the MoR decision
- * (FQ:407-584); error sums are 0 for blocks that did not need them.  4 floats per block. */
+ * (FQ:407-584); error sums are 0 for blocks that did not need them.  4 floats per block.  The sums of a
+ * block are the reference's bit for bit when they are within 1e-5 of each other, and for every block with
+ * MOR_FLAG_REFERENCE_ORDER_SUMS; otherwise they agree with the reference's within 1e-6 relative. */
 MOR_API int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t block_rows, int64_t block_cols,
-                  double clamp_threshold, int64_t mode, int64_t sf_type, float* stats, void* stream);
+                  double clamp_threshold, int64_t mode, int64_t sf_type, float* stats, uint32_t flags, void* stream);
 
 /*
  * Exhaustive on-device comparison of the gfx950 FP8 convert instructions with the software

@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmor_hip.so")
 FLAG_DEFAULT = 0
 FLAG_TORCH_EMULATION = 1
 FLAG_SOFTWARE_CAST = 2
+FLAG_REFERENCE_ORDER_SUMS = 4
 FMT_E4M3, FMT_E5M2, FMT_E3M2, FMT_E2M3 = 0, 1, 2, 3
 OP_FAKE_QUANTIZE, OP_BLOCK_SCALING, OP_CHANNEL_SCALING, OP_E8MX = 0, 1, 2, 3
 
@@ -30,7 +31,7 @@ SIGNATURES = {
     "mor_quant_dequant": (_int, [_vp, _vp, _i64, _int, _vp]),
     "mor_e4m3_with_e8_scale": (_int, [_vp, _vp, _i64, _int, _vp]),
     "mor_block_stats": (_int, [_vp, _i64, _i64, _i64, _i64, C.c_float, _vp, _vp, _vp, _vp]),
-    "mor_mor_stats": (_int, [_vp, _i64, _i64, _i64, _i64, _f64, _i64, _i64, _vp, _vp]),
+    "mor_mor_stats": (_int, [_vp, _i64, _i64, _i64, _i64, _f64, _i64, _i64, _vp, _u32, _vp]),
     "mor_selftest_hw_cast": (_int, [_vp, _vp]),
     "mor_selftest_hw_wire": (_int, [_vp, _vp]),
     "mor_selftest_mx_mfma": (_int, [_vp, _vp, _vp, _vp, _int, _vp, _vp]),

@@ -134,7 +134,7 @@ static int block_nt_class(int64_t bytes) { return bytes >= ((int64_t)64 << 20) ?
 template <bool MOR, bool E8, int NV>
 static void launch_batch_blocks_nv(const BlockArgs& a, int nt, hipStream_t st) {
     const uint32_t grid = a.first[a.n];
-    const size_t dyn_lds = (NV == 8 && grid >= 4096) ? 53000 : 0;    // three workgroups per CU on large grids (launch_wgblock_nv)
+    const size_t dyn_lds = (NV == 8 && grid >= 4096) ? 53000 - (MOR ? REF_SUMS_LDS_BYTES : 0) : 0;    // three workgroups per CU on large grids (launch_wgblock_nv)
     if (nt == 1) k_batch_blocks<MOR, E8, NV, 1><<<grid, WG, dyn_lds, st>>>(a);
     else if (nt == 2) k_batch_blocks<MOR, E8, NV, 2><<<grid, WG, dyn_lds, st>>>(a);
     else k_batch_blocks<MOR, E8, NV, 0><<<grid, WG, dyn_lds, st>>>(a);

@@ -21,7 +21,7 @@ static void launch_dual(const uint4* in, uint4* out, int32_t* meta, uint4* out_t
     const int shift = (nblocks >= 2048 && sh.gx % 8 == 0 && nblocks % 8 == 0) ? (4 | 256) : 4;
     // large grids: three workgroups per CU, as for the one-output kernel (unused dynamic LDS on top of the tile's 32 KiB;
     // 8192^2: 83 -> 81 us)
-    const size_t dl = nblocks >= 4096 ? 20000 : 0;
+    const size_t dl = nblocks >= 4096 ? 20000 - (MOR ? REF_SUMS_LDS_BYTES : 0) : 0;
     for_slices(nblocks, [&](int64_t first, int count) {
         if (ntm == 1) k_wgblock<MOR, E8, 8, true, 1, WG, false, true><<<count, WG, dl, st>>>(in, out, meta, nullptr, sh, qa, 16, shift, first, out_t, meta_t);
         else if (ntm == 2) k_wgblock<MOR, E8, 8, true, 2, WG, false, true><<<count, WG, 0, st>>>(in, out, meta, nullptr, sh, qa, 16, shift, first, out_t, meta_t);

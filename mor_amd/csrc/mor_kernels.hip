@@ -526,6 +526,7 @@ extern "C" int mor_fake_quantize(const void* input, void* output, int32_t* meta,
         }
         return mor_check_launch("k_copy / k_fill_i32");
     }
+    qa.ref_sums = (flags & MOR_FLAG_REFERENCE_ORDER_SUMS) ? 1 : 0;
     return run_quantize(input, output, meta, nullptr, rows, cols, brows, bcols, qa, e8, flags, st);
 }
 
@@ -541,14 +542,15 @@ extern "C" int mor_block_format(const void* input, void* output,
 }
 
 extern "C" int mor_mor_stats(const void* input, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,
-                             double clamp_threshold, int64_t mode, int64_t sf_type, float* stats, void* stream) {
+                             double clamp_threshold, int64_t mode, int64_t sf_type, float* stats, uint32_t flags, void* stream) {
     if (int rc = mor_validate_shape(input, rows, cols, brows, bcols)) return rc;
     if (!stats) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "stats is NULL");
     QuantArgs qa{};
     qa.qmode = 1; qa.fmt = -1; qa.meta_val = -1;
     qa.clamp = (float)clamp_threshold;
     qa.dyn_range = (mode / 100 > 0) ? 1 : 0;
-    return run_quantize(input, nullptr, nullptr, stats, rows, cols, brows, bcols, qa, sf_type == 2, MOR_FLAG_DEFAULT, static_cast<hipStream_t>(stream));
+    qa.ref_sums = (flags & MOR_FLAG_REFERENCE_ORDER_SUMS) ? 1 : 0;
+    return run_quantize(input, nullptr, nullptr, stats, rows, cols, brows, bcols, qa, sf_type == 2, flags, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mor_block_stats(const void* input, int64_t rows, int64_t cols, int64_t brows, int64_t bcols,

@@ -218,10 +218,10 @@ extern "C" int mor_mor_quantize(const void* input, void* payload, int32_t* tags,
     const int shift = (nblocks >= 2048 && sh.gx % 8 == 0 && nblocks % 8 == 0) ? (4 | 256) : 4;
     // four workgroups per CU on large grids (the bf16 kernel runs three: half the bytes are written here; 8192^2 from HBM:
     // 42.0 us with three, 39.3 with four, 39.1 - 40.0 without a cap)
-    const size_t dl = nblocks >= 4096 ? 36000 : 0;
+    const bool mor = qa.qmode == 1;
+    const size_t dl = nblocks >= 4096 ? 36000 - (mor ? REF_SUMS_LDS_BYTES : 0) : 0;
     const uint4* in = static_cast<const uint4*>(input);
     uint4* out = static_cast<uint4*>(payload);
-    const bool mor = qa.qmode == 1;
     for_slices(nblocks, [&](int64_t first, int count) {
 #define MOR_TILE_CODES(MOR_, NT_) k_wgblock<MOR_, false, 8, true, NT_, WG, false, false, true><<<count, WG, dl, st>>>(in, out, tags, scales, sh, qa, 16, shift, first, nullptr, nullptr)
         if (mor) { if (stream_loads) MOR_TILE_CODES(true, 1); else MOR_TILE_CODES(true, 0); }

@@ -21,6 +21,7 @@ struct QuantArgs {
     int meta_val;     // value written to meta for qmode 2 / 4; < 0: leave meta alone
     int dyn_range;    // MoR decision by dynamic range instead of quantization error
     float clamp;      // clamp_threshold
+    int ref_sums;     // MoR: every error sum with the reference's divisions in the reference's order (else only the close ones)
 };
 
 // ------------------------------------------------------------------------------------------------
@@ -83,6 +84,105 @@ __device__ __forceinline__ void err_terms_exact(float x, bool e8, const Scale& s
         e4 += fabsf(q4 / x - 1.0f);
         e5 += fabsf(q5 / x - 1.0f);
     }
+}
+
+// The two MoR error sums of one block as the reference computes them (FQ:487-584): its arithmetic (err_terms_exact)
+// and the order of its additions.  The reference runs tbx x tby threads on a block: 16 x 32 on blocks of more than
+// 1024 elements, (block_cols / 2) x block_rows otherwise (FQ:1770-1789).  Thread (tx, ty) walks the rows ty, ty + tby,
+// ... and in each the packed words tx, tx + tbx, ..., adding (term of the odd column + term of the even column) of
+// every word to its own sum; 32 consecutive threads (in row-major order of (ty, tx)) then add their sums in a
+// shuffle-down tree (lane i += lane i + 16, 8, 4, 2, 1) and the warps' sums meet in one more such tree over 32 slots,
+// the unused ones zero.  Here the workgroup's threads take the reference's threads ("virtual threads") in turn, the
+// sums go through LDS and the trees are made of the same additions.  Shapes the reference cannot launch (odd widths,
+// thread counts that are not whole warps) have no such order: their terms are added in double and rounded once.
+// Called by all WGS threads of the workgroup with the same arguments; ld(r, c) returns the bf16 bits of element (r, c)
+// of the block's valid part bh x bw; every thread gets the sums.
+// This is the rare path (error sums too close to call) and the exact path: its cost does not matter.
+// Its LDS: one copy per kernel, however many call sites the kernel has.
+constexpr int REF_SUMS_MAXVT = 1024;                  // the reference's largest thread block
+struct RefSumsLds { float p4[REF_SUMS_MAXVT], p5[REF_SUMS_MAXVT], w4[32], w5[32]; double d[2][16]; };
+constexpr int REF_SUMS_LDS_BYTES = (int)sizeof(RefSumsLds);
+__device__ __forceinline__ RefSumsLds& ref_sums_lds() {
+    __shared__ RefSumsLds s;
+    return s;
+}
+template <bool EMU, int WGS, class Ld>
+__device__ __forceinline__ void err_sums_reference_order(Ld&& ld, int bh, int bw, int64_t brows, int64_t bcols, bool even_cols,
+                                                         bool e8, const Scale& s4, const Scale& s5, float& e4, float& e5) {
+    static_assert(WGS / 64 <= 16, "at most 16 waves");
+    constexpr int MAXVT = REF_SUMS_MAXVT;
+    RefSumsLds& L = ref_sums_lds();
+    float* s_p4 = L.p4; float* s_p5 = L.p5; float* s_w4 = L.w4; float* s_w5 = L.w5;
+    double (*s_d)[16] = L.d;
+    const int tid = threadIdx.x;
+    int tbx = 16, tby = 32;
+    bool geom = even_cols && (bcols % 2 == 0);
+    if (brows * bcols > 1024) {
+        if (bcols < 32 || brows < 32) geom = false;
+    } else {
+        tbx = (int)(bcols / 2); tby = (int)brows;
+    }
+    const int nvt = tbx * tby;
+    if (nvt <= 0 || nvt % 32 != 0 || nvt > MAXVT) geom = false;
+    __syncthreads();                                   // earlier readers of the LDS arrays are done
+    if (!geom) {
+        double d4 = 0.0, d5 = 0.0;
+#pragma unroll 1
+        for (int i = tid; i < bh * bw; i += WGS) {
+            const int r = i / bw, c = i - r * bw;
+            float t4 = 0.0f, t5 = 0.0f;
+            err_terms_exact<EMU>(bf16_one(ld(r, c)), e8, s4, s5, t4, t5);
+            d4 += (double)t4; d5 += (double)t5;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) { d4 += __shfl_xor(d4, off); d5 += __shfl_xor(d5, off); }
+        if ((tid & 63) == 0) { s_d[0][tid >> 6] = d4; s_d[1][tid >> 6] = d5; }
+        __syncthreads();
+        d4 = 0.0; d5 = 0.0;
+#pragma unroll
+        for (int w = 0; w < WGS / 64; ++w) { d4 += s_d[0][w]; d5 += s_d[1][w]; }
+        e4 = (float)d4; e5 = (float)d5;
+        return;
+    }
+    const int pw = bw >> 1;                            // packed words per row of the valid part
+#pragma unroll 1
+    for (int vt = tid; vt < nvt; vt += WGS) {
+        const int ty = vt / tbx, tx = vt - ty * tbx;
+        float a4 = 0.0f, a5 = 0.0f;
+#pragma unroll 1
+        for (int r = ty; r < bh; r += tby)
+#pragma unroll 1
+            for (int pc = tx; pc < pw; pc += tbx) {
+                float h4 = 0.0f, h5 = 0.0f, l4 = 0.0f, l5 = 0.0f;
+                err_terms_exact<EMU>(bf16_one(ld(r, 2 * pc + 1)), e8, s4, s5, h4, h5);
+                err_terms_exact<EMU>(bf16_one(ld(r, 2 * pc)), e8, s4, s5, l4, l5);
+                a4 += (h4 + l4);
+                a5 += (h5 + l5);
+            }
+        s_p4[vt] = a4; s_p5[vt] = a5;
+    }
+    __syncthreads();
+    // the shuffle-down tree of every warp: in a step only lanes below `off` matter, and they read lanes they do not write
+#pragma unroll 1
+    for (int off = 16; off > 0; off >>= 1) {
+#pragma unroll 1
+        for (int vt = tid; vt < nvt; vt += WGS)
+            if ((vt & 31) < off) { s_p4[vt] += s_p4[vt + off]; s_p5[vt] += s_p5[vt + off]; }
+        __syncthreads();
+    }
+    // the warps' sums in the first warp's tree
+    if (tid < 32) {
+        const int nw = nvt >> 5;
+        s_w4[tid] = tid < nw ? s_p4[32 * tid] : 0.0f;
+        s_w5[tid] = tid < nw ? s_p5[32 * tid] : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll 1
+    for (int off = 16; off > 0; off >>= 1) {
+        if (tid < off) { s_w4[tid] += s_w4[tid + off]; s_w5[tid] += s_w5[tid + off]; }
+        __syncthreads();
+    }
+    e4 = s_w4[0]; e5 = s_w5[0];
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -197,8 +297,10 @@ __device__ __forceinline__ void for_block_elements(int64_t bh, int64_t bw, int64
 // generic_block: one workgroup quantizes one block of any shape straight from memory with the exact arithmetic.
 // It is the body of k_generic and the fallback of k_wgblock for blocks outside the fast range.  FAST (k_generic, default
 // flavour): blocks whose scale is in the fast range use the few-instruction arithmetic, with the same safeguard on
-// close MoR decisions as k_wgblock.
-template <bool EMU, bool FAST = false, int WGS = WG>
+// close MoR decisions as k_wgblock.  The exact MoR error sums are the reference's, addition by addition
+// (err_sums_reference_order).
+// MORP: whether the caller can be in MoR mode at all (a kernel that never is leaves the decision's code and LDS out).
+template <bool EMU, bool FAST = false, int WGS = WG, bool MORP = true>
 __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out, int32_t* meta, float* stats,
                                               const Shape& sh, const QuantArgs& qa, bool e8, int64_t bid,
                                               float (*s_f)[WGS / 64], uint32_t* s_u, bool allow_fast = false,
@@ -231,7 +333,7 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
     int fmt = qa.fmt;
     int meta_val = qa.meta_val;
     float e4 = 0.0f, e5 = 0.0f;
-    if (qa.qmode == 1) {
+    if constexpr (MORP) if (qa.qmode == 1) {
         int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
         if (qt == Q_UNKNOWN) {
             const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
@@ -248,20 +350,13 @@ __device__ __forceinline__ void generic_block(const uint16_t* in, uint16_t* out,
                     __syncthreads();
                     e4 = lds_sum<NW>(s_f[0]);
                     e5 = lds_sum<NW>(s_f[1]);
-                    exact = !(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5));       // too close: repeat with the reference's divisions
-                    if (exact) { e4 = 0.0f; e5 = 0.0f; }
+                    // too close to call (or asked for): the reference's divisions in the reference's order
+                    exact = qa.ref_sums || !(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5));
                 }
             }
-            if (exact) {
-                for_block_elements<WGS>(bh, bw, sh.cols, tid, [&](int64_t at) { err_terms_exact<EMU>(bf16_one(bin[at]), e8, s4, s5, e4, e5); });
-                e4 = wave_sum(e4);
-                e5 = wave_sum(e5);
-                __syncthreads();
-                if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
-                __syncthreads();
-                e4 = lds_sum<NW>(s_f[0]);
-                e5 = lds_sum<NW>(s_f[1]);
-            }
+            if (exact)
+                err_sums_reference_order<EMU, WGS>([&](int r, int c) { return bin[(int64_t)r * sh.cols + c]; },
+                                                   (int)bh, (int)bw, sh.brows, sh.bcols, sh.cols % 2 == 0, e8, s4, s5, e4, e5);
             qt = mor_decide_error(amax, qa.clamp, e4, e5);
         }
         meta_val = qt;

@@ -93,7 +93,7 @@ __global__ __launch_bounds__(WG) void k_subblock(const uint4* in, uint4* out, in
         e4 = group_sum(e4, L);
         e5 = group_sum(e5, L);
         if (want) {
-            if (!(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) hard = true;        // too close for the reciprocal-based sums
+            if (qa.ref_sums || !(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) hard = true;        // too close for the reciprocal-based sums (or the reference's order is asked for)
             else qt = mor_decide_error(amax, qa.clamp, e4, e5);
         }
         meta_val = qt;
@@ -148,8 +148,8 @@ __global__ __launch_bounds__(WG) void k_subblock(const uint4* in, uint4* out, in
     for (int g2 = 0; g2 < groups; ++g2) {
         if (!s_hard[g2]) continue;                 // uniform over the workgroup
         __syncthreads();
-        generic_block<false, false, WG>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
-                                        sh, qa, E8, bid0 + g2, s_f, s_u);
+        generic_block<false, false, WG, MOR>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
+                                             sh, qa, E8, bid0 + g2, s_f, s_u);
     }
 }
 
@@ -218,8 +218,8 @@ __global__ __launch_bounds__(BIG_WG) void k_bigblock(const uint4* in, uint4* out
     const Scale s4 = make_scale(448.0f / amax), s5 = make_scale(57344.0f / amax);
     // a NaN in the block, or a scale outside the range of the few-instruction arithmetic: the exact path
     if (amax_b > 0x7F800000u || (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast))) {           // uniform over the workgroup
-        generic_block<false, false, WGS>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
-                                         sh, qa, E8, bid, s_f, s_u);
+        generic_block<false, false, WGS, MOR>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
+                                              sh, qa, E8, bid, s_f, s_u);
         return;
     }
 
@@ -244,23 +244,13 @@ __global__ __launch_bounds__(BIG_WG) void k_bigblock(const uint4* in, uint4* out
             __syncthreads();
             e4 = lds_sum<NW>(s_f[0]);
             e5 = lds_sum<NW>(s_f[1]);
-            if (!(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) {
-                // too close for the reciprocal-based sums to be trusted with the decision: IEEE divisions (rare)
-                const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in);
-                const int64_t bh = rows_valid, bw = min(sh.bcols, sh.cols - c0);
-                e4 = 0.0f; e5 = 0.0f;
-#pragma unroll 1
-                for (int64_t i = tid; i < bh * bw; i += WGS) {
-                    int64_t r = i / bw, c = i - r * bw;
-                    err_terms_exact<false>(bf16_one(in16[(r0 + r) * sh.cols + c0 + c]), E8, s4, s5, e4, e5);
-                }
-                e4 = wave_sum(e4);
-                e5 = wave_sum(e5);
-                __syncthreads();
-                if (lane == 0) { s_f[0][wave] = e4; s_f[1][wave] = e5; }
-                __syncthreads();
-                e4 = lds_sum<NW>(s_f[0]);
-                e5 = lds_sum<NW>(s_f[1]);
+            if (qa.ref_sums || !(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) {
+                // too close for the reciprocal-based sums and this kernel's order of additions to be trusted with the
+                // decision (or asked for): the reference's divisions in the reference's order (rare)
+                const uint16_t* b16 = reinterpret_cast<const uint16_t*>(in) + (r0 * sh.cols + c0);
+                err_sums_reference_order<false, WGS>([&](int r, int c) { return b16[(int64_t)r * sh.cols + c]; },
+                                                     rows_valid, (int)min(sh.bcols, sh.cols - c0), sh.brows, sh.bcols, sh.cols % 2 == 0,
+                                                     E8, s4, s5, e4, e5);
             }
             qt = mor_decide_error(amax, qa.clamp, e4, e5);
         }

@@ -103,8 +103,11 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
         if (ok[k]) v[k] = load16<(NT == 1)>(bin + off[k]);
     }
     }
-    // the store of one result vector (GATHER: pair by pair along the same walk, which `put` is called in order of)
+    // the store of one result vector (GATHER: pair by pair along the same walk, which `put` is called in order of;
+    // DUAL: to `out` and to the LDS copy of the tile that out_t is written from -- both, unless the transposed tile
+    // decided on another format, see below)
     int g_r = tid / g_pr, g_cp = tid - g_r * g_pr;
+    bool to_out = true, to_lds = true;
     auto put = [&](int k, uint4 q) {
         if constexpr (GATHER) {
             uint16_t* dst = reinterpret_cast<uint16_t*>(out) + (r0 * sh.cols + c0);
@@ -119,9 +122,11 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
                 g_r += g_step_r; g_cp += g_step_c;
                 if (g_cp >= g_pr) { g_cp -= g_pr; ++g_r; }
             }
+        } else if constexpr (DUAL) {
+            if (to_out) store16<(NT != 0)>(bout + off[k], q);
+            if (to_lds) dual_tile_put(s_t, (k * WGS + tid) >> 4, tid & 15, q);
         } else {
             store16<(NT != 0)>(bout + off[k], q);
-            if constexpr (DUAL) dual_tile_put(s_t, (k * WGS + tid) >> 4, tid & 15, q);
         }
     };
     // DUAL: the tile in LDS -> out_t, a lane per 8 consecutive rows of one column; the tile's entry of meta_t
@@ -177,13 +182,13 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
     if (amax_b > 0x7F800000u || (amax > 0.0f && !(s4.e8 >= -90 && s4.e8 <= 90 && s4.fast))) {           // uniform over the workgroup
         if constexpr (WIRE) {
             // the exact path's decision and values; the tile is stored as their bf16 image
-            generic_block<false, false, WGS>(reinterpret_cast<const uint16_t*>(in), nullptr, meta, nullptr, sh, qa, E8, bid, s_f, s_u, false,
+            generic_block<false, false, WGS, MOR>(reinterpret_cast<const uint16_t*>(in), nullptr, meta, nullptr, sh, qa, E8, bid, s_f, s_u, false,
                                              reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(out) + (int64_t)bid * TILE_PAYLOAD_BYTES));
             if (tid == 0) { meta[bid] |= TILE_STORED_BF16; stats[bid] = 1.0f; }      // (thread 0 wrote the decision there)
             return;
         }
-        generic_block<false, false, WGS>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
-                             sh, qa, E8, bid, s_f, s_u);
+        generic_block<false, false, WGS, MOR>(reinterpret_cast<const uint16_t*>(in), reinterpret_cast<uint16_t*>(out), meta, stats,
+                                  sh, qa, E8, bid, s_f, s_u);
         if constexpr (DUAL) {
             // the tile as generic_block has just written it (this workgroup's own stores), through LDS to out_t
             __syncthreads();
@@ -200,6 +205,7 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
 
     int fmt = qa.fmt;
     int meta_val = qa.meta_val;
+    int qt_t = Q_UNKNOWN;                  // DUAL: the decision of the transposed tile where it has sums of its own
     float e4 = 0.0f, e5 = 0.0f;
     if constexpr (MOR) {
         int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
@@ -222,24 +228,23 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
             __syncthreads();
             e4 = lds_sum<NW>(s_e[0]);
             e5 = lds_sum<NW>(s_e[1]);
-            if (!(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) {
-                // The sums above divide with a Newton step.  When they are too close for that to be trusted with
-                // the decision, repeat them with IEEE divisions (from memory, non-unrolled: this is rare).
-                const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in);
-                const int64_t bh = min(sh.brows, sh.rows - r0), bw = min(sh.bcols, sh.cols - c0);
-                e4 = 0.0f; e5 = 0.0f;
+            if (qa.ref_sums || !(fabsf(e4 - e5) > 1e-5f * fmaxf(e4, e5))) {
+                // The sums above use reciprocals and this kernel's own order of additions.  When they are too close for
+                // that to be trusted with the decision (or the caller asks for it), they are replaced by the reference's:
+                // its divisions, its order of additions (from memory, non-unrolled: this is rare).  A tile and its
+                // transpose hold the same terms, but the reference adds them in another order on the transposed
+                // tensor: there the transposed tile gets sums, and a decision, of its own.
+                const uint16_t* b16 = reinterpret_cast<const uint16_t*>(in) + (r0 * sh.cols + c0);
+                const int bh = (int)min(sh.brows, sh.rows - r0), bw = (int)min(sh.bcols, sh.cols - c0);
 #pragma unroll 1
-                for (int64_t i = tid; i < bh * bw; i += WGS) {
-                    int64_t r = i / bw, c = i - r * bw;
-                    err_terms_exact<false>(bf16_one(in16[(r0 + r) * sh.cols + c0 + c]), E8, s4, s5, e4, e5);
+                for (int o = 0; o < (DUAL ? 2 : 1); ++o) {
+                    float t4, t5;
+                    err_sums_reference_order<false, WGS>([&](int r, int c) { return o ? b16[(int64_t)c * sh.cols + r] : b16[(int64_t)r * sh.cols + c]; },
+                                                         o ? bw : bh, o ? bh : bw, o ? sh.bcols : sh.brows, o ? sh.brows : sh.bcols,
+                                                         (o ? sh.rows : sh.cols) % 2 == 0, E8, s4, s5, t4, t5);
+                    if (o == 0) { e4 = t4; e5 = t5; }
+                    else qt_t = mor_decide_error(amax, qa.clamp, t4, t5);
                 }
-                e4 = wave_sum(e4);
-                e5 = wave_sum(e5);
-                __syncthreads();                 // every wave has read the first sums
-                if (lane == 0) { s_e[0][wave] = e4; s_e[1][wave] = e5; }
-                __syncthreads();
-                e4 = lds_sum<NW>(s_e[0]);
-                e5 = lds_sum<NW>(s_e[1]);
             }
             qt = mor_decide_error(amax, qa.clamp, e4, e5);
         }
@@ -349,6 +354,18 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
             break;
     }
     };
+    if constexpr (DUAL && MOR) {
+        if (qt_t != Q_UNKNOWN && mor_fmt_of(qt_t) != fmt) {
+            // the transposed tile decided on the other format (sums that agree to their last bits, added in two orders):
+            // the tile is quantized twice, for `out` and then for the LDS copy that out_t is written from
+            to_lds = false;
+            pass3();
+            __syncthreads();               // the readers of the first table are done
+            fmt = mor_fmt_of(qt_t);
+            meta_val = qt_t;
+            to_out = false; to_lds = true;
+        }
+    }
     pass3();
     write_transposed(meta_val);
 }

@@ -24,7 +24,8 @@ static void launch_wgblock_nv(bool full, int grid, const uint4* i4, uint4* o4, i
     // fewer tiles in flight keep the memory system on fewer DRAM pages at a time (8192^2 from HBM, MoR 128 x 128:
     // 49.4 -> 47.5 us; 16384 x 14336: 161 -> 156 us), while a grid that fits the chip at once wants every slot
     // (4096^2: 9.2 against 10.8 us).
-    const size_t dyn_lds = ((NV == 8 && WGS == WG) || (NV == 4 && WGS == 512)) && grid >= 4096 ? 53000 : 0;
+    // (the MoR kernels hold REF_SUMS_LDS_BYTES of static LDS for the reference-order sums)
+    const size_t dyn_lds = ((NV == 8 && WGS == WG) || (NV == 4 && WGS == 512)) && grid >= 4096 ? 53000 - (MOR ? REF_SUMS_LDS_BYTES : 0) : 0;
     // Consecutive workgroup ids go round the 8 XCDs.  In band order each XCD takes a band of gx / 8 block columns and
     // walks it row by row, so that the blocks sharing a DRAM page are in flight on one XCD at about the same time
     // (from HBM, 128 x 128 blocks: 8192^2 MoR 50.4 -> 47.5 us, 16384 x 14336 170 -> 156 us; a tensor that sits in the

@@ -380,6 +380,12 @@ static void block_error(const blk_t* b, float amax, int e8, int flavour, float* 
     *e5_o = block_tree_sum(p5, (int)nthreads);
 }
 
+/* The per-element terms of FQ:504-542 for n elements of a block whose amax is given (what block_error adds up):
+ * exported so that tests can construct blocks whose two sums meet. */
+void mor_oracle_mor_error_terms(const uint16_t* x, size_t n, float amax, int e8, int flavour, float* e4, float* e5) {
+    for (size_t i = 0; i < n; ++i) err_terms(mor_oracle_bf16_to_fp32(x[i]), amax, e8, flavour, &e4[i], &e5[i]);
+}
+
 /* MorQuantType, FQ:600-608 */
 enum { Q_UNKNOWN = 0, Q_E4M3 = 1, Q_E5M2 = 2, Q_BF16 = 3, Q_E2M3 = 4, Q_E4M3_SMALL = 11, Q_E5M2_SMALL = 12 };
 

@@ -50,6 +50,10 @@ float    mor_oracle_scaling_factor(float global_amax, float block_amax, int ss_m
 float    mor_oracle_e8m(float v, int mbits);                  /* FQ:1243-1327 */
 float    mor_oracle_e8mx_scaling_factor(float global_amax, int mbits, int strategy); /* FQ:1335-1359 */
 
+/* the two per-element terms |q / x - 1| of the MoR error sums (FQ:504-542) for n elements of a block with the
+ * given amax; e8: power-of-two scale */
+void mor_oracle_mor_error_terms(const uint16_t* x, size_t n, float amax, int e8, int flavour, float* e4, float* e5);
+
 /* vectorised scalar pieces */
 void mor_oracle_cast_sw_n(const float* in, float* out, size_t n, int fmt);
 void mor_oracle_cast_hw_n(const float* in, float* out, size_t n, int fmt);

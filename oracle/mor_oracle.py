@@ -43,6 +43,7 @@ def lib():
             "mor_oracle_scaling_factor": (f32, [f32, f32, C.c_int]),
             "mor_oracle_e8m": (f32, [f32, C.c_int]),
             "mor_oracle_e8mx_scaling_factor": (f32, [f32, C.c_int, C.c_int]),
+            "mor_oracle_mor_error_terms": (None, [vp, sz, f32, C.c_int, C.c_int, vp, vp]),
             "mor_oracle_cast_sw_n": (None, [vp, vp, sz, C.c_int]),
             "mor_oracle_cast_hw_n": (None, [vp, vp, sz, C.c_int]),
             "mor_oracle_fake_quantize": (C.c_int, [vp, vp, vp, i64, i64, i64, i64, f32, i64, i64, C.c_int, vp]),
@@ -95,6 +96,15 @@ def cast_hw(x, fmt):
     out = np.empty_like(x)
     lib().mor_oracle_cast_hw_n(_p(x), _p(out), x.size, fmt)
     return out
+
+
+def mor_error_terms(x_u16, amax, sf_type, flavour=KERNEL):
+    """The E4M3 and E5M2 terms |q / x - 1| of the MoR error sums for the elements x (bf16 bits) of a block with that amax."""
+    x = np.ascontiguousarray(x_u16, dtype=np.uint16).ravel()
+    e4 = np.empty(x.size, np.float32)
+    e5 = np.empty(x.size, np.float32)
+    lib().mor_oracle_mor_error_terms(_p(x), x.size, float(amax), int(sf_type == 2), flavour, _p(e4), _p(e5))
+    return e4, e5
 
 
 def fake_quantize(a, block_x, block_y, clamp_threshold, mode, sf_type, flavour=KERNEL, want_stats=False):

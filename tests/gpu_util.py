@@ -50,12 +50,12 @@ def block_format(a_u16, block_x, block_y, fmt, sf_type, flags=0):
     return to_host_u16(out)
 
 
-def mor_stats(a_u16, block_x, block_y, clamp, mode, sf_type):
+def mor_stats(a_u16, block_x, block_y, clamp, mode, sf_type, flags=0):
     L = _cabi.lib()
     rows, cols = a_u16.shape
     x = to_dev_u16(a_u16)
     st = torch.zeros((cdiv(rows, block_x), cdiv(cols, block_y), 4), dtype=torch.float32, device=dev())
-    _cabi.check(L.mor_mor_stats(x.data_ptr(), rows, cols, block_x, block_y, float(clamp), mode, sf_type, st.data_ptr(), stream_ptr()))
+    _cabi.check(L.mor_mor_stats(x.data_ptr(), rows, cols, block_x, block_y, float(clamp), mode, sf_type, st.data_ptr(), flags, stream_ptr()))
     torch.cuda.synchronize()
     return st.cpu().numpy()
 

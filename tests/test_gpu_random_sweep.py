@@ -6,6 +6,8 @@ import torch
 
 from oracle import mor_oracle as O
 
+IN_WINDOW = []          # scaling cases whose mean error is within 1e-5 (relative) of the threshold
+
 pytestmark = pytest.mark.gpu
 
 
@@ -124,11 +126,19 @@ def test_scaling_sweep(G, case):
     assert gamax[0] == wamax[0] and gnnz[0] == wnnz[0], case
     np.testing.assert_allclose(gerr[0], werr[0], rtol=1e-6, atol=0)
     avg = werr[0] / max(wnnz[0], 1)
-    if abs(avg - thr) > 1e-5 * thr:
+    if abs(avg - thr) <= 1e-5 * thr:          # the kernels' sum is not added in the reference's order: counted, none expected
+        IN_WINDOW.append(case)
+    else:
         assert meta[0] == wmeta[0], case
     if meta[0] == wmeta[0]:
         bad = np.argwhere(out != want)
         assert len(bad) == 0, (case, len(bad), tuple(bad[0]), hex(int(out[tuple(bad[0])])), hex(int(want[tuple(bad[0])])))
+
+
+def test_scaling_sweep_no_case_within_the_threshold_window():
+    """runs after the sweep above: the cases whose decision the order of the additions could have changed"""
+    print("scaling sweep cases inside the 1e-5 threshold window:", len(IN_WINDOW), flush=True)
+    assert not IN_WINDOW, IN_WINDOW
 
 
 def wire_cases():
@@ -209,6 +219,7 @@ def test_more_random_cases_on_request(G):
     bs_blocks = [(1, 32), (1, 256), (1, 2048), (1, 4096), (128, 128), (64, 64), (32, 16), (16, 120), (20, 12), (64, 1), (256, 1), (8, 1),
                  (8, 8), (128, 256), (512, 1)]
     bad = []
+    in_window = 0
     for i in range(n):
         data_rng = np.random.default_rng(seed0 * 100003 + i)
         kind = int(rng.integers(4))
@@ -220,11 +231,8 @@ def test_more_random_cases_on_request(G):
             a = make_data(data_rng, rows, cols, kind)
             out, meta = G.fake_quantize(a, br, bc, clamp, mode, sf)
             want, wmeta, stats = O.fake_quantize(a, br, bc, clamp, mode, sf, want_stats=True)
-            flips = meta != wmeta
-            if flips.any():
-                e4, e5 = stats[..., 2][flips], stats[..., 3][flips]
-                if not (np.abs(e4 - e5) <= 1e-6 * np.maximum(e4, e5)).all():
-                    bad.append(("decision", i, rows, cols, br, bc, mode, sf, kind))
+            if (meta != wmeta).any():            # (close sums are added in the reference's order: no decision may differ)
+                bad.append(("decision", i, rows, cols, br, bc, mode, sf, kind))
             elif not np.array_equal(out, want):
                 bad.append(("values", i, rows, cols, br, bc, mode, sf, kind))
         else:
@@ -238,10 +246,11 @@ def test_more_random_cases_on_request(G):
             case = ("scaling", i, rows, cols, br, bc, ss, kind % 3, inplace, thr)
             if gamax[0] != wamax[0] or gnnz[0] != wnnz[0] or abs(float(gerr[0]) - float(werr[0])) > 2e-6 * abs(float(werr[0])):
                 bad.append(case)
+            elif abs(werr[0] / max(wnnz[0], 1) - thr) <= 1e-5 * thr:
+                in_window += 1
             elif meta[0] != wmeta[0]:
-                if abs(werr[0] / max(wnnz[0], 1) - thr) > 1e-5 * thr:
-                    bad.append(case)
+                bad.append(case)
             elif not np.array_equal(out, want):
                 bad.append(case)
-    print("extra random cases:", n, "seed", seed0, "disagreements:", len(bad), flush=True)
+    print("extra random cases:", n, "seed", seed0, "disagreements:", len(bad), "scaling cases inside the 1e-5 threshold window:", in_window, flush=True)
     assert not bad, bad[:10]

@@ -38,6 +38,9 @@ def reference_chain(shape, br, bc, channel):
     return max(per_block, -(-nb // 1024))
 
 
+IN_WINDOW = []          # cases whose mean error is within 1e-5 (relative) of the threshold
+
+
 def check_scaling(G, a, br, bc, thr, ss, channel, flags=0, inplace=False):
     print("scaling", a.shape, br, bc, thr, ss, channel, flags, inplace, flush=True)
     out, meta, gamax, gnnz, gerr = G.block_scaling(a, br, bc, thr, ss, channel=channel, flags=flags, inplace=inplace)
@@ -48,8 +51,13 @@ def check_scaling(G, a, br, bc, thr, ss, channel, flags=0, inplace=False):
     if not flags & 1:
         np.testing.assert_allclose(gerr[0], O.last_exact_error(), rtol=1e-6, atol=0)
     np.testing.assert_allclose(gerr[0], werr[0], rtol=max(1e-6, reference_chain(a.shape, br, bc, channel) * 2.0 ** -24), atol=0)
+    # The bf16 fallback compares sum / count with the threshold (fake_quantize.cu:1214).  The kernels' sum is within
+    # 1e-6 of the reference's but not added in its order, so a mean within 1e-5 of the threshold could fall on the other
+    # side; such cases are counted (IN_WINDOW) and the test at the end of this file expects none.
     avg = werr[0] / max(wnnz[0], 1)
-    if abs(avg - thr) > 1e-5 * thr:                                        # decision not within the tolerance of the sum
+    if abs(avg - thr) <= 1e-5 * thr:
+        IN_WINDOW.append((a.shape, br, bc, thr, ss, channel, flags, inplace))
+    else:
         assert meta[0] == wmeta[0]
     if meta[0] == wmeta[0]:
         bad = np.argwhere(out != want)
@@ -281,3 +289,9 @@ def test_scaling_denormal_elements(G, ss, shape):
     a[pick] = (a[pick] & 0x8000) | rng.integers(1, 0x100, int(pick.sum())).astype(np.uint16)     # 2^-133 .. 2^-125
     check_scaling(G, a, br, bc, 0.045, ss, channel)
     check_scaling(G, a, br, bc, 0.2, ss, channel, inplace=True)
+
+
+def test_zz_no_case_was_within_the_threshold_window():
+    """runs last in this file: how many of the cases above had a mean error within 1e-5 of the threshold"""
+    print("scaling cases inside the 1e-5 threshold window:", len(IN_WINDOW), flush=True)
+    assert not IN_WINDOW, IN_WINDOW
