@@ -54,6 +54,10 @@ extern "C" {
 #define MOR_FMT_E5M2 1
 #define MOR_FMT_E3M2 2
 #define MOR_FMT_E2M3 3
+/* mor_block_format only: no quantization.  The kernel that would quantize blocks of this shape reads every block,
+ * finds its amax and writes the block back unchanged: what the memory system gives that kernel's access pattern
+ * (a measurement aid; blocks of one row and up to 2048 elements go through the general block kernels for it). */
+#define MOR_FMT_COPY (-1)
 
 /* op ids for mor_workspace_bytes */
 #define MOR_OP_FAKE_QUANTIZE 0
@@ -258,8 +262,10 @@ MOR_API int mor_fake_quantize_dual(const void* input, void* output_rows, int32_t
  * A tile and its transpose hold the same elements, so they share amax, scale and format: the tile is
  * quantized once and stored twice.  (MoR compares two fp32 error sums; the call on x^T adds the same
  * terms in another order, so a tile whose two sums agree to the last bits could come out in the other
- * format there.  The decision taken here is that of the call on x.)
- * rows and cols multiples of 128; three different 16-byte aligned tensors.
+ * format there: for tiles whose sums are that close both are added again in the reference's two
+ * orders, and each orientation gets the decision, and the values, of its own call.  The one exception
+ * is a tile whose scale is outside 2^+-90: there the decision of the call on x stands for both.)
+ * rows and cols multiples of 128 and below 2^27; three different 16-byte aligned tensors.
  */
 MOR_API int mor_fake_quantize_dual_tiles(const void* input, void* output, int32_t* meta, void* output_t,
                                          int32_t* meta_t, int64_t rows, int64_t cols, double clamp_threshold,
@@ -285,7 +291,8 @@ MOR_API int mor_fake_quantize_dual_tiles(const void* input, void* output, int32_
  * divided by the scale (IEEE), rounded to bf16 half-up (FQ:312-316).
  * mode % 10: 1 (MoR), or 2 / 3: every tile E4M3 / E5M2 with its own fp32 scale (block scaling in 128 x 128
  * tiles: tags 1 / 2); mode / 100 as in mor_fake_quantize; default flavour, fp32 scales.
- * rows and cols multiples of 128; tensor and payload 16-byte aligned, different buffers.
+ * rows and cols multiples of 128 and below 2^27, at most 2^30 tiles; tensor and payload 16-byte aligned,
+ * different buffers.
  */
 #define MOR_TILE_PAYLOAD_BYTES 32768
 #define MOR_TILE_STORED_BF16 0x100
@@ -299,8 +306,10 @@ MOR_API int mor_mor_dequantize(const void* payload, const int32_t* tags, const f
  * reference, whose callers quantize x.t().contiguous() in a call of its own): tile (i, j) of
  * [tile_rows, tile_cols] tiles becomes tile (j, i) of [tile_cols, tile_rows] tiles with its codes
  * transposed; tags and scales move with it (a tile and its transpose hold the same elements, so they
- * share format and scale).  mor_mor_dequantize of the result is the transpose of mor_mor_dequantize of
- * the source, bit for bit.  Source and destination are different buffers; payloads 16-byte aligned.
+ * share format and scale; only for a MoR tile whose two error sums agree to their last bits can
+ * mor_mor_quantize of the transposed tensor, which adds them in another order, choose the other format).
+ * mor_mor_dequantize of the result is the transpose of mor_mor_dequantize of the source, bit for bit.  Source and destination are different buffers; payloads 16-byte aligned;
+ * tile_rows and tile_cols at most 2^20, their product at most 2^30.
  */
 MOR_API int mor_mor_transpose(const void* payload, const int32_t* tags, const float* scales, void* payload_t,
                               int32_t* tags_t, float* scales_t, int64_t tile_rows, int64_t tile_cols, void* stream);

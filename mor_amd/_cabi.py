@@ -13,6 +13,7 @@ FLAG_TORCH_EMULATION = 1
 FLAG_SOFTWARE_CAST = 2
 FLAG_REFERENCE_ORDER_SUMS = 4
 FMT_E4M3, FMT_E5M2, FMT_E3M2, FMT_E2M3 = 0, 1, 2, 3
+FMT_COPY = -1          # mor_block_format only: the block kernels' access pattern without the arithmetic
 OP_FAKE_QUANTIZE, OP_BLOCK_SCALING, OP_CHANNEL_SCALING, OP_E8MX = 0, 1, 2, 3
 
 _vp, _i64, _i32p, _f64, _u32, _int, _sz = C.c_void_p, C.c_int64, C.c_void_p, C.c_double, C.c_uint32, C.c_int, C.c_size_t

@@ -186,7 +186,10 @@ extern "C" int mor_fake_quantize_batch(const MorTensorDesc* descs, int64_t n, ui
         const int64_t nblocks = cdiv(d.rows, d.block_rows) * cdiv(d.cols, d.block_cols);
         if (d.rows * d.cols > BATCH_SMALL || nblocks > (1 << 16)) {
             QuantArgs tq;
-            const int64_t nch = (d.block_cols % 8 == 0) ? d.block_rows * (d.block_cols / 8) : 0;     // 16-byte chunks per block
+            // 16-byte chunks per block (block dims beyond the tensor's, which may be anything, never make whole blocks:
+            // left out before the product, which they could overflow)
+            const bool dims_ok = d.block_rows <= d.rows && d.block_cols <= d.cols;
+            const int64_t nch = (dims_ok && d.block_cols % 8 == 0) ? d.block_rows * (d.block_cols / 8) : 0;
             const int64_t cpr = d.block_cols / 8;
             bool blocks = fast_ok && (nch == WG || nch == 2 * WG || nch == 4 * WG || nch == 8 * WG)
                           && d.rows % d.block_rows == 0 && d.cols % d.block_cols == 0 && (d.block_rows == 1 || is_pow2(cpr))

@@ -376,9 +376,10 @@ int mor_validate_shape(const void* input, int64_t rows, int64_t cols, int64_t br
     if (!input) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "input is NULL");
     if (rows <= 0 || cols <= 0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "rows and cols must be positive (got %lld x %lld)", (long long)rows, (long long)cols);
     if (brows <= 0 || bcols <= 0) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "block dims must be positive (got %lld x %lld)", (long long)brows, (long long)bcols);
-    if (cdiv(rows, brows) * cdiv(cols, bcols) > 0x7FFFFFFFll) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many blocks");
     // 2^35 elements (64 GiB of bf16): the flat kernels' grids, one workgroup per 512 vectors, stay below 2^24 workgroups
+    // (checked first: with rows * cols bounded, the block count below cannot overflow)
     if (rows > MOR_MAX_ELEMENTS / cols) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor too large (more than 2^35 elements)");
+    if (cdiv(rows, brows) * cdiv(cols, bcols) > 0x7FFFFFFFll) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many blocks");
     return MOR_OK;
 }
 
@@ -461,7 +462,7 @@ static int run_quantize(const void* input, void* output, int32_t* meta, float* s
     const bool vec_ok = fast_ok && aligned16(input) && (!output || aligned16(output)) && cols % 8 == 0 && bcols % 8 == 0
                         && brows * (cols / 8) < 0x7FFFFFFFll;
     const int64_t G = bcols / 8;
-    if (qa.qmode == 2 && !stats && output && vec_ok && brows == 1 && cols % bcols == 0 && is_pow2(G) && G <= 256) {
+    if (qa.qmode == 2 && qa.fmt >= 0 && !stats && output && vec_ok && brows == 1 && cols % bcols == 0 && is_pow2(G) && G <= 256) {
         if (e8) launch_rowgroup<true>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
         else launch_rowgroup<false>(qa.fmt, input, output, meta, rows * cols / 8, (int)G, meta ? qa.meta_val : -1, st);
         return mor_check_launch("k_rowgroup");
@@ -535,7 +536,7 @@ extern "C" int mor_block_format(const void* input, void* output,
                                 int fmt, int64_t sf_type, uint32_t flags, void* stream) {
     if (int rc = mor_validate_shape(input, rows, cols, brows, bcols)) return rc;
     if (!output) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "output is NULL");
-    if (fmt < 0 || fmt > 3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "unknown format %d", fmt);
+    if (fmt < MOR_FMT_COPY || fmt > 3) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "unknown format %d", fmt);
     QuantArgs qa{};
     qa.qmode = 2; qa.fmt = fmt; qa.meta_val = -1;
     return run_quantize(input, output, nullptr, nullptr, rows, cols, brows, bcols, qa, sf_type == 2, flags, static_cast<hipStream_t>(stream));

@@ -199,8 +199,9 @@ static int check_tiles(const void* a, const void* b, const void* tags, const voi
     if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u)
         return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor and payload must be 16-byte aligned");
     if (a == b) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "tensor and payload must be different buffers");
-    if (cols >= ((int64_t)1 << 27))                  // (a tile row's chunk offsets are 32-bit)
-        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "more than 2^27 columns (%lld)", (long long)cols);
+    // (a tile row's chunk offsets are 32-bit; mor_mor_transpose takes tile grids of up to 2^20 x 2^20 and 2^30 tiles)
+    if (cols >= ((int64_t)1 << 27) || rows >= ((int64_t)1 << 27) || (rows / 128) * (cols / 128) > ((int64_t)1 << 30))
+        return mor_fail(MOR_ERR_INVALID_ARGUMENT, "more than 2^27 rows or columns, or more than 2^30 tiles (%lld x %lld)", (long long)rows, (long long)cols);
     return MOR_OK;
 }
 

@@ -191,7 +191,8 @@ __global__ __launch_bounds__(WG) void k_bs_amax_sub(const uint4* in, uint32_t* w
 }
 
 
-// pass 1, column blocks N x 1 (FQ:1538-1610): a workgroup covers 256 adjacent columns (32 groups of 8) with 8 row
+// pass 1, column blocks N x 1 (FQ:1538-1610) for the tensors k_bs_colmax does not take (other flavour, power-of-two
+// scale, unaligned rows): a workgroup covers 256 adjacent columns (32 groups of 8) with 8 row
 // lanes; a thread takes every 8th row of a row segment, the 8 row lanes meet in LDS and one thread per column merges
 // into the (zero-initialised) per-block maxima with atomicMax on the bit patterns of non-negative floats.
 __global__ __launch_bounds__(WG) void k_bs_amax_col(const uint16_t* in, uint32_t* ws, float* block_amax, Shape sh,
@@ -200,12 +201,13 @@ __global__ __launch_bounds__(WG) void k_bs_amax_col(const uint16_t* in, uint32_t
     __shared__ float s_f[WAVES];
     __shared__ int s_i[WAVES];
     const int cg = threadIdx.x & 31, rl = threadIdx.x >> 5;
-    const int64_t col0 = ((int64_t)blockIdx.x * 32 + cg) * 8;
     const int64_t segs_per_block = (sh.brows + rows_per_wg - 1) / rows_per_wg;
-    const int ncol = (int)max((int64_t)0, min((int64_t)8, sh.cols - col0));
     float gmax = 0.0f;
     int nnz = 0;
-    // row segments of all block rows, taken grid-stride along y
+    // groups of 256 columns grid-stride along x, row segments of all block rows grid-stride along y
+    for (int64_t bx = blockIdx.x; bx * 256 < sh.cols; bx += gridDim.x) {
+    const int64_t col0 = (bx * 32 + cg) * 8;
+    const int ncol = (int)max((int64_t)0, min((int64_t)8, sh.cols - col0));
     for (int64_t seg = blockIdx.y; seg < sh.gy * segs_per_block; seg += gridDim.y) {
         const int64_t by = seg / segs_per_block;
         const int64_t r_begin = by * sh.brows + (seg - by * segs_per_block) * rows_per_wg;
@@ -241,9 +243,10 @@ __global__ __launch_bounds__(WG) void k_bs_amax_col(const uint16_t* in, uint32_t
         float cm = s_m[0][threadIdx.x];
 #pragma unroll
         for (int k = 1; k < 8; ++k) cm = fmaxf(cm, s_m[k][threadIdx.x]);
-        const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        const int64_t c = bx * 256 + threadIdx.x;
         if (c < sh.cols && cm > 0.0f) atomicMax(reinterpret_cast<uint32_t*>(&block_amax[by * sh.cols + c]), f2u(cm));
         gmax = fmaxf(gmax, cm);
+    }
     }
     const uint32_t slot = blockIdx.x + gridDim.x * blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -254,6 +257,207 @@ __global__ __launch_bounds__(WG) void k_bs_amax_col(const uint16_t* in, uint32_t
     if (threadIdx.x == 0) {
         reinterpret_cast<float*>(ws)[WS_PAMAX + slot] = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
         reinterpret_cast<int*>(ws)[WS_PNNZ + slot] = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    }
+}
+
+// Column blocks N x 1 with aligned rows, default flavour, fp32 scale: three kernels and the plan they share.
+//   k_bs_colmax   reads the tensor in the order it lies in memory (a workgroup owns whole rows, or NG * 4 KiB of each
+//                 of its rows): every lane meets the same few column groups again and again and keeps their packed
+//                 16-bit maxima; a block's rows are cut into P segments, one row of partial maxima per segment (bf16
+//                 bits, no atomics, nothing to clear);
+//   k_bs_colfold  folds the P partial rows of every block and column and leaves the column's scale and its reciprocal;
+//   k_bs_quant_col quantizes, a lane holding 8 rows of its 8 columns, strips as wide as a row allows.
+// W = lanes a row (or a slab of it) is wide in pass 1: min(256, column groups), a power of two; a row of more than 256
+// groups is NG * 256 groups (or slabs of that width).  Tensors whose group count fits neither form take the general
+// kernels.
+constexpr int COL_PASS1_WGS = 512;
+struct ColPlan {
+    int w_log;                  // pass 1: log2 of the lanes per row sweep (256 groups and more: 8)
+    int ng;                     // pass 1: column groups per lane (1 when a sweep holds one or several whole rows)
+    int64_t slabs;              // pass 1: slabs of ng * 256 groups a row is cut into
+    int r1, P;                  // pass 1: rows per batch, workgroups (and partial rows) per block and slab
+    int64_t items1;             // (slab, block row, segment) triples, slabs fastest
+    int cg_log;                 // pass 2: log2 of the lanes a strip is wide
+    int64_t strips, items2;     // pass 2: strips per row; (strip, block row, workgroup) triples
+    int Q;                      // pass 2: workgroups per block and strip
+};
+static bool col_plan(int64_t rows, int64_t cols, int64_t brows, ColPlan& p) {
+    p = ColPlan{};
+    if (cols % 8 != 0 || brows <= 0 || rows % brows != 0) return false;
+    const int64_t groups = cols / 8, gyb = rows / brows;
+    if (groups <= WG) {
+        if (!is_pow2(groups)) return false;
+        p.w_log = ilog2(groups); p.ng = 1; p.slabs = 1;
+    } else {
+        if (groups % WG != 0) return false;
+        const int64_t q = groups / WG;
+        p.w_log = 8;
+        p.ng = 1;
+        for (int g = 8; g >= 1; --g) if (q % g == 0) { p.ng = g; break; }
+        p.slabs = q / p.ng;
+    }
+    // pass 1: a block's rows in batches of whole sweeps (8 loads in flight per lane where the rows allow), dealt out in
+    // turn to the P workgroups of the block and slab; about COL_PASS1_WGS workgroups (more read no faster and leave more
+    // partial rows to fold: 16384 x 14336 takes 76 + 10 us with 512, 90 + 17 us with 1024), never more than PASS1_MAX (each
+    // publishes a partial of the tensor amax and of the non-zero count)
+    const int64_t rows_per_sweep = (int64_t)WG >> p.w_log;                 // (1 for 256 groups and more)
+    p.r1 = (int)(rows_per_sweep * (p.ng >= 6 ? 1 : p.ng >= 3 ? 2 : 8 / p.ng));          // rows of a batch (UN sweeps of k_bs_colmax)
+    const int64_t nb1 = cdiv(brows, p.r1);
+    p.P = (int)std::max<int64_t>(1, std::min<int64_t>(nb1, COL_PASS1_WGS / std::max<int64_t>(1, gyb * p.slabs)));
+    p.items1 = p.slabs * gyb * p.P;
+    // pass 2: strips of up to 256 lanes; a block's rows in batches of 4 per row lane, dealt out in turn to the Q workgroups
+    // of the block and strip; about PASS2_MAX workgroups (each publishes a partial of the error sum)
+    p.cg_log = (int)std::min<int64_t>(8, ilog2(groups + 1) - 1);          // floor(log2(groups))
+    p.strips = cdiv(groups, (int64_t)1 << p.cg_log);
+    const int64_t nb2 = cdiv(brows, 4 * ((int64_t)WG >> p.cg_log));
+    p.Q = (int)std::max<int64_t>(1, std::min<int64_t>(cdiv(nb2, 2), PASS2_MAX / std::max<int64_t>(1, gyb * p.strips)));
+    p.items2 = p.strips * gyb * p.Q;
+    return true;
+}
+// 32-bit words of the workspace this path takes behind the header: the partial maxima ([block row][segment][column]
+// 16-bit) and the columns' scales ([block row][column] pairs of floats)
+static int64_t col_words(int64_t rows, int64_t cols, int64_t brows) {
+    ColPlan p;
+    if (!col_plan(rows, cols, brows, p)) return 0;
+    return (rows / brows) * cols * 2 + (rows / brows) * p.P * cols / 2;
+}
+
+// a packed word with the halves that hold a NaN set to +0
+__device__ __forceinline__ uint32_t drop_nan_pk(uint32_t w) {
+    const uint32_t lo = ((w & 0x7FFFu) > 0x7F80u) ? 0u : (w & 0xFFFFu), hi = ((w & 0x7FFF0000u) > 0x7F800000u) ? 0u : (w & 0xFFFF0000u);
+    return lo | hi;
+}
+// pass 1 (FQ:1538-1610 without the atomics).  item = (slab, block row, workgroup of the P that share them), slabs fastest.
+template <int NG>
+__global__ __launch_bounds__(WG) void k_bs_colmax(const uint4* in, uint32_t* ws, uint16_t* partial, Shape sh, ColPlan p) {
+    __shared__ uint4 s_m[WG];
+    __shared__ float s_f[WAVES];
+    __shared__ int s_i[WAVES];
+    constexpr int UN = NG >= 6 ? 1 : NG >= 3 ? 2 : 8 / NG;               // sweeps of a batch: NG * UN = 6 to 8 loads in flight per lane
+    const int tid = threadIdx.x, W = 1 << p.w_log, cl = tid & (W - 1), rsub = tid >> p.w_log, rps = WG >> p.w_log;
+    const int64_t row_stride = sh.cols >> 3, groups = row_stride;
+    const bool nt = streams_in(sh.rows * sh.cols);
+    uint32_t gmax2 = 0;
+    int nnz = 0;
+    for (int64_t item = blockIdx.x; item < p.items1; item += gridDim.x) {
+        const int64_t seg = item / p.slabs, slab = item - seg * p.slabs;
+        const int64_t by = seg / p.P, sg = seg - by * p.P;
+        // the block's batches sg, sg + P, ...: workgroups that run side by side read neighbouring rows
+        const int64_t b_rows = by * sh.brows, r_end = (by + 1) * sh.brows, step = p.r1, stride = step * p.P;
+        const int64_t r_first = b_rows + sg * step + rsub;
+        const uint4* col = in + (slab * NG * WG + cl);                    // this lane's first column group
+        uint32_t m[NG][4];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) { m[g][0] = 0; m[g][1] = 0; m[g][2] = 0; m[g][3] = 0; }
+#pragma unroll 1
+        for (int64_t r = r_first; r < r_end; r += stride) {
+            uint4 v[UN][NG];
+#pragma unroll
+            for (int u = 0; u < UN; ++u)
+#pragma unroll
+                for (int g = 0; g < NG; ++g) {
+                    v[u][g] = make_uint4(0, 0, 0, 0);
+                    if (r + u * rps < r_end) v[u][g] = load16_rt(col + (r + u * rps) * row_stride + g * WG, nt);
+                }
+            // the batch's maxima and count; a NaN wins a packed maximum and counts as non-zero where the reference's float
+            // maximum and its count (FQ:998-999) skip it: a batch that holds one is folded again with its NaNs set to zero
+            uint32_t t[NG][4], nz2 = 0;
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                t[g][0] = 0; t[g][1] = 0; t[g][2] = 0; t[g][3] = 0;
+#pragma unroll
+                for (int u = 0; u < UN; ++u) {
+                    acc_amax_pk(t[g][0], v[u][g].x); acc_amax_pk(t[g][1], v[u][g].y); acc_amax_pk(t[g][2], v[u][g].z); acc_amax_pk(t[g][3], v[u][g].w);
+                    acc_nnz_pk(nz2, v[u][g].x); acc_nnz_pk(nz2, v[u][g].y); acc_nnz_pk(nz2, v[u][g].z); acc_nnz_pk(nz2, v[u][g].w);
+                }
+            }
+            uint32_t any = 0;
+#pragma unroll
+            for (int g = 0; g < NG; ++g) any = pk_max_u16(any, pk_max_u16(pk_max_u16(t[g][0], t[g][1]), pk_max_u16(t[g][2], t[g][3])));
+            if (amax_bits_of(any) > 0x7F800000u) {          // (rare)
+                nz2 = 0;
+#pragma unroll
+                for (int g = 0; g < NG; ++g) {
+                    t[g][0] = 0; t[g][1] = 0; t[g][2] = 0; t[g][3] = 0;
+#pragma unroll
+                    for (int u = 0; u < UN; ++u) {
+                        const uint32_t w[4] = {drop_nan_pk(v[u][g].x), drop_nan_pk(v[u][g].y), drop_nan_pk(v[u][g].z), drop_nan_pk(v[u][g].w)};
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) { acc_amax_pk(t[g][j], w[j]); acc_nnz_pk(nz2, w[j]); }
+                    }
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                m[g][0] = pk_max_u16(m[g][0], t[g][0]); m[g][1] = pk_max_u16(m[g][1], t[g][1]);
+                m[g][2] = pk_max_u16(m[g][2], t[g][2]); m[g][3] = pk_max_u16(m[g][3], t[g][3]);
+            }
+            nnz += (int)((nz2 & 0xFFFFu) + (nz2 >> 16));          // (at most 8 * UN * NG <= 128 per batch: the 16-bit counts cannot wrap)
+        }
+        // several rows per sweep (fewer than 256 groups): the lanes of one column group meet in LDS
+        if (rps > 1) {
+            __syncthreads();                       // the previous item's readers are done
+            s_m[tid] = make_uint4(m[0][0], m[0][1], m[0][2], m[0][3]);
+            __syncthreads();
+            if (rsub == 0) {
+#pragma unroll 1
+                for (int k = 1; k < rps; ++k) {
+                    const uint4 o = s_m[(k << p.w_log) + cl];
+                    m[0][0] = pk_max_u16(m[0][0], o.x); m[0][1] = pk_max_u16(m[0][1], o.y); m[0][2] = pk_max_u16(m[0][2], o.z); m[0][3] = pk_max_u16(m[0][3], o.w);
+                }
+            }
+        }
+        if (rsub == 0) {
+            uint4* prow = reinterpret_cast<uint4*>(partial) + (seg * groups + slab * NG * WG + cl);
+#pragma unroll
+            for (int g = 0; g < NG; ++g) prow[g * WG] = make_uint4(m[g][0], m[g][1], m[g][2], m[g][3]);
+        }
+#pragma unroll
+        for (int g = 0; g < NG; ++g) gmax2 = pk_max_u16(gmax2, pk_max_u16(pk_max_u16(m[g][0], m[g][1]), pk_max_u16(m[g][2], m[g][3])));
+    }
+    publish_partial(ws, u2f(amax_bits_of(gmax2)), nnz, s_f, s_i);
+}
+
+__device__ __forceinline__ float scaling_factor(float global_amax, float block_amax, int ss_mode);
+
+// pass 1b: for every block row and column the maximum over the P partial rows, turned into the column's scale and its
+// reciprocal (0 for a scale outside the fast range).  A workgroup takes 8 column groups (64 columns, whole cache lines of the partial rows) of one block row,
+// 32 lanes of partial rows each: the 8 of a wave meet by shuffles, the waves in LDS.
+constexpr int FOLD_G = 8;
+__global__ __launch_bounds__(WG) void k_bs_colfold(const uint16_t* partial, float2* scales, uint32_t* ws, int npart1, int ss_mode,
+                                                   Shape sh, ColPlan p) {
+    __shared__ float s_f[WAVES];
+    __shared__ uint4 s_m[WAVES][FOLD_G];
+    const float gamax = reduce_partial_amax(ws, npart1, s_f);
+    const int tid = threadIdx.x, c = tid & (FOLD_G - 1), pl = tid / FOLD_G, lane = tid & 63, wave = tid >> 6;
+    const int64_t groups = sh.cols >> 3, gw = (groups + FOLD_G - 1) / FOLD_G;
+    const int64_t by = blockIdx.x / gw, cg0 = (blockIdx.x - by * gw) * FOLD_G, cg = cg0 + c;
+    const uint4* prow = reinterpret_cast<const uint4*>(partial) + by * p.P * groups;
+    uint32_t m[4] = {0, 0, 0, 0};
+    if (cg < groups) {
+#pragma unroll 8
+        for (int k = pl; k < p.P; k += WG / FOLD_G) {
+            const uint4 o = prow[k * groups + cg];
+            m[0] = pk_max_u16(m[0], o.x); m[1] = pk_max_u16(m[1], o.y); m[2] = pk_max_u16(m[2], o.z); m[3] = pk_max_u16(m[3], o.w);
+        }
+    }
+#pragma unroll
+    for (int off = FOLD_G; off < 64; off <<= 1)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) m[j] = pk_max_u16(m[j], (uint32_t)__shfl_xor((int)m[j], off));
+    if (lane < FOLD_G) s_m[wave][lane] = make_uint4(m[0], m[1], m[2], m[3]);
+    __syncthreads();
+    if (tid < 8 * FOLD_G) {                    // one thread per column
+        const int g = tid >> 3, j = tid & 7;
+        uint32_t mb = 0;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) mb = max(mb, (uint32_t)reinterpret_cast<const uint16_t*>(&s_m[w][g])[j]);
+        const float amax = u2f(mb << 16);
+        Scale sc = make_scale(scaling_factor(gamax, amax, ss_mode));
+        // a column of zeros (FQ:1063-1064: its scale is 448 / 1e-35, outside the fast range) gives +0 with any scale
+        if (!(amax > 0.0f)) { sc.s = 1.0f; sc.r = 1.0f; sc.fast = true; }
+        const int64_t col = (cg0 + g) * 8 + j;
+        if (col < sh.cols) scales[by * sh.cols + col] = make_float2(sc.s, sc.fast ? sc.r : 0.0f);
     }
 }
 
@@ -466,26 +670,36 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
     }
 }
 
-// One vector of 8 adjacent columns, each with the scale of its own column block (all in the fast range): the
-// arithmetic of bs_pair_fast with a scale per half of a word; a vector that holds a NaN takes the exact arithmetic.
+// One vector of 8 adjacent columns, each with the scale cs[j] of its own column block and its reciprocal cr[j] (all in
+// the fast range): the arithmetic of bs_pair_fast with a scale per half of a word; a vector that holds a NaN takes the
+// exact arithmetic.
+__device__ __forceinline__ Scale scale_only(float s) {
+    Scale sc;
+    sc.s = s; sc.r = 0.0f; sc.e8 = 0; sc.fast = false;
+    return sc;
+}
+// the same vector with the exact arithmetic (a scale outside the fast range, a NaN)
+__device__ __forceinline__ uint4 bs_cols_vec_exact(uint4 v, const float (&cs)[8], float& err) {
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float q0 = bs_element<false, false>(bf16_lo(w[j]), scale_only(cs[2 * j]), err);
+        float q1 = bs_element<false, false>(bf16_hi(w[j]), scale_only(cs[2 * j + 1]), err);
+        w[j] = store_pair<false>(q0, q1);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
 template <bool WRITE, bool ERR>
-__device__ __forceinline__ uint4 bs_cols_vec_fast(uint4 v, const Scale (&sc)[8], float& err) {
+__device__ __forceinline__ uint4 bs_cols_vec_fast(uint4 v, const float (&cs)[8], const float (&cr)[8], float& err) {
+    if (vec_has_nan(v)) return bs_cols_vec_exact(v, cs, err);          // (rare)
     uint32_t w[4] = {v.x, v.y, v.z, v.w};
     float row_err = 0.0f;
-    if (vec_has_nan(v)) {          // (rare)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float q0 = bs_element<false, false>(bf16_lo(w[j]), sc[2 * j], row_err);
-            float q1 = bs_element<false, false>(bf16_hi(w[j]), sc[2 * j + 1], row_err);
-            w[j] = store_pair<false>(q0, q1);
-        }
-    } else
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const float a = fabsf(bf16_lo(w[j])), b = fabsf(bf16_hi(w[j]));
-        const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc[2 * j].s, b * sc[2 * j + 1].s));
-        const float qa = div_by_scale(c.x, sc[2 * j].s, sc[2 * j].r);
-        const float qb = div_by_scale(c.y, sc[2 * j + 1].s, sc[2 * j + 1].r);
+        const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * cs[2 * j], b * cs[2 * j + 1]));
+        const float qa = div_by_scale(c.x, cs[2 * j], cr[2 * j]);
+        const float qb = div_by_scale(c.y, cs[2 * j + 1], cr[2 * j + 1]);
         if constexpr (ERR) {
             row_err = rel_err_fast(qa, a, row_err);
             row_err = rel_err_fast(qb, b, row_err);
@@ -498,82 +712,86 @@ __device__ __forceinline__ uint4 bs_cols_vec_fast(uint4 v, const Scale (&sc)[8],
     err += row_err;
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
-// the same vector with the exact arithmetic (a scale outside the fast range)
-__device__ __forceinline__ uint4 bs_cols_vec_exact(uint4 v, const Scale (&sc)[8], float& err) {
-    uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        float q0 = bs_element<false, false>(bf16_lo(w[j]), sc[2 * j], err);
-        float q1 = bs_element<false, false>(bf16_hi(w[j]), sc[2 * j + 1], err);
-        w[j] = store_pair<false>(q0, q1);
-    }
-    return make_uint4(w[0], w[1], w[2], w[3]);
-}
 
-// pass 2 / pass 4 for column blocks N x 1 with aligned rows (the geometry of k_bs_amax_col): a thread owns 8 adjacent
-// columns over a segment of rows, so its 8 scales and their reciprocals are computed once.  Threads whose scales are
-// not all in the fast range use the exact arithmetic.  A workgroup is 2^cg_log column groups wide and 256 >> cg_log row
-// lanes deep (a tensor of fewer than 2048 columns still fills it); row lane l takes the rows l, l + lanes, ... of a segment.
+// pass 2 / pass 4 for column blocks N x 1 with aligned rows: item = (strip, block row, workgroup of the Q that share
+// them), strips fastest.  A lane owns 8 adjacent columns: it loads their scales and reciprocals (k_bs_colfold) once and
+// takes every Q-th batch of 4 rows per row lane of the block, the next batch on its way while this one is quantized
+// (the arithmetic, 18 issue slots per element with the error term, overlaps the loads of the same wave; workgroups
+// that run side by side work on neighbouring rows).  Lanes whose scales are not all in the fast range use the exact
+// arithmetic.
 template <bool WRITE, bool ERR>
-__global__ __launch_bounds__(WG) void k_bs_quant_col(const uint16_t* in, uint16_t* out, uint32_t* ws, const float* scales,
-                                                     Finish fin, int gate, int ss_mode, int npart1, Shape sh, int rows_per_wg,
-                                                     int cg_log) {
+__global__ __launch_bounds__(WG) void k_bs_quant_col(const uint4* in, uint4* out, uint32_t* ws, const float2* scales,
+                                                     Finish fin, int gate, Shape sh, ColPlan p) {
     __shared__ float s_f[2 * WAVES];
     __shared__ int s_i[WAVES];
     if (gate > 0 && finish_decision(fin, s_f, s_i) != gate) return;
-    const float gamax = reduce_partial_amax(ws, npart1, s_f);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int row_lane = (int)threadIdx.x >> cg_log, row_lanes = WG >> cg_log;
-    const int64_t col0 = (((int64_t)blockIdx.x << cg_log) + (threadIdx.x & ((1 << cg_log) - 1))) * 8;
-    const int64_t segs_per_block = (sh.brows + rows_per_wg - 1) / rows_per_wg;
-    const int64_t row_stride = sh.cols >> 3;
-    const uint4* in4 = reinterpret_cast<const uint4*>(in);
-    uint4* out4 = reinterpret_cast<uint4*>(out);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cl = tid & ((1 << p.cg_log) - 1), rl = tid >> p.cg_log, row_lanes = WG >> p.cg_log;
+    const int64_t row_stride = sh.cols >> 3, groups = row_stride;
+    const bool nt_in = streams_last_read(sh.rows * sh.cols), nt_out = streams_out(sh.rows * sh.cols);
     float err = 0.0f;
-    const bool nt = streams_out(sh.rows * sh.cols);
-    if (col0 < sh.cols) {
-        for (int64_t seg = blockIdx.y; seg < sh.gy * segs_per_block; seg += gridDim.y) {
-            const int64_t by = seg / segs_per_block;
-            const int64_t r_begin = by * sh.brows + (seg - by * segs_per_block) * rows_per_wg;
-            const int64_t r_end = min(r_begin + rows_per_wg, (by + 1) * sh.brows);
-            const int64_t sp = by * sh.cols + col0;
-            Scale sc[8];
-            bool fast = true;
+    for (int64_t item = blockIdx.x; item < p.items2; item += gridDim.x) {
+        const int64_t pid = item / p.strips, strip = item - pid * p.strips;
+        const int64_t by = pid / p.Q, pc = pid - by * p.Q;
+        const int64_t cg = (strip << p.cg_log) + cl;
+        if (cg >= groups) continue;
+        // the block's batches pc, pc + Q, ... of 4 rows per row lane (neighbouring workgroups on neighbouring rows)
+        const int64_t step = 4 * (int64_t)row_lanes, stride = step * p.Q;
+        const int64_t r_first = by * sh.brows + pc * step + rl, r_end = (by + 1) * sh.brows;
+        const uint4* sp = reinterpret_cast<const uint4*>(scales + by * sh.cols + cg * 8);
+        const uint4 t0 = sp[0], t1 = sp[1], t2 = sp[2], t3 = sp[3];
+        const uint4* cin = in + cg;
+        uint4* cout = out + cg;
+        auto load_batch = [&](uint4 (&v)[4], int64_t r) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) { sc[j] = make_scale(block_scale(gamax, scales, sp + j, ss_mode)); fast = fast && sc[j].fast; }
+            for (int k = 0; k < 4; ++k) {
+                v[k] = make_uint4(0, 0, 0, 0);
+                if (r + k * row_lanes < r_end) v[k] = load16_rt(cin + (r + k * row_lanes) * row_stride, nt_in);
+            }
+        };
+        uint4 va[4], vb[4];
+        load_batch(va, r_first);
+        const float cs[8] = {u2f(t0.x), u2f(t0.z), u2f(t1.x), u2f(t1.z), u2f(t2.x), u2f(t2.z), u2f(t3.x), u2f(t3.z)};
+        const float cr[8] = {u2f(t0.y), u2f(t0.w), u2f(t1.y), u2f(t1.w), u2f(t2.y), u2f(t2.w), u2f(t3.y), u2f(t3.w)};
+        bool fast = true;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) fast = fast && (cr[j] != 0.0f);
+        auto do_batch = [&](uint4 (&v)[4], int64_t r) {
             if (fast) {
-#pragma unroll 1
-                for (int64_t r = r_begin + row_lane; r < r_end; r += 4 * row_lanes) {
-                    uint4 v[4];
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        v[k] = make_uint4(0, 0, 0, 0);
-                        if (r + k * row_lanes < r_end) v[k] = load16_rt(in4 + (r + k * row_lanes) * row_stride + (col0 >> 3), streams_last_read(sh.rows * sh.cols));
-                    }
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const uint4 q = bs_cols_vec_fast<WRITE, ERR>(v[k], sc, err);
-                        if constexpr (WRITE) {
-                            if (r + k * row_lanes < r_end) store16_rt(out4 + (r + k * row_lanes) * row_stride + (col0 >> 3), q, nt);
-                        }
+                for (int k = 0; k < 4; ++k) {
+                    const uint4 q = bs_cols_vec_fast<WRITE, ERR>(v[k], cs, cr, err);
+                    if constexpr (WRITE) {
+                        if (r + k * row_lanes < r_end) store16_rt(cout + (r + k * row_lanes) * row_stride, q, nt_out);
                     }
                 }
             } else {
+                // (from memory again, non-unrolled: indexing the register arrays with a run-time k would move them to
+                // scratch memory for the fast path as well)
 #pragma unroll 1
-                for (int64_t r = r_begin + row_lane; r < r_end; r += row_lanes) {
-                    const uint4 q = bs_cols_vec_exact(in4[r * row_stride + (col0 >> 3)], sc, err);
-                    if constexpr (WRITE) out4[r * row_stride + (col0 >> 3)] = q;
+                for (int k = 0; k < 4; ++k) {
+                    if (r + k * row_lanes >= r_end) break;
+                    const uint4 q = bs_cols_vec_exact(cin[(r + k * row_lanes) * row_stride], cs, err);
+                    if constexpr (WRITE) cout[(r + k * row_lanes) * row_stride] = q;
                 }
             }
+        };
+#pragma unroll 1
+        for (int64_t r = r_first; r < r_end; r += 2 * stride) {
+            load_batch(vb, r + stride);
+            asm volatile("" ::: "memory");         // (the loads stay ahead of the arithmetic they are meant to overlap)
+            do_batch(va, r);
+            load_batch(va, r + 2 * stride);
+            asm volatile("" ::: "memory");
+            do_batch(vb, r + stride);
         }
     }
     if constexpr (ERR) {
         err = wave_sum(err);
-        __syncthreads();                   // every wave has read the tensor amax from these slots
+        __syncthreads();
         if (lane == 0) s_f[wave] = err;
         __syncthreads();
-        if (threadIdx.x == 0)
-            reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x + gridDim.x * blockIdx.y] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+        if (threadIdx.x == 0) reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
     }
 }
 
@@ -948,12 +1166,20 @@ __global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, 
 
 using namespace mor;
 
+// 32-bit words of the workspace behind the header and the partial arrays: one float per block, or, for column blocks
+// N x 1, the scales and the partial maxima of the column kernels where they take more
+static int64_t block_words(int64_t rows, int64_t cols, int64_t brows, int64_t bcols) {
+    int64_t words = cdiv(rows, brows) * cdiv(cols, bcols);
+    if (bcols == 1 && brows > 1) words = std::max(words, col_words(rows, cols, brows));
+    return words;
+}
+
 extern "C" size_t mor_workspace_bytes(int op, int64_t rows, int64_t cols, int64_t brows, int64_t bcols) {
     if (rows <= 0 || cols <= 0 || brows <= 0 || bcols <= 0) return 0;
     switch (op) {
         case MOR_OP_BLOCK_SCALING:
         case MOR_OP_CHANNEL_SCALING:
-            return (size_t)(WS_BLOCKS + cdiv(rows, brows) * cdiv(cols, bcols)) * 4;
+            return (size_t)(WS_BLOCKS + block_words(rows, cols, brows, bcols)) * 4;
         case MOR_OP_E8MX:
             return (size_t)WS_BLOCKS * 4;
         default:
@@ -1119,15 +1345,30 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
     // amax and the non-zero count
     const int64_t G = bcols / 8;
     int npart;
+    // column blocks with aligned rows, default flavour, fp32 scale: k_bs_colmax / k_bs_quant_col (16-byte accesses to the
+    // partial maxima in the workspace)
+    ColPlan cp;
+    const bool col_fast = col && vec && !emu && ss_mode != 2 && aligned16(blocks) && col_plan(rows, cols, brows, cp);
+    float2* col_scales = reinterpret_cast<float2*>(blocks);                                   // [block row][column]
+    uint16_t* col_partial = reinterpret_cast<uint16_t*>(blocks + sh.gy * cols * 2);           // [block row][segment][column]
     if (ss_mode == 4 && !col && vec && n % 8 == 0) {
         npart = (int)std::min<int64_t>(cdiv(n / 8, 8 * WG), PASS1_MAX);
         k_bs_amax_flat<<<npart, WG, 0, st>>>(static_cast<const uint4*>(input), ws, nullptr, n / 8, 1, 0);
+    } else if (col_fast) {
+        // column blocks, the fast path: rows of partial maxima (no atomics, nothing to clear), folded into the columns' scales
+        npart = (int)std::min<int64_t>(cp.items1, PASS1_MAX);
+        const uint4* i4 = static_cast<const uint4*>(input);
+        switch (cp.ng) {
+#define MOR_COLMAX(NG) case NG: k_bs_colmax<NG><<<npart, WG, 0, st>>>(i4, ws, col_partial, sh, cp); break
+            MOR_COLMAX(1); MOR_COLMAX(2); MOR_COLMAX(3); MOR_COLMAX(4); MOR_COLMAX(5); MOR_COLMAX(6); MOR_COLMAX(7); MOR_COLMAX(8);
+#undef MOR_COLMAX
+        }
+        k_bs_colfold<<<(unsigned)(sh.gy * cdiv(cols / 8, FOLD_G)), WG, 0, st>>>(col_partial, col_scales, ws, npart, (int)ss_mode, sh, cp);
     } else if (col) {
         k_zero_f32<<<grid_for(nb), WG, 0, st>>>(blocks, nb);
         const int rows_per_wg = (int)std::min<int64_t>(brows, 256);
-        const unsigned gx = (unsigned)cdiv(cols, 256);
+        const unsigned gx = (unsigned)std::min<int64_t>(cdiv(cols, 256), PASS1_MAX);
         const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
-        if ((int64_t)gx > PASS1_MAX) return mor_fail(MOR_ERR_INVALID_ARGUMENT, "too many columns (%lld)", (long long)cols);
         const unsigned gy = (unsigned)std::min<int64_t>(segs, std::max<int64_t>(PASS1_MAX / gx, 1));
         npart = (int)(gx * gy);
         k_bs_amax_col<<<dim3(gx, gy), WG, 0, st>>>(in16, ws, blocks, sh, rows_per_wg, vec);
@@ -1154,18 +1395,14 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
     // the pass-1 partials to the tensor amax and computes its blocks' scales from it
     // end: bf16 fallback (out of place: copy if meta == 3) or the quantized write (in place: only if meta == 1)
     const bool e8 = (ss_mode == 2);
-    if (col && vec && !emu && !e8) {
-        // a workgroup is min(256, column groups) lanes wide (a power of two) and the rest of its threads deep: 32 rows per
-        // thread and segment (16384 x 1024: 128 lanes x 2 row lanes instead of half-empty workgroups, the op 41.5 -> 34.4 us)
-        const int cg_log = std::min(8, ilog2(cdiv(cols, 8)));
-        const int rows_per_wg = (int)std::min<int64_t>(brows, 32 * (WG >> cg_log));
-        const unsigned gx = (unsigned)cdiv(cdiv(cols, 8), (int64_t)1 << cg_log);
-        const int64_t segs = sh.gy * cdiv(brows, rows_per_wg);
-        const dim3 grid(gx, (unsigned)std::min<int64_t>(segs, std::max<int64_t>(PASS2_MAX / gx, 1)));
-        fin.nerr = (int)(grid.x * grid.y);
-        if (inplace) k_bs_quant_col<false, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 0, (int)ss_mode, npart, sh, rows_per_wg, cg_log);
-        else k_bs_quant_col<true, true><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 0, (int)ss_mode, npart, sh, rows_per_wg, cg_log);
-        if (inplace) k_bs_quant_col<true, false><<<grid, WG, 0, st>>>(in16, out16, ws, blocks, fin, 1, (int)ss_mode, npart, sh, rows_per_wg, cg_log);
+    if (col_fast) {
+        const int grid = (int)std::min<int64_t>(cp.items2, PASS2_MAX);
+        fin.nerr = grid;
+        const uint4* i4 = static_cast<const uint4*>(input);
+        uint4* o4 = static_cast<uint4*>(output);
+        if (inplace) k_bs_quant_col<false, true><<<grid, WG, 0, st>>>(i4, o4, ws, col_scales, fin, 0, sh, cp);
+        else k_bs_quant_col<true, true><<<grid, WG, 0, st>>>(i4, o4, ws, col_scales, fin, 0, sh, cp);
+        if (inplace) k_bs_quant_col<true, false><<<grid, WG, 0, st>>>(i4, o4, ws, col_scales, fin, 1, sh, cp);
     } else {
         const bool vec2 = vec && (col || bcols % 8 == 0) && n / 8 < 0xFFFFFFFFll;
         const int64_t work = vec2 ? n / 8 : n;
@@ -1215,9 +1452,9 @@ extern "C" int mor_block_scaling_static(const void* input, void* output, int32_t
                                         uint32_t flags, void* stream) {
     if (int rc = block_scaling_check(input, output, meta, global_amax, global_non_zero, global_error, rows, cols, brows, bcols, ss_mode, channel)) return rc;
     const int64_t nb = (rows / brows) * (cols / bcols);
-    if (nb > (int64_t)MOR_STATIC_MAX_BLOCKS)
-        return mor_fail(MOR_ERR_WORKSPACE, "mor_block_scaling_static takes at most %lld blocks (got %lld): use mor_block_scaling with a workspace",
-                        (long long)MOR_STATIC_MAX_BLOCKS, (long long)nb);
+    if (nb > (int64_t)MOR_STATIC_MAX_BLOCKS || block_words(rows, cols, brows, bcols) > (int64_t)MOR_STATIC_MAX_BLOCKS)
+        return mor_fail(MOR_ERR_WORKSPACE, "mor_block_scaling_static takes at most %lld blocks (got %lld; column blocks take up to 32 "
+                        "workspace words each): use mor_block_scaling with a workspace", (long long)MOR_STATIC_MAX_BLOCKS, (long long)nb);
     void* ws = nullptr;
     if (int rc = static_scratch(&ws)) return rc;
     return block_scaling_run(input, output, meta, global_amax, global_non_zero, global_error, rows, cols, brows, bcols,

@@ -1,8 +1,9 @@
 """`mor.ops` for MI355X: the operator layer of the reference (mor/ops.py, mor/csrc/fake_quantize.cpp) over libmor_hip.so.
 
 The 14 operator schemas are registered verbatim under the `mor` namespace (mor/csrc/fake_quantize.cpp:12-25), their
-implementations are registered for the CUDA dispatch key (which HIP tensors use under ROCm), and the Python wrappers
-and straight-through autograd registrations mirror mor/ops.py:11-156 name for name and argument for argument.
+implementations are registered for the CUDA dispatch key (which HIP tensors use under ROCm) by libmor_torch.so
+(csrc/torch_binding.cpp), and the Python wrappers and straight-through autograd registrations mirror
+mor/ops.py:11-156 name for name and argument for argument.
 
 Differences from the reference, all of them relaxations:
   * launches go to torch's current stream instead of the legacy default stream;
@@ -46,8 +47,7 @@ def set_flavour(name: str) -> None:
     the calling thread's later calls only."""
     _flavour.flags = {"kernel": _cabi.FLAG_DEFAULT, "torch_emulation": _cabi.FLAG_TORCH_EMULATION,
                       "software_cast": _cabi.FLAG_SOFTWARE_CAST}[name]
-    if _native is not None:
-        _native.mor_torch_set_flags(_flavour.flags)
+    _native.mor_torch_set_flags(_flavour.flags)
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -70,142 +70,17 @@ _lib.define("fake_quantize_channel_scaling_inplace(Tensor input, int dim_x, int 
 
 
 # ----------------------------------------------------------------------------------------------------------------------
-# host launchers: the checks of FQ:1841-1844, 1887-1890, 1912-1915, 2016-2021, then one C ABI call
-def _check_input(t: Tensor, dtype, rows: int, cols: int, what: str = "input") -> None:
-    if t.dtype != dtype:
-        raise RuntimeError(f"mor: {what} must be {dtype}, got {t.dtype}")
-    if t.dim() != 2 or t.size(0) != rows or t.size(1) != cols:
-        raise RuntimeError(f"mor: {what} must have shape ({rows}, {cols}), got {tuple(t.shape)}")
-    if not t.is_cuda:
-        raise RuntimeError(f"mor: {what} must be a GPU tensor")
-
-
-def _check_result(t: Tensor, rows: int, cols: int) -> None:
-    _check_input(t, torch.bfloat16, rows, cols, "result")
-    if not t.is_contiguous():
-        raise RuntimeError("mor: result must be contiguous")
-
-
-def _stream(t: Tensor) -> int:
-    return torch._C._cuda_getCurrentRawStream(t.device.index)
-
-
-class _on_device:
-    """`with torch.cuda.device(d)` only when d is not already the current device (the usual case costs nothing)."""
-    __slots__ = ("ctx",)
-
-    def __init__(self, device):
-        self.ctx = None if device.index == torch.cuda.current_device() else torch.cuda.device(device)
-
-    def __enter__(self):
-        if self.ctx is not None:
-            self.ctx.__enter__()
-
-    def __exit__(self, *exc):
-        if self.ctx is not None:
-            self.ctx.__exit__(*exc)
-        return False
-
-
-def _cdiv(a: int, b: int) -> int:
-    return (a + b - 1) // b
-
-
-def _check_blocks(block_x: int, block_y: int) -> None:
-    if block_x <= 0 or block_y <= 0:
-        raise RuntimeError(f"mor: block dims must be positive, got ({block_x}, {block_y})")
-
-
-def _fake_quantize_impl(input, dim_x, dim_y, block_x, block_y, clamp_threshold, mode, sf_type):
-    _check_input(input, torch.bfloat16, dim_x, dim_y)
-    _check_blocks(block_x, block_y)
-    x = input.contiguous()
-    with _on_device(x.device):
-        out = torch.empty_like(x)
-        meta = torch.empty((_cdiv(dim_x, block_x), _cdiv(dim_y, block_y)), dtype=torch.int32, device=x.device)
-        _cabi.check(_L.mor_fake_quantize(x.data_ptr(), out.data_ptr(), meta.data_ptr(), dim_x, dim_y, block_x, block_y,
-                                         clamp_threshold, mode, sf_type, _flavour.flags, _stream(x)))
-    return [out, meta]
-
-
-def _fake_quantize_no_alloc_impl(input, dim_x, dim_y, block_x, block_y, clamp_threshold, mode, sf_type, result):
-    _check_input(input, torch.bfloat16, dim_x, dim_y)
-    _check_result(result, dim_x, dim_y)
-    _check_blocks(block_x, block_y)
-    x = input.contiguous()
-    with _on_device(x.device):
-        meta = torch.empty((_cdiv(dim_x, block_x), _cdiv(dim_y, block_y)), dtype=torch.int32, device=x.device)
-        _cabi.check(_L.mor_fake_quantize(x.data_ptr(), result.data_ptr(), meta.data_ptr(), dim_x, dim_y, block_x, block_y,
-                                         clamp_threshold, mode, sf_type, _flavour.flags, _stream(x)))
-    return meta
-
-
-def _scaling_impl(input, dim_x, dim_y, block_x, block_y, e4m3_threshold, ss_mode, channel, inplace):
-    _check_input(input, torch.bfloat16, dim_x, dim_y)
-    _check_blocks(block_x, block_y)
-    if dim_x % block_x or dim_y % block_y:
-        raise RuntimeError(f"mor: block ({block_x}, {block_y}) does not divide the tensor ({dim_x}, {dim_y})")
-    x = input.contiguous()
-    with _on_device(x.device):
-        dev = x.device
-        out = x if inplace else torch.empty_like(x)
-        meta = torch.empty(1, dtype=torch.int32, device=dev)
-        gamax = torch.empty(1, dtype=torch.float32, device=dev)
-        gnnz = torch.empty(1, dtype=torch.int32, device=dev)
-        gerr = torch.empty(1, dtype=torch.float32, device=dev)
-        op = _cabi.OP_CHANNEL_SCALING if channel else _cabi.OP_BLOCK_SCALING
-        nbytes = _L.mor_workspace_bytes(op, dim_x, dim_y, block_x, block_y)
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-        _cabi.check(_L.mor_block_scaling(x.data_ptr(), out.data_ptr(), meta.data_ptr(), gamax.data_ptr(), gnnz.data_ptr(),
-                                         gerr.data_ptr(), dim_x, dim_y, block_x, block_y, e4m3_threshold, ss_mode,
-                                         1 if channel else 0, ws.data_ptr(), nbytes, _flavour.flags, _stream(x)))
-        if inplace and x.data_ptr() != input.data_ptr():
-            input.copy_(x)            # a non-contiguous input was quantized through a contiguous copy
-    return [meta, gamax, gnnz, gerr] if inplace else [out, meta, gamax, gnnz, gerr]
-
-
-def _e8mx_impl(input, dim_x, dim_y, block_x, block_y, quantize_type, scaling_strategy, result=None):
-    _check_input(input, torch.bfloat16, dim_x, dim_y)
-    _check_blocks(block_x, block_y)
-    if result is not None:
-        _check_result(result, dim_x, dim_y)
-    x = input.contiguous()
-    with _on_device(x.device):
-        out = torch.empty_like(x) if result is None else result
-        nbytes = _L.mor_workspace_bytes(_cabi.OP_E8MX, dim_x, dim_y, block_x, block_y)
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
-        _cabi.check(_L.mor_e8mx(x.data_ptr(), out.data_ptr(), dim_x, dim_y, block_x, block_y, quantize_type, scaling_strategy,
-                                ws.data_ptr(), nbytes, _flavour.flags, _stream(x)))
-    return out
-
-
-def _quant_dequant_impl(input, dim_x, dim_y, fmt):
-    _check_input(input, torch.float32, dim_x, dim_y)
-    x = input.contiguous()
-    with _on_device(x.device):
-        out = torch.empty_like(x)
-        _cabi.check(_L.mor_quant_dequant(x.data_ptr(), out.data_ptr(), x.numel(), fmt, _stream(x)))
-    return out
-
-
-def _e8_scale_impl(input, dim_x, dim_y, rne):
-    _check_input(input, torch.float32, dim_x, dim_y)
-    x = input.contiguous()
-    with _on_device(x.device):
-        out = torch.empty_like(x)
-        _cabi.check(_L.mor_e4m3_with_e8_scale(x.data_ptr(), out.data_ptr(), x.numel(), rne, _stream(x)))
-    return out
-
-
-# registrations for the CUDA key: FQ:2663-2678.  The C++ registrations of csrc/torch_binding.cpp (libmor_torch.so)
-# are used when that library has been built: the same checks, allocations and C ABI calls without the interpreter
-# (about 6 instead of 14 microseconds per call).  The Python implementations below are the same path otherwise.
+# Implementations for the CUDA dispatch key (which HIP tensors use under ROCm), FQ:2663-2678: the C++ registrations of
+# csrc/torch_binding.cpp (libmor_torch.so) -- the checks of FQ:1841-1844, 1887-1890, 1912-1915, 2016-2021, the
+# allocations, one C ABI call -- and the straight-through autograd of the four differentiable forward ops.  There is no
+# second implementation: without that library the import fails, as it does without libmor_hip.so.
 def _load_native():
     import ctypes
     import os
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libmor_torch.so")
-    if os.environ.get("MOR_PYTHON_OPS") == "1" or not os.path.exists(path):
-        return None
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'`; "
+                          "the mor operators have no other implementation")
     torch.ops.load_library(path)
     lib = ctypes.CDLL(path)
     lib.mor_torch_set_flags.argtypes = [ctypes.c_uint32]
@@ -216,36 +91,8 @@ def _load_native():
 _native = _load_native()
 
 
-class _PythonImpls:
-    """Registers an implementation only when the C++ ones are not loaded."""
-
-    @staticmethod
-    def impl(name, fn, key):
-        if _native is None:
-            _lib.impl(name, fn, key)
-
-
-_reg = _PythonImpls
-_reg.impl("fake_quantize", _fake_quantize_impl, "CUDA")
-_reg.impl("fake_quantize_no_alloc", _fake_quantize_no_alloc_impl, "CUDA")
-_reg.impl("quant_dequant_e4m3", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E4M3), "CUDA")
-_reg.impl("quant_dequant_e5m2", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E5M2), "CUDA")
-_reg.impl("quant_dequant_e3m2", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E3M2), "CUDA")
-_reg.impl("quant_dequant_e2m3", lambda i, x, y, bx, by: _quant_dequant_impl(i, x, y, _cabi.FMT_E2M3), "CUDA")
-_reg.impl("e4m3_with_e8_scale_rne", lambda i, x, y, bx, by: _e8_scale_impl(i, x, y, 1), "CUDA")
-_reg.impl("e4m3_with_e8_scale_rz", lambda i, x, y, bx, by: _e8_scale_impl(i, x, y, 0), "CUDA")
-_reg.impl("fake_quantize_block_scaling", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, False, False), "CUDA")
-_reg.impl("fake_quantize_block_scaling_inplace", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, False, True), "CUDA")
-_reg.impl("fake_quantize_channel_scaling", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, True, False), "CUDA")
-_reg.impl("fake_quantize_channel_scaling_inplace", lambda i, x, y, bx, by, t, s: _scaling_impl(i, x, y, bx, by, t, s, True, True), "CUDA")
-_reg.impl("fake_quantize_e8mx", lambda i, x, y, bx, by, q, s: _e8mx_impl(i, x, y, bx, by, q, s), "CUDA")
-
-
-def _e8mx_inplace_impl(input, dim_x, dim_y, block_x, block_y, quantize_type, scaling_strategy, result):
-    _e8mx_impl(input, dim_x, dim_y, block_x, block_y, quantize_type, scaling_strategy, result)
-
-
-_reg.impl("fake_quantize_e8mx_inplace", _e8mx_inplace_impl, "CUDA")
+def _cdiv(a: int, b: int) -> int:
+    return (a + b - 1) // b
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -369,7 +216,7 @@ def e4m3_with_e8_scale_rz(a: Tensor, dim_x: int, dim_y: int, block_x: int, block
 
 # (op, number of non-tensor arguments that get a None gradient); fake_quantize_e8mx_inplace has no autograd
 # registration in the reference either (mor/ops.py:104-106).  The four differentiable forward ops have their
-# straight-through autograd in C++ when libmor_torch.so is loaded.
+# straight-through autograd in C++ (libmor_torch.so).
 _NATIVE_AUTOGRAD = ("fake_quantize", "fake_quantize_block_scaling", "fake_quantize_channel_scaling", "fake_quantize_e8mx")
 for _name, _n in (("fake_quantize", 7), ("fake_quantize_no_alloc", 8),
                   ("fake_quantize_block_scaling", 6), ("fake_quantize_block_scaling_inplace", 6),
@@ -377,5 +224,5 @@ for _name, _n in (("fake_quantize", 7), ("fake_quantize_no_alloc", 8),
                   ("fake_quantize_e8mx", 6),
                   ("quant_dequant_e4m3", 4), ("quant_dequant_e5m2", 4), ("quant_dequant_e2m3", 4), ("quant_dequant_e3m2", 4),
                   ("e4m3_with_e8_scale_rne", 4), ("e4m3_with_e8_scale_rz", 4)):
-    if _native is None or _name not in _NATIVE_AUTOGRAD:
+    if _name not in _NATIVE_AUTOGRAD:
         torch.library.register_autograd(f"mor::{_name}", _ste(_n), setup_context=_noop_setup_context)

@@ -35,13 +35,23 @@ def static_call(G, a, br, bc, thr, ss, channel, inplace=False):
     gnnz = torch.zeros(1, dtype=torch.int32, device=G.dev())
     gerr = torch.zeros(1, dtype=torch.float32, device=G.dev())
     torch.cuda.synchronize()
+    # torch's allocator counts torch's own allocations only; the free bytes of the device (hipMemGetInfo) would also
+    # show a hipMalloc made inside the library.  The first call on a device loads the code object with its static
+    # array, so the device-level comparison starts with the second.
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]
     rc = L.mor_block_scaling_static(x.data_ptr(), out.data_ptr(), meta.data_ptr(), gamax.data_ptr(), gnnz.data_ptr(),
                                     gerr.data_ptr(), rows, cols, br, bc, float(thr), ss, int(channel), 0, G.stream_ptr())
     _cabi.check(rc)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    if static_call.warm:
+        assert torch.cuda.mem_get_info()[0] == free_before, "the device's free memory changed during the call"
+    static_call.warm = True
     return G.to_host_u16(out), meta.cpu().numpy(), gamax.cpu().numpy(), gnnz.cpu().numpy(), gerr.cpu().numpy()
+
+
+static_call.warm = False
 
 
 def same(got, want, what):
