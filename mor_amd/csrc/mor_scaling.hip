@@ -565,8 +565,9 @@ __device__ __forceinline__ float rel_err_fast(float q, float a, float acc) {
 // No selects: a zero element's magnitude bits are 0; the sign of the input is kept for non-zero halves only (zero inputs come back as +0, FQ:1133-1134), through a
 // packed 16-bit mask.
 // ERR / OUT: whether the error terms / the output word are wanted (the in-place phases need one of them each).
+// (`codes`: the register the convert writes half of, carried from word to word so that no fresh zero is needed)
 template <bool E8, bool ERR = true, bool OUT = true>
-__device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, float rs, float& err) {
+__device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, float rs, float& err, uint32_t& codes) {
     const float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
     float qa, qb;
     if constexpr (E8) {
@@ -577,7 +578,8 @@ __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, fl
         qa = (a == 0.0f) ? 0.0f : fmaxf(q.x, art);
         qb = (b == 0.0f) ? 0.0f : fmaxf(q.y, art);
     } else {
-        const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * sc.s, b * sc.s));
+        codes = hw_pack2_low_keep<FMT_E4M3>(a * sc.s, b * sc.s, codes);
+        const f32x2 c = hw_unpack2_low<FMT_E4M3>(codes);
         qa = div_by_scale(c.x, sc.s, rs);
         qb = div_by_scale(c.y, sc.s, rs);
     }
@@ -592,10 +594,11 @@ __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, fl
 template <bool E8, bool ERR, bool OUT>
 __device__ __forceinline__ uint4 bs_vec_fast(uint4 v, const Scale& sc, float& err) {
     uint4 q;
-    q.x = bs_pair_fast<E8, ERR, OUT>(v.x, sc, sc.r, err);
-    q.y = bs_pair_fast<E8, ERR, OUT>(v.y, sc, sc.r, err);
-    q.z = bs_pair_fast<E8, ERR, OUT>(v.z, sc, sc.r, err);
-    q.w = bs_pair_fast<E8, ERR, OUT>(v.w, sc, sc.r, err);
+    uint32_t codes = 0;
+    q.x = bs_pair_fast<E8, ERR, OUT>(v.x, sc, sc.r, err, codes);
+    q.y = bs_pair_fast<E8, ERR, OUT>(v.y, sc, sc.r, err, codes);
+    q.z = bs_pair_fast<E8, ERR, OUT>(v.z, sc, sc.r, err, codes);
+    q.w = bs_pair_fast<E8, ERR, OUT>(v.w, sc, sc.r, err, codes);
     return q;
 }
 
@@ -636,8 +639,9 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
                 const Scale sc = make_scale(block_scale(gamax, scales, (int64_t)by * sh.gx + bx, ss_mode));
                 if (!EMU && sc.fast && !vec_has_nan(v)) {
                     const float rs = 1.0f / sc.s;
+                    uint32_t codes = 0;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) w[j] = bs_pair_fast<E8, ERR, WRITE>(w[j], sc, rs, err);
+                    for (int j = 0; j < 4; ++j) w[j] = bs_pair_fast<E8, ERR, WRITE>(w[j], sc, rs, err, codes);
                 } else {
 #pragma unroll 1
                     for (int j = 0; j < 4; ++j) {
@@ -694,10 +698,12 @@ __device__ __forceinline__ uint4 bs_cols_vec_fast(uint4 v, const float (&cs)[8],
     if (vec_has_nan(v)) return bs_cols_vec_exact(v, cs, err);          // (rare)
     uint32_t w[4] = {v.x, v.y, v.z, v.w};
     float row_err = 0.0f;
+    uint32_t codes = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const float a = fabsf(bf16_lo(w[j])), b = fabsf(bf16_hi(w[j]));
-        const f32x2 c = hw_unpack2_low<FMT_E4M3>(hw_pack2_low<FMT_E4M3>(a * cs[2 * j], b * cs[2 * j + 1]));
+        codes = hw_pack2_low_keep<FMT_E4M3>(a * cs[2 * j], b * cs[2 * j + 1], codes);
+        const f32x2 c = hw_unpack2_low<FMT_E4M3>(codes);
         const float qa = div_by_scale(c.x, cs[2 * j], cr[2 * j]);
         const float qb = div_by_scale(c.y, cs[2 * j + 1], cr[2 * j + 1]);
         if constexpr (ERR) {
@@ -960,6 +966,103 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
         if (npart1 == 0) {
             reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = n;
             reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = red_fmax();
+        }
+    }
+}
+
+// The same single pass for row blocks of 512 * NVW elements, NVW = 2, 4 or 8 (rows of 4096 elements: per-channel
+// scaling of a weight matrix): a wave per block.  A lane holds NVW vectors of its row, the block's amax and non-zero
+// count meet by DPP and two shuffles inside the wave, so a workgroup works on four rows at once without a barrier or an
+// LDS exchange between them, every wave's loads in flight while the others quantize (one workgroup per row: 58 us for
+// 16384 rows of 4096 elements from HBM, the plain quantization of the same rows 43).  Rows are dealt out to the waves in
+// turn, so that the waves that run side by side work on neighbouring rows.  Phases and npart1 as in k_bs_fused.
+template <bool E8, int NVW>
+__global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* out, uint32_t* ws, Shape sh, int ss_mode,
+                                                      int64_t nrows, Finish fin, int phase, int npart1) {
+    __shared__ float s_f[2 * WAVES];
+    __shared__ int s_i[WAVES];
+    if (phase == 2 && finish_decision(fin, s_f, s_i) != 1) return;
+    const float gamax = npart1 > 0 ? reduce_partial_amax(ws, npart1, s_f) : 0.0f;
+    __syncthreads();
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool write = phase != 1;
+    const bool nt_out = streams_out(sh.rows * sh.cols), nt_in = streams_last_read(sh.rows * sh.cols);
+    constexpr int ROW = 64 * NVW;                                   // chunks of a block
+    float gmax = 0.0f, err = 0.0f;
+    int nnz_total = 0;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < nrows; row += (int64_t)gridDim.x * WAVES) {
+        const uint4* bin = in + row * ROW + lane;
+        uint4* bout = out + row * ROW + lane;
+        uint4 v[NVW];
+#pragma unroll
+        for (int k = 0; k < NVW; ++k) v[k] = load16_rt(bin + 64 * k, nt_in);
+        uint32_t amax2 = 0, nnz2 = 0;
+#pragma unroll
+        for (int k = 0; k < NVW; ++k) {
+            acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+            acc_nnz_pk(nnz2, v[k].x); acc_nnz_pk(nnz2, v[k].y); acc_nnz_pk(nnz2, v[k].z); acc_nnz_pk(nnz2, v[k].w);
+            opaque(v[k]);
+        }
+        const uint32_t amax_b = group_umax(amax_bits_of(amax2), 64);
+        const bool has_nan = amax_b > 0x7F800000u;                  // uniform over the wave
+        float amax = u2f(amax_b);
+        int nnz_row = (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
+        if (has_nan) {                            // the float maximum and the count of the reference skip a NaN (rare)
+            amax = 0.0f;
+#pragma unroll
+            for (int k = 0; k < NVW; ++k) {
+                acc_amax(amax, v[k].x); acc_amax(amax, v[k].y); acc_amax(amax, v[k].z); acc_amax(amax, v[k].w);
+                nnz_row -= nan_word(v[k].x) + nan_word(v[k].y) + nan_word(v[k].z) + nan_word(v[k].w);
+            }
+            amax = group_max(amax, 64);
+        }
+        gmax = fmaxf(gmax, amax);
+        nnz_total += nnz_row;
+        const Scale sc = make_scale(scaling_factor(gamax, amax, ss_mode));
+        if (!has_nan && (sc.fast || !(amax > 0.0f))) {          // an all-zero block gives +0 whatever its (clamped) scale is
+            if (phase == 1) {                      // decision pass of the in-place variant: error terms only
+#pragma unroll
+                for (int k = 0; k < NVW; ++k) { opaque(v[k]); bs_vec_fast<E8, true, false>(v[k], sc, err); asm volatile("" : "+v"(err)); }
+            } else if (phase == 2) {               // write pass of the in-place variant: no error terms
+#pragma unroll
+                for (int k = 0; k < NVW; ++k) {
+                    opaque(v[k]);
+                    uint4 q = bs_vec_fast<E8, false, true>(v[k], sc, err);
+                    opaque(q);
+                    store16_rt(bout + 64 * k, q, nt_out);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < NVW; ++k) {
+                    opaque(v[k]);
+                    uint4 q = bs_vec_fast<E8, true, true>(v[k], sc, err);
+                    opaque(q);
+                    asm volatile("" : "+v"(err));
+                    store16_rt(bout + 64 * k, q, nt_out);
+                }
+            }
+        } else {
+            // the exact arithmetic, from memory again (non-unrolled: no run-time index into the register array)
+            const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in) + row * ROW * 8;
+            uint16_t* out16 = reinterpret_cast<uint16_t*>(out) + row * ROW * 8;
+#pragma unroll 1
+            for (int i = lane; i < ROW * 8; i += 64) {
+                const float q = bs_element<E8, false>(bf16_one(in16[i]), sc, err);
+                if (write) out16[i] = store_bf16<false>(q);
+            }
+        }
+    }
+    err = wave_sum(err);
+    nnz_total = wave_sum_i(nnz_total);
+    gmax = group_max(gmax, 64);
+    __syncthreads();
+    if (lane == 0) { s_f[wave] = err; s_f[4 + wave] = gmax; s_i[wave] = nnz_total; }
+    __syncthreads();
+    if (tid == 0 && phase != 2) {
+        reinterpret_cast<float*>(ws)[WS_ERR + blockIdx.x] = (s_f[0] + s_f[1]) + (s_f[2] + s_f[3]);
+        if (npart1 == 0) {
+            reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+            reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = fmaxf(fmaxf(s_f[4], s_f[5]), fmaxf(s_f[6], s_f[7]));
         }
     }
 }
@@ -1283,6 +1386,25 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
         k_bs_amax_flat<<<npart1, WG, 0, st>>>(static_cast<const uint4*>(input), ws, nullptr, n / 8, 1, 0);
     };
     const bool flat_ok = !emu && vec && n % 8 == 0;
+    if (flat_ok && brows == 1 && ss_mode != 4 && (blk_chunks == 128 || blk_chunks == 256 || blk_chunks == 512)) {
+        // row blocks of 1024, 2048 or 4096 elements: a wave per block
+        if (global) tensor_amax_pass();
+        // (four workgroups per CU: 16384 rows of 4096 elements from HBM take 54.7 us with 1024 workgroups, 59 with 2048, 57.6 with 4096)
+        const int grid = (int)std::min<int64_t>(cdiv(nb, WAVES), 1024);
+        fin.nerr = grid;
+        fin.nstat = global ? npart1 : grid;
+        const uint4* i4 = static_cast<const uint4*>(input);
+        uint4* o4 = static_cast<uint4*>(output);
+        const int nvw = (int)(blk_chunks / 64);
+        for (int phase = inplace ? 1 : 0; phase <= (inplace ? 2 : 0); ++phase) {
+#define MOR_BS_WAVE(E8, NVW) k_bs_fused_wave<E8, NVW><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, nb, fin, phase, npart1)
+            if (ss_mode == 2) { if (nvw == 2) MOR_BS_WAVE(true, 2); else if (nvw == 4) MOR_BS_WAVE(true, 4); else MOR_BS_WAVE(true, 8); }
+            else { if (nvw == 2) MOR_BS_WAVE(false, 2); else if (nvw == 4) MOR_BS_WAVE(false, 4); else MOR_BS_WAVE(false, 8); }
+#undef MOR_BS_WAVE
+        }
+        if (!inplace) gated_copy();
+        return mor_check_launch("mor_block_scaling (single pass, a wave per row block)");
+    }
     if (flat_ok && !col && ss_mode != 4 && blk_chunks >= WG && blk_chunks <= 8 * 1024
         && brows * (cols / 8) < 0x7FFFFFFFll && (is_pow2(bcols / 8) || brows == 1)) {
         if (global) tensor_amax_pass();
