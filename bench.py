@@ -9,8 +9,11 @@ MoR 128 x 128 pass over an 8192 x 8192 N(0,1) tensor (four launches).  The launc
 output buffer pairs, so that every byte comes from HBM and not from the 256 MB last-level cache.  The printed JSON
 line reports algorithmic HBM GB/s (2 B read + 2 B written per element + 4 B of meta per block where the op returns
 meta) for the whole step, the roofline fraction of the kernel furthest below the roofline from HIP events recorded
-around its launches in the timed region (with the cache-warm figure of every kernel beside it), the other
-configurations, and the CPU oracle timed on bounded samples of the same workloads on the host cores.
+around its launches in the timed region (with the cache-warm figure of every kernel beside it), the roofline
+fraction of every BASELINE configuration from HBM (`roofline.per_config`), what bounds the MoR kernel
+(`roofline.mor_128x128_breakdown`), the clocks and the power over the first milliseconds after idle
+(`after_idle_transient`), the other configurations, and the CPU oracle timed on bounded samples of the same workloads
+on the host cores.
 """
 import argparse
 import json
@@ -20,7 +23,6 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
 
@@ -193,10 +195,11 @@ def main():
         return [marks[i].elapsed_time(marks[i + 1]) / k for i in range(len(launches))], wall
 
     # In the first 15 ms of load after the GPU has been idle the MoR kernel, the one with the most arithmetic, goes
-    # through a transient: 48 us per launch at the start, up to 57 us between 2 and 8 ms, back at 48 us from 15 ms on,
-    # where it stays (kernel trace over 600 launches; the MX kernels stay at 42-44 us throughout).  A measurement of 20
-    # steps right after 5 warmup steps sits in the middle of it.  Those first 20 steps are timed for the record, and then
-    # untimed steps run for --preheat-ms before the W warmup steps: the timed region measures the sustained rate.
+    # through a transient: 48-49 us per launch at the start, 52-54 us between 3 and 6 ms, 47 us from 15 ms on, where it
+    # stays (after_idle_transient below records it with the shader clock and the power; the MX kernels stay at 42-44 us
+    # throughout).  A measurement of 20 steps right after 5 warmup steps sits in the middle of it.  Those first 20 steps
+    # are timed for the record, and then untimed steps run for --preheat-ms before the W warmup steps: the timed region
+    # measures the sustained rate.
     for _, fn, _ in launches:               # (the very first launch of a kernel also loads its code: not part of any figure)
         rotating(fn)
     first_ms, first_wall = timed_groups(20)
@@ -247,9 +250,17 @@ def main():
     x = x_mx
     del xs_mx, xs_mor, outs
 
+    transient = None
     extra = {}
     if not args.no_extra:
+        roofline["per_config"] = per_config_from_hbm(torch, run, _cabi, per_kernel, rows, cols)
+        roofline["mor_128x128_breakdown"] = mor_breakdown(torch, run, _cabi, rows, cols)
+        transient = after_idle_transient(torch, run, rows, cols)
         extra = other_configs(torch, run, _cabi, max(5, K // 2), max(2, W // 2))
+        c5 = extra.get("c5_llama3_8b_layer", {})
+        for fam in ("mor_128x128", "block_e4m3_128x128", "per_channel_rows_and_columns"):
+            if fam in c5:
+                roofline["per_config"]["c5_llama3_8b_layer_" + fam] = {k: c5[fam][k] for k in ("total_ms", "total_GB", "GBps", "frac")}
 
     cpu = None
     if not args.no_cpu:
@@ -264,15 +275,200 @@ def main():
                                f"plus MoR 128x128 (fp32 scale, error criterion) on a {rows}x{cols} N(0,1) tensor, per step; "
                                f"{ROT} buffer pairs in rotation",
                    "arithmetic": "bf16 tensors, fp32 / integer arithmetic, gfx950 fp8 / fp6 converts",
-                   "preheat": f"{preheat_steps} untimed steps ({args.preheat_ms:g} ms) before the {W} warmup steps: the first 15 ms of load after idle are "
-                              f"a transient of the MoR kernel (up to a fifth slower between 2 and 8 ms); the first 20 steps after idle took "
-                              f"{first_wall:.5f} ms each (per kernel: first_20_steps_after_idle), the timed steps are the sustained rate",
+                   "preheat": f"{preheat_steps} untimed steps ({args.preheat_ms:g} ms) before the {W} warmup steps: between 2 and 8 ms of load after idle the "
+                              f"MoR kernel runs up to a tenth slower (after_idle_transient: per-batch times with the shader clock and the power beside "
+                              f"them -- the clock stays within 4 % of 2.4 GHz throughout, the power sensor climbs from 300 W to 700 W over 60 ms); the "
+                              f"first 20 steps after idle took {first_wall:.5f} ms each (per kernel: first_20_steps_after_idle), the timed steps are "
+                              f"the sustained rate",
                    "elements_per_s": round(4 * nelem / (ms_per_step * 1e-3), 0), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "after_idle_transient": transient,
         "other_configs": extra,
     }
     print(json.dumps(line))
+
+
+def cold_launches(torch, make_fn, nbufs, target_ms=10.0, preheat_ms=30.0):
+    """ms per launch of fn(i), i rotating over nbufs buffer sets (so that nothing is found in the last-level cache),
+    over about target_ms of back-to-back launches after preheat_ms of untimed ones."""
+    fn = make_fn
+    i = 0
+    t_end = time.perf_counter() + preheat_ms * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(8):
+            fn(i % nbufs)
+            i += 1
+        torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(10):
+        fn(i % nbufs)
+        i += 1
+    b.record()
+    torch.cuda.synchronize()
+    n = max(10, min(2000, int(target_ms / (a.elapsed_time(b) / 10))))
+    a.record()
+    for _ in range(n):
+        fn(i % nbufs)
+        i += 1
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / n
+
+
+def rate_of(nbytes, nelem, ms):
+    return {"ms": round(ms, 5), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "elements_per_s": round(nelem / (ms * 1e-3), 0), "bytes": nbytes}
+
+
+def per_config_from_hbm(torch, run, cabi, per_kernel, rows, cols):
+    """Every BASELINE configuration with its data coming from HBM: tensors smaller than the 256 MB last-level cache
+    rotate over 6 buffer pairs.  C2 and MoR on the benchmark tensor are the timed step's own figures; C5 is added by
+    the layer sweep (its tensors are 8 to 470 MB each and follow one another)."""
+    res = {}
+    NB = 6
+    for k in ("mx_e4m3", "mx_e5m2", "mx_e2m3"):
+        res["c2_" + k + f"_{rows}x{cols}"] = {kk: per_kernel[k][kk] for kk in ("ms", "GBps", "frac", "bytes")}
+    res[f"mor_128x128_{rows}x{cols}_normal"] = {kk: per_kernel["mor_128x128"][kk] for kk in ("ms", "GBps", "frac", "bytes")}
+    # C1: per-tensor E4M3 on 4096 x 4096 N(0,1): with the caller's scale (one pass, 4 B/element) and with the tensor amax
+    # found on the GPU (block-scaling op, ss_mode 4: two reads and a write, 6 B/element)
+    g = torch.Generator(device="cuda").manual_seed(1001)
+    x1 = torch.randn(4096, 4096, device="cuda", generator=g).to(torch.bfloat16)
+    xs = [x1] + [x1.clone() for _ in range(NB - 1)]
+    outs = [torch.empty_like(x1) for _ in range(NB)]
+    m1 = torch.empty((32, 32), dtype=torch.int32, device="cuda")
+    scale = float(448.0 / x1.float().abs().max().item())
+    n = x1.numel()
+    res["c1_per_tensor_e4m3_4096x4096_callers_scale"] = rate_of(n * 4, n, cold_launches(torch, lambda i: run.fake_quantize(xs[i], outs[i], m1, 128, 128, scale, 4, 1), NB))
+    st1 = run.scaling_state(4096, 4096, 128, 128, False)
+    res["c1_per_tensor_e4m3_4096x4096_gpu_amax_ss4"] = rate_of(n * 6, n, cold_launches(torch, lambda i: run.block_scaling(xs[i], outs[i], st1, 128, 128, 0.045, 4), NB))
+    res["c1_per_tensor_e4m3_4096x4096_gpu_amax_ss4"]["note"] = "three dependent launches on a 32 MiB tensor; 6 B/element (4 B/element: frac x 2/3)"
+    del xs, outs, x1
+    # C3: per-row fp32 scale on the 16384 x 4096 weight matrix: fake_quantize (E4M3, E5M2) and the channel-scaling op the
+    # reference's callers use (ss_mode 3; amax, non-zero count, error sum and the bf16 fallback decision included)
+    g = torch.Generator(device="cuda").manual_seed(1003)
+    w = torch.randn(16384, 4096, device="cuda", generator=g) * 0.02
+    w[torch.randperm(16384, device="cuda", generator=g)[:164]] *= 100
+    w[7] = 0
+    w = w.to(torch.bfloat16)
+    ws = [w] + [w.clone() for _ in range(NB - 1)]
+    ows = [torch.empty_like(w) for _ in range(NB)]
+    mw = torch.empty((16384, 1), dtype=torch.int32, device="cuda")
+    n = w.numel()
+    res["c3_per_row_e4m3_16384x4096"] = rate_of(n * 4 + 16384 * 4, n, cold_launches(torch, lambda i: run.fake_quantize(ws[i], ows[i], mw, 1, 4096, 0.0, 2, 1), NB))
+    res["c3_per_row_e5m2_16384x4096"] = rate_of(n * 4 + 16384 * 4, n, cold_launches(torch, lambda i: run.fake_quantize(ws[i], ows[i], mw, 1, 4096, 0.0, 3, 1), NB))
+    st3 = run.scaling_state(16384, 4096, 1, 4096, True)
+    res["c3_per_row_e4m3_16384x4096_channel_op_ss3"] = rate_of(n * 4, n, cold_launches(torch, lambda i: run.block_scaling(ws[i], ows[i], st3, 1, 4096, 0.045, 3), NB))
+    del ws, ows, w
+    # C4: MoR 128 x 128 on the 16384 x 14336 tile mixture (470 MB: nothing of it is found in a cache)
+    x4 = gen_c4_gpu(torch, 16384, 14336)
+    o4 = torch.empty_like(x4)
+    m4 = torch.empty((128, 112), dtype=torch.int32, device="cuda")
+    n = x4.numel()
+    res["c4_mor_128x128_16384x14336_mixture"] = rate_of(n * 4 + m4.numel() * 4, n, cold_launches(torch, lambda i: run.fake_quantize(x4, o4, m4, 128, 128, 1e-15, 1, 1), 1))
+    torch.cuda.synchronize()
+    hist = torch.bincount(m4.flatten(), minlength=13).tolist()
+    res["c4_mor_128x128_16384x14336_mixture"]["meta_histogram"] = {str(i): h for i, h in enumerate(hist) if h}
+    return res
+
+
+def mor_breakdown(torch, run, cabi, rows, cols):
+    """What bounds the MoR 128 x 128 kernel on the benchmark tensor, all from HBM (6 buffer pairs in rotation): the
+    library's linear copy, a copy through the tile kernel's own walk (mor_block_format with MOR_FMT_COPY: every 128 x 128
+    tile read, its amax found, written back unchanged), block E4M3 on the same tiles, and MoR on a tensor whose tiles
+    are all decided by their range (no error pass) and on one whose tiles all take the error pass."""
+    NB = 6
+    g = torch.Generator(device="cuda").manual_seed(1001)
+    base = torch.randn(rows, cols, device="cuda", generator=g)
+    meta = torch.empty((rows // 128, cols // 128), dtype=torch.int32, device="cuda")
+    n = rows * cols
+    nb = n * 4 + meta.numel() * 4
+    res = {}
+
+    def bufs(t):
+        t = t.to(torch.bfloat16)
+        return [t] + [t.clone() for _ in range(NB - 1)]
+
+    xs = bufs(base)
+    outs = [torch.empty_like(xs[0]) for _ in range(NB)]
+    res["linear_copy_mode7"] = rate_of(nb, n, cold_launches(torch, lambda i: run.fake_quantize(xs[i], outs[i], meta, 128, 128, 0.0, 7, 1), NB))
+    res["tile_walk_copy_128x128"] = rate_of(n * 4, n, cold_launches(torch, lambda i: run.block_format(xs[i], outs[i], 128, 128, cabi.FMT_COPY, 1), NB))
+    res["block_e4m3_128x128"] = rate_of(nb, n, cold_launches(torch, lambda i: run.fake_quantize(xs[i], outs[i], meta, 128, 128, 0.0, 2, 1), NB))
+    res["mor_normal_data"] = rate_of(nb, n, cold_launches(torch, lambda i: run.fake_quantize(xs[i], outs[i], meta, 128, 128, 1e-15, 1, 1), NB))
+    torch.cuda.synchronize()
+    del xs
+    xs = bufs(torch.sign(base) * (base.abs() + 0.02))            # amax / amin of every tile below 114688: E4M3 by range
+    res["mor_every_tile_decided_by_range"] = rate_of(nb, n, cold_launches(torch, lambda i: run.fake_quantize(xs[i], outs[i], meta, 128, 128, 1e-15, 1, 1), NB))
+    del xs
+    t = base.clone()
+    t[::128, ::128] = 1e-6                                       # one tiny element per tile: every tile takes the error pass
+    xs = bufs(t)
+    del t
+    res["mor_every_tile_takes_the_error_pass"] = rate_of(nb, n, cold_launches(torch, lambda i: run.fake_quantize(xs[i], outs[i], meta, 128, 128, 1e-15, 1, 1), NB))
+    return res
+
+
+def after_idle_transient(torch, run, rows, cols):
+    """The first milliseconds of load after the GPU has been idle: 40 batches of 20 MoR launches (an event pair each) with
+    the shader clock and the board power read from sysfs by a host thread meanwhile (pp_dpm_sclk, hwmon power1_input)."""
+    import glob
+    import threading
+    dev = "/sys/class/drm/card0/device"
+    power_files = glob.glob(dev + "/hwmon/*/power1_input")
+
+    def read(path):
+        try:
+            with open(path) as f:
+                return f.read()
+        except OSError:
+            return ""
+
+    def sclk():
+        for line in read(dev + "/pp_dpm_sclk").splitlines():
+            if "*" in line:
+                return line.split(":")[1].replace("*", "").strip()
+        return None
+
+    g = torch.Generator(device="cuda").manual_seed(1001)
+    x = torch.randn(rows, cols, device="cuda", generator=g).to(torch.bfloat16)
+    xs = [x] + [x.clone() for _ in range(5)]
+    outs = [torch.empty_like(x) for _ in range(6)]
+    meta = torch.empty((rows // 128, cols // 128), dtype=torch.int32, device="cuda")
+    run.fake_quantize(xs[0], outs[0], meta, 128, 128, 1e-15, 1, 1)
+    torch.cuda.synchronize()
+    time.sleep(2.0)                                   # idle
+    samples, stop = [], [False]
+
+    def sampler():
+        while not stop[0]:
+            samples.append((time.perf_counter(), sclk(), read(power_files[0]).strip() if power_files else ""))
+
+    th = threading.Thread(target=sampler)
+    th.start()
+    time.sleep(0.01)
+    t0 = time.perf_counter()
+    pairs = []
+    for b in range(40):
+        a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(20):
+            run.fake_quantize(xs[(b * 20 + i) % 6], outs[(b * 20 + i) % 6], meta, 128, 128, 1e-15, 1, 1)
+        e.record()
+        pairs.append((a, e))
+    torch.cuda.synchronize()
+    stop[0] = True
+    th.join()
+    first = pairs[0][0]
+    batches = [{"start_ms": round(first.elapsed_time(a), 2), "us_per_launch": round(a.elapsed_time(e) / 20 * 1e3, 2)} for a, e in pairs]
+    series, last = [], None
+    for t, s, p in samples:
+        if (s, p) != last and t >= t0 - 0.005:
+            series.append({"t_ms": round((t - t0) * 1e3, 2), "sclk": s, "power_W": round(int(p) / 1e6, 0) if p.isdigit() else None})
+            last = (s, p)
+    slow = max(batches, key=lambda b: b["us_per_launch"])
+    return {"what": "MoR 128x128 launches back to back from an idle GPU, 20 per batch; sclk and power (the sensor's running average) from sysfs",
+            "batches": batches, "slowest_batch": slow, "last_batch": batches[-1], "sclk_and_power": series[:40]}
 
 
 def other_configs(torch, run, cabi, K, W):
@@ -588,6 +784,7 @@ def cpu_baseline(torch, x_gpu, x_mor_gpu):
     432-436) where that exists for the configuration."""
     from oracle import mor_oracle as O
     import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "tests"))          # the CPU leg restates the reference's torch emulation: test infrastructure
     import torch_emulation as E
     O.lib()
     torch.set_num_threads(os.cpu_count() or 1)
