@@ -97,3 +97,24 @@ def test_mutating_ops_have_no_fake_kernel():
             op.default(x, 64, 64, 1, 64, 0.045, 3)
     with pytest.raises((NotImplementedError, RuntimeError)):
         torch.ops.mor.fake_quantize_e8mx_inplace.default(x, 64, 64, 32, 32, 2, 1, x)
+
+
+def test_import_fails_loudly_without_the_host_library():
+    """libmor_torch.so is the only implementation behind the operators: when it is absent the import raises instead of
+    registering anything else (run in a child process that hides the file from os.path.exists)."""
+    import subprocess
+    import sys
+    code = (
+        "import os, sys\n"
+        "real = os.path.exists\n"
+        "os.path.exists = lambda p: False if str(p).endswith('libmor_torch.so') else real(p)\n"
+        "try:\n"
+        "    import mor\n"
+        "except ImportError as e:\n"
+        "    assert 'libmor_torch.so' in str(e), e\n"
+        "    sys.exit(42)\n"
+        "sys.exit(0)\n"
+    )
+    root = __import__("os").path.dirname(__import__("os").path.dirname(__import__("os").path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 42, (r.returncode, r.stderr[-400:])
