@@ -446,8 +446,27 @@ __device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
     asm("v_pk_min_u16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
     return r;
 }
+// Read as signed 16-bit integers the halves of a packed bf16 word have one smallest value, 0x8000: the bf16 -0.  A
+// running signed minimum over words therefore ends with a half of 0x8000 exactly when a -0 was among them: one
+// instruction per word to learn whether the sign bits of a group of words may be copied as they are.
+__device__ __forceinline__ uint32_t pk_min_i16(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_pk_min_i16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+constexpr uint32_t NEGZERO_INIT = 0x7FFF7FFFu;
+__device__ __forceinline__ void acc_negzero_pk(uint32_t& m, uint32_t w) { m = pk_min_i16(m, w); }
+__device__ __forceinline__ bool saw_negzero(uint32_t m) { return (m & 0xFFFFu) == 0x8000u || (m >> 16) == 0x8000u; }
 __device__ __forceinline__ uint32_t pk_sub_u16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, a) - __builtin_bit_cast(u16x2, b));
+}
+// a packed word with its -0 halves set to +0
+__device__ __forceinline__ uint32_t drop_negzero_pk(uint32_t w) {
+    const uint32_t nonzero = pk_min_u16(w & 0x7FFF7FFFu, 0x00010001u);        // 1 in each half that is not +-0
+    return w & ((nonzero << 15) | 0x7FFF7FFFu);
+}
+__device__ __forceinline__ uint4 drop_negzero_vec(uint4 v) {
+    return make_uint4(drop_negzero_pk(v.x), drop_negzero_pk(v.y), drop_negzero_pk(v.z), drop_negzero_pk(v.w));
 }
 __device__ __forceinline__ void acc_amax_pk(uint32_t& amax2, uint32_t w) { amax2 = pk_max_u16(amax2, w & 0x7FFF7FFFu); }
 __device__ __forceinline__ void acc_amin_pk(uint32_t& amin2_m1, uint32_t w) {

@@ -322,6 +322,9 @@ static int64_t col_words(int64_t rows, int64_t cols, int64_t brows) {
     return (rows / brows) * cols * 2 + (rows / brows) * p.P * cols / 2;
 }
 
+// Magnitudes leave bit 15 of each half of a partial word free.  In the first word of a column group those two bits
+// say what the group's 8 columns held in the rows the partial covers: a NaN, a -0.
+constexpr uint32_t COL_FLAG_NAN = 0x00008000u, COL_FLAG_NEGZERO = 0x80000000u, COL_FLAGS = COL_FLAG_NAN | COL_FLAG_NEGZERO;
 // a packed word with the halves that hold a NaN set to +0
 __device__ __forceinline__ uint32_t drop_nan_pk(uint32_t w) {
     const uint32_t lo = ((w & 0x7FFFu) > 0x7F80u) ? 0u : (w & 0xFFFFu), hi = ((w & 0x7FFF0000u) > 0x7F800000u) ? 0u : (w & 0xFFFF0000u);
@@ -349,6 +352,9 @@ __global__ __launch_bounds__(WG) void k_bs_colmax(const uint4* in, uint32_t* ws,
         uint32_t m[NG][4];
 #pragma unroll
         for (int g = 0; g < NG; ++g) { m[g][0] = 0; m[g][1] = 0; m[g][2] = 0; m[g][3] = 0; }
+        // what pass 2 wants to know about this lane's columns besides their maxima: whether one of them holds a NaN (then
+        // they take the exact arithmetic) or a -0 (then the sign bits are not copied blindly)
+        uint32_t negz2 = NEGZERO_INIT, flags = 0;
 #pragma unroll 1
         for (int64_t r = r_first; r < r_end; r += stride) {
             uint4 v[UN][NG];
@@ -369,12 +375,14 @@ __global__ __launch_bounds__(WG) void k_bs_colmax(const uint4* in, uint32_t* ws,
                 for (int u = 0; u < UN; ++u) {
                     acc_amax_pk(t[g][0], v[u][g].x); acc_amax_pk(t[g][1], v[u][g].y); acc_amax_pk(t[g][2], v[u][g].z); acc_amax_pk(t[g][3], v[u][g].w);
                     acc_nnz_pk(nz2, v[u][g].x); acc_nnz_pk(nz2, v[u][g].y); acc_nnz_pk(nz2, v[u][g].z); acc_nnz_pk(nz2, v[u][g].w);
+                    acc_negzero_pk(negz2, v[u][g].x); acc_negzero_pk(negz2, v[u][g].y); acc_negzero_pk(negz2, v[u][g].z); acc_negzero_pk(negz2, v[u][g].w);
                 }
             }
             uint32_t any = 0;
 #pragma unroll
             for (int g = 0; g < NG; ++g) any = pk_max_u16(any, pk_max_u16(pk_max_u16(t[g][0], t[g][1]), pk_max_u16(t[g][2], t[g][3])));
             if (amax_bits_of(any) > 0x7F800000u) {          // (rare)
+                flags |= COL_FLAG_NAN;
                 nz2 = 0;
 #pragma unroll
                 for (int g = 0; g < NG; ++g) {
@@ -395,22 +403,25 @@ __global__ __launch_bounds__(WG) void k_bs_colmax(const uint4* in, uint32_t* ws,
             nnz += (int)((nz2 & 0xFFFFu) + (nz2 >> 16));          // (at most 8 * UN * NG <= 128 per batch: the 16-bit counts cannot wrap)
         }
         // several rows per sweep (fewer than 256 groups): the lanes of one column group meet in LDS
+        if (saw_negzero(negz2)) flags |= COL_FLAG_NEGZERO;
         if (rps > 1) {
             __syncthreads();                       // the previous item's readers are done
-            s_m[tid] = make_uint4(m[0][0], m[0][1], m[0][2], m[0][3]);
+            s_m[tid] = make_uint4(m[0][0] | flags, m[0][1], m[0][2], m[0][3]);
             __syncthreads();
             if (rsub == 0) {
 #pragma unroll 1
                 for (int k = 1; k < rps; ++k) {
                     const uint4 o = s_m[(k << p.w_log) + cl];
-                    m[0][0] = pk_max_u16(m[0][0], o.x); m[0][1] = pk_max_u16(m[0][1], o.y); m[0][2] = pk_max_u16(m[0][2], o.z); m[0][3] = pk_max_u16(m[0][3], o.w);
+                    flags |= o.x & COL_FLAGS;
+                    m[0][0] = pk_max_u16(m[0][0], o.x & ~COL_FLAGS); m[0][1] = pk_max_u16(m[0][1], o.y); m[0][2] = pk_max_u16(m[0][2], o.z); m[0][3] = pk_max_u16(m[0][3], o.w);
                 }
             }
         }
         if (rsub == 0) {
+            // (the flags are the lane's: they ride in the two free top bits of the first word of each of its column groups)
             uint4* prow = reinterpret_cast<uint4*>(partial) + (seg * groups + slab * NG * WG + cl);
 #pragma unroll
-            for (int g = 0; g < NG; ++g) prow[g * WG] = make_uint4(m[g][0], m[g][1], m[g][2], m[g][3]);
+            for (int g = 0; g < NG; ++g) prow[g * WG] = make_uint4(m[g][0] | flags, m[g][1], m[g][2], m[g][3]);
         }
 #pragma unroll
         for (int g = 0; g < NG; ++g) gmax2 = pk_max_u16(gmax2, pk_max_u16(pk_max_u16(m[g][0], m[g][1]), pk_max_u16(m[g][2], m[g][3])));
@@ -428,36 +439,47 @@ __global__ __launch_bounds__(WG) void k_bs_colfold(const uint16_t* partial, floa
                                                    Shape sh, ColPlan p) {
     __shared__ float s_f[WAVES];
     __shared__ uint4 s_m[WAVES][FOLD_G];
+    __shared__ uint32_t s_flags[WAVES][FOLD_G];
     const float gamax = reduce_partial_amax(ws, npart1, s_f);
     const int tid = threadIdx.x, c = tid & (FOLD_G - 1), pl = tid / FOLD_G, lane = tid & 63, wave = tid >> 6;
     const int64_t groups = sh.cols >> 3, gw = (groups + FOLD_G - 1) / FOLD_G;
     const int64_t by = blockIdx.x / gw, cg0 = (blockIdx.x - by * gw) * FOLD_G, cg = cg0 + c;
     const uint4* prow = reinterpret_cast<const uint4*>(partial) + by * p.P * groups;
-    uint32_t m[4] = {0, 0, 0, 0};
+    uint32_t m[4] = {0, 0, 0, 0}, flags = 0;
     if (cg < groups) {
 #pragma unroll 8
         for (int k = pl; k < p.P; k += WG / FOLD_G) {
             const uint4 o = prow[k * groups + cg];
-            m[0] = pk_max_u16(m[0], o.x); m[1] = pk_max_u16(m[1], o.y); m[2] = pk_max_u16(m[2], o.z); m[3] = pk_max_u16(m[3], o.w);
+            flags |= o.x & COL_FLAGS;
+            m[0] = pk_max_u16(m[0], o.x & ~COL_FLAGS); m[1] = pk_max_u16(m[1], o.y); m[2] = pk_max_u16(m[2], o.z); m[3] = pk_max_u16(m[3], o.w);
         }
     }
 #pragma unroll
-    for (int off = FOLD_G; off < 64; off <<= 1)
+    for (int off = FOLD_G; off < 64; off <<= 1) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) m[j] = pk_max_u16(m[j], (uint32_t)__shfl_xor((int)m[j], off));
-    if (lane < FOLD_G) s_m[wave][lane] = make_uint4(m[0], m[1], m[2], m[3]);
+        flags |= (uint32_t)__shfl_xor((int)flags, off);
+    }
+    if (lane < FOLD_G) { s_m[wave][lane] = make_uint4(m[0], m[1], m[2], m[3]); s_flags[wave][lane] = flags; }
     __syncthreads();
     if (tid < 8 * FOLD_G) {                    // one thread per column
         const int g = tid >> 3, j = tid & 7;
-        uint32_t mb = 0;
+        uint32_t mb = 0, fl = 0;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) mb = max(mb, (uint32_t)reinterpret_cast<const uint16_t*>(&s_m[w][g])[j]);
+        for (int w = 0; w < WAVES; ++w) {
+            mb = max(mb, (uint32_t)reinterpret_cast<const uint16_t*>(&s_m[w][g])[j]);
+            fl |= s_flags[w][g];
+        }
         const float amax = u2f(mb << 16);
         Scale sc = make_scale(scaling_factor(gamax, amax, ss_mode));
         // a column of zeros (FQ:1063-1064: its scale is 448 / 1e-35, outside the fast range) gives +0 with any scale
         if (!(amax > 0.0f)) { sc.s = 1.0f; sc.r = 1.0f; sc.fast = true; }
+        // second word: the reciprocal; 0 = the column takes the exact arithmetic (scale outside the fast range, a NaN
+        // in the column group); negative = a -0 in the column group
+        float r = (sc.fast && !(fl & COL_FLAG_NAN)) ? sc.r : 0.0f;
+        if (fl & COL_FLAG_NEGZERO) r = -r;
         const int64_t col = (cg0 + g) * 8 + j;
-        if (col < sh.cols) scales[by * sh.cols + col] = make_float2(sc.s, sc.fast ? sc.r : 0.0f);
+        if (col < sh.cols) scales[by * sh.cols + col] = make_float2(sc.s, r);
     }
 }
 
@@ -565,8 +587,10 @@ __device__ __forceinline__ float rel_err_fast(float q, float a, float acc) {
 // No selects: a zero element's magnitude bits are 0; the sign of the input is kept for non-zero halves only (zero inputs come back as +0, FQ:1133-1134), through a
 // packed 16-bit mask.
 // ERR / OUT: whether the error terms / the output word are wanted (the in-place phases need one of them each).
+// NZ: whether the word may hold a -0.  Callers that know it does not (acc_negzero_pk over the words they hold, -0
+// halves cleared by drop_negzero_pk in the rare case) pass false, and the sign bits are copied as they are.
 // (`codes`: the register the convert writes half of, carried from word to word so that no fresh zero is needed)
-template <bool E8, bool ERR = true, bool OUT = true>
+template <bool E8, bool ERR = true, bool OUT = true, bool NZ = true>
 __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, float rs, float& err, uint32_t& codes) {
     const float a = fabsf(bf16_lo(w)), b = fabsf(bf16_hi(w));
     float qa, qb;
@@ -588,18 +612,23 @@ __device__ __forceinline__ uint32_t bs_pair_fast(uint32_t w, const Scale& sc, fl
         err = rel_err_fast(qb, b, err);
     }
     if constexpr (!OUT) return 0u;
+    if constexpr (!NZ) return store_pair<false>(qa, qb) | (w & 0x80008000u);
     const uint32_t nonzero = pk_min_u16(w & 0x7FFF7FFFu, 0x00010001u);        // 1 in each half that is not +-0
     return store_pair<false>(qa, qb) | (w & (nonzero << 15));
 }
-template <bool E8, bool ERR, bool OUT>
+template <bool E8, bool ERR, bool OUT, bool NZ = true>
 __device__ __forceinline__ uint4 bs_vec_fast(uint4 v, const Scale& sc, float& err) {
     uint4 q;
     uint32_t codes = 0;
-    q.x = bs_pair_fast<E8, ERR, OUT>(v.x, sc, sc.r, err, codes);
-    q.y = bs_pair_fast<E8, ERR, OUT>(v.y, sc, sc.r, err, codes);
-    q.z = bs_pair_fast<E8, ERR, OUT>(v.z, sc, sc.r, err, codes);
-    q.w = bs_pair_fast<E8, ERR, OUT>(v.w, sc, sc.r, err, codes);
+    q.x = bs_pair_fast<E8, ERR, OUT, NZ>(v.x, sc, sc.r, err, codes);
+    q.y = bs_pair_fast<E8, ERR, OUT, NZ>(v.y, sc, sc.r, err, codes);
+    q.z = bs_pair_fast<E8, ERR, OUT, NZ>(v.z, sc, sc.r, err, codes);
+    q.w = bs_pair_fast<E8, ERR, OUT, NZ>(v.w, sc, sc.r, err, codes);
     return q;
+}
+// whether one of a vector's 8 values is a -0 (4 instructions and a test)
+__device__ __forceinline__ bool vec_has_negzero(uint4 v) {
+    return saw_negzero(pk_min_i16(pk_min_i16(v.x, v.y), pk_min_i16(v.z, v.w)));
 }
 
 // pass 2 / pass 4: quantize every element with its block's scale (from the block's amax, per chunk, or per column in
@@ -640,8 +669,12 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
                 if (!EMU && sc.fast && !vec_has_nan(v)) {
                     const float rs = 1.0f / sc.s;
                     uint32_t codes = 0;
+                    if (WRITE && vec_has_negzero(v)) {          // (rare)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) w[j] = bs_pair_fast<E8, ERR, WRITE>(w[j], sc, rs, err, codes);
+                        for (int j = 0; j < 4; ++j) w[j] = drop_negzero_pk(w[j]);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) w[j] = bs_pair_fast<E8, ERR, WRITE, false>(w[j], sc, rs, err, codes);
                 } else {
 #pragma unroll 1
                     for (int j = 0; j < 4; ++j) {
@@ -693,9 +726,10 @@ __device__ __forceinline__ uint4 bs_cols_vec_exact(uint4 v, const float (&cs)[8]
     }
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
-template <bool WRITE, bool ERR>
+// (no NaN among the values: the columns that hold one are marked by k_bs_colfold and take the exact arithmetic;
+// NZ: whether a -0 may be among them, as in bs_pair_fast)
+template <bool WRITE, bool ERR, bool NZ>
 __device__ __forceinline__ uint4 bs_cols_vec_fast(uint4 v, const float (&cs)[8], const float (&cr)[8], float& err) {
-    if (vec_has_nan(v)) return bs_cols_vec_exact(v, cs, err);          // (rare)
     uint32_t w[4] = {v.x, v.y, v.z, v.w};
     float row_err = 0.0f;
     uint32_t codes = 0;
@@ -711,8 +745,12 @@ __device__ __forceinline__ uint4 bs_cols_vec_fast(uint4 v, const float (&cs)[8],
             row_err = rel_err_fast(qb, b, row_err);
         }
         if constexpr (WRITE) {
-            const uint32_t nonzero = pk_min_u16(w[j] & 0x7FFF7FFFu, 0x00010001u);
-            w[j] = store_pair<false>(qa, qb) | (w[j] & (nonzero << 15));
+            if constexpr (NZ) {
+                const uint32_t nonzero = pk_min_u16(w[j] & 0x7FFF7FFFu, 0x00010001u);
+                w[j] = store_pair<false>(qa, qb) | (w[j] & (nonzero << 15));
+            } else {
+                w[j] = store_pair<false>(qa, qb) | (w[j] & 0x80008000u);
+            }
         }
     }
     err += row_err;
@@ -758,17 +796,36 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint4* in, uint4* out
         uint4 va[4], vb[4];
         load_batch(va, r_first);
         const float cs[8] = {u2f(t0.x), u2f(t0.z), u2f(t1.x), u2f(t1.z), u2f(t2.x), u2f(t2.z), u2f(t3.x), u2f(t3.z)};
-        const float cr[8] = {u2f(t0.y), u2f(t0.w), u2f(t1.y), u2f(t1.w), u2f(t2.y), u2f(t2.w), u2f(t3.y), u2f(t3.w)};
-        bool fast = true;
+        const uint32_t crb[8] = {t0.y, t0.w, t1.y, t1.w, t2.y, t2.w, t3.y, t3.w};
+        bool fast = true, negz_lane = false;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) fast = fast && (cr[j] != 0.0f);
+        for (int j = 0; j < 8; ++j) { fast = fast && ((crb[j] & 0x7FFFFFFFu) != 0u); negz_lane = negz_lane || (crb[j] >> 31); }
+        const float cr[8] = {u2f(crb[0] & 0x7FFFFFFFu), u2f(crb[1] & 0x7FFFFFFFu), u2f(crb[2] & 0x7FFFFFFFu), u2f(crb[3] & 0x7FFFFFFFu),
+                             u2f(crb[4] & 0x7FFFFFFFu), u2f(crb[5] & 0x7FFFFFFFu), u2f(crb[6] & 0x7FFFFFFFu), u2f(crb[7] & 0x7FFFFFFFu)};
+        const bool negz = WRITE && __builtin_amdgcn_ballot_w64(negz_lane) != 0;            // uniform over the wave
         auto do_batch = [&](uint4 (&v)[4], int64_t r) {
             if (fast) {
+                if (negz) {
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const uint4 q = bs_cols_vec_fast<WRITE, ERR>(v[k], cs, cr, err);
-                    if constexpr (WRITE) {
-                        if (r + k * row_lanes < r_end) store16_rt(cout + (r + k * row_lanes) * row_stride, q, nt_out);
+                    for (int k = 0; k < 4; ++k) {
+                        opaque(v[k]);                  // one vector at a time: interleaved, the four take 165 registers
+                        uint4 q = bs_cols_vec_fast<WRITE, ERR, true>(v[k], cs, cr, err);
+                        opaque(q);
+                        if constexpr (ERR) asm volatile("" : "+v"(err));
+                        if constexpr (WRITE) {
+                            if (r + k * row_lanes < r_end) store16_rt(cout + (r + k * row_lanes) * row_stride, q, nt_out);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        opaque(v[k]);                  // one vector at a time: interleaved, the four take 165 registers
+                        uint4 q = bs_cols_vec_fast<WRITE, ERR, false>(v[k], cs, cr, err);
+                        opaque(q);
+                        if constexpr (ERR) asm volatile("" : "+v"(err));
+                        if constexpr (WRITE) {
+                            if (r + k * row_lanes < r_end) store16_rt(cout + (r + k * row_lanes) * row_stride, q, nt_out);
+                        }
                     }
                 }
             } else {
@@ -862,12 +919,14 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
         // unpacked magnitudes the quantize pass then uses again (measured faster for NV <= 2).
         constexpr bool PACKED = NV > 2;
         uint32_t amax_b, nnz2 = 0;
+        uint32_t negz2 = NEGZERO_INIT;            // whether this lane holds a -0 (its sign must not reach the output)
         if constexpr (PACKED) {
             uint32_t amax2 = 0;
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
                 acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
                 acc_nnz_pk(nnz2, v[k].x); acc_nnz_pk(nnz2, v[k].y); acc_nnz_pk(nnz2, v[k].z); acc_nnz_pk(nnz2, v[k].w);
+                acc_negzero_pk(negz2, v[k].x); acc_negzero_pk(negz2, v[k].y); acc_negzero_pk(negz2, v[k].z); acc_negzero_pk(negz2, v[k].w);
                 opaque(v[k]);
             }
             amax_b = group_umax(amax_bits_of(amax2), 64);
@@ -878,10 +937,12 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
             for (int k = 0; k < NV; ++k) {
                 acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
                 nnzf += nnz_word(v[k].x) + nnz_word(v[k].y) + nnz_word(v[k].z) + nnz_word(v[k].w);
+                acc_negzero_pk(negz2, v[k].x); acc_negzero_pk(negz2, v[k].y); acc_negzero_pk(negz2, v[k].z); acc_negzero_pk(negz2, v[k].w);
             }
             nnz2 = (uint32_t)nnzf;
             amax_b = group_umax(amax_bits_of(amax2), 64);
         }
+        const bool negz = saw_negzero(negz2);     // (rare) zeros leave as +0 (FQ:1133-1134): the lane clears its -0 first
         __syncthreads();                          // the previous block's readers of s_f are done
         if (lane == 0) s_f[wave] = u2f(amax_b);
         __syncthreads();
@@ -923,7 +984,8 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
 #pragma unroll
                 for (int k = 0; k < NV; ++k) {
                     if constexpr (PACKED) opaque(v[k]);
-                    uint4 q = bs_vec_fast<E8, false, true>(v[k], sc, err);
+                    if (negz) v[k] = drop_negzero_vec(v[k]);
+                    uint4 q = bs_vec_fast<E8, false, true, false>(v[k], sc, err);
                     if constexpr (PACKED) opaque(q);
                     if (ok[k]) store16_rt(out + base + off_k(k) + off_tid, q, nt);
                 }
@@ -931,7 +993,8 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
 #pragma unroll
                 for (int k = 0; k < NV; ++k) {
                     if constexpr (PACKED) opaque(v[k]);
-                    uint4 q = bs_vec_fast<E8, true, true>(v[k], sc, err);
+                    if (negz) v[k] = drop_negzero_vec(v[k]);
+                    uint4 q = bs_vec_fast<E8, true, true, false>(v[k], sc, err);
                     if constexpr (PACKED) { opaque(q); asm volatile("" : "+v"(err)); }
                     if (ok[k]) store16_rt(out + base + off_k(k) + off_tid, q, nt);
                 }
@@ -996,13 +1059,15 @@ __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* ou
         uint4 v[NVW];
 #pragma unroll
         for (int k = 0; k < NVW; ++k) v[k] = load16_rt(bin + 64 * k, nt_in);
-        uint32_t amax2 = 0, nnz2 = 0;
+        uint32_t amax2 = 0, nnz2 = 0, negz2 = NEGZERO_INIT;
 #pragma unroll
         for (int k = 0; k < NVW; ++k) {
             acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
             acc_nnz_pk(nnz2, v[k].x); acc_nnz_pk(nnz2, v[k].y); acc_nnz_pk(nnz2, v[k].z); acc_nnz_pk(nnz2, v[k].w);
+            acc_negzero_pk(negz2, v[k].x); acc_negzero_pk(negz2, v[k].y); acc_negzero_pk(negz2, v[k].z); acc_negzero_pk(negz2, v[k].w);
             opaque(v[k]);
         }
+        const bool negz = saw_negzero(negz2);     // (rare) zeros leave as +0 (FQ:1133-1134): the lane clears its -0 first
         const uint32_t amax_b = group_umax(amax_bits_of(amax2), 64);
         const bool has_nan = amax_b > 0x7F800000u;                  // uniform over the wave
         float amax = u2f(amax_b);
@@ -1027,7 +1092,8 @@ __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* ou
 #pragma unroll
                 for (int k = 0; k < NVW; ++k) {
                     opaque(v[k]);
-                    uint4 q = bs_vec_fast<E8, false, true>(v[k], sc, err);
+                    if (negz) v[k] = drop_negzero_vec(v[k]);
+                    uint4 q = bs_vec_fast<E8, false, true, false>(v[k], sc, err);
                     opaque(q);
                     store16_rt(bout + 64 * k, q, nt_out);
                 }
@@ -1035,7 +1101,8 @@ __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* ou
 #pragma unroll
                 for (int k = 0; k < NVW; ++k) {
                     opaque(v[k]);
-                    uint4 q = bs_vec_fast<E8, true, true>(v[k], sc, err);
+                    if (negz) v[k] = drop_negzero_vec(v[k]);
+                    uint4 q = bs_vec_fast<E8, true, true, false>(v[k], sc, err);
                     opaque(q);
                     asm volatile("" : "+v"(err));
                     store16_rt(bout + 64 * k, q, nt_out);
@@ -1113,9 +1180,10 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
             const Scale sc = GM == 2 ? scu : make_scale(scaling_factor(gamax, amax, ss_mode));
             float e = 0.0f;
             uint4 q;
+            if (phase != 1 && vec_has_negzero(v[k])) v[k] = drop_negzero_vec(v[k]);       // (rare) zeros leave as +0 (FQ:1133-1134)
             if (phase == 1) q = bs_vec_fast<E8, true, false>(v[k], sc, e);          // in place: decision pass,
-            else if (phase == 2) q = bs_vec_fast<E8, false, true>(v[k], sc, e);     // write pass
-            else q = bs_vec_fast<E8, true, true>(v[k], sc, e);
+            else if (phase == 2) q = bs_vec_fast<E8, false, true, false>(v[k], sc, e);     // write pass
+            else q = bs_vec_fast<E8, true, true, false>(v[k], sc, e);
             if (!has_nan && (sc.fast || !(amax > 0.0f))) {      // an all-zero block gives +0 whatever its (clamped) scale is
                 err += e;
                 if (c < nchunks && write) store16_rt(out + c, q, nt);

@@ -291,6 +291,34 @@ def test_scaling_denormal_elements(G, ss, shape):
     check_scaling(G, a, br, bc, 0.2, ss, channel, inplace=True)
 
 
+@pytest.mark.parametrize("ss", [1, 2, 3, 4])
+@pytest.mark.parametrize("shape", [(256, 256, 128, 128, False), (64, 4096, 1, 4096, True), (48, 2048, 1, 1024, True), (64, 512, 1, 32, True),
+                                   (512, 64, 128, 1, True), (96, 80, 32, 16, False), (2048, 256, 2048, 1, True), (1024, 4096, 512, 1, True),
+                                   (256, 1024, 64, 256, False)])
+def test_scaling_zeros_of_both_signs(G, ss, shape):
+    """Zeros leave as +0 whatever their sign (fake_quantize.cu:1133-1134) while a negative element that quantizes to zero
+    keeps its sign: a third of the elements are +0 or -0, some rows, columns and vectors hold nothing else, tiny negative
+    elements sit beside them, and one column group holds a NaN next to a -0."""
+    rows, cols, br, bc, channel = shape
+    a = uniform_bits(77 + ss, rows, cols, -200.0, 200.0)
+    rng = np.random.default_rng(rows * 3 + cols + ss)
+    u = rng.random((rows, cols))
+    a[u < 0.17] = 0x8000
+    a[(u >= 0.17) & (u < 0.33)] = 0x0000
+    tiny = (u >= 0.33) & (u < 0.40)
+    a[tiny] = 0x8000 | rng.integers(0x0080, 0x3000, int(tiny.sum())).astype(np.uint16)        # -1e-38 .. -5e-10
+    a[5, :] = 0x8000
+    a[:, 9] = np.where(rng.random(rows) < 0.5, 0x8000, 0).astype(np.uint16)
+    a[7, 16:24] = 0x8000
+    assert check_scaling(G, a, br, bc, 10.0, ss, channel) == 1
+    check_scaling(G, a, br, bc, 10.0, ss, channel, inplace=True)
+    a[11, 40] = 0x7FC0
+    a[12, 41] = 0x8000
+    out, meta, gamax, gnnz, gerr = G.block_scaling(a, br, bc, 10.0, ss, channel=channel)
+    want, wmeta, wamax, wnnz, werr = O.block_scaling(a, br, bc, 10.0, ss, channel=channel)
+    assert gnnz[0] == wnnz[0] and np.array_equal(out, want)
+
+
 def test_zz_no_case_was_within_the_threshold_window():
     """runs last in this file: how many of the cases above had a mean error within 1e-5 of the threshold"""
     print("scaling cases inside the 1e-5 threshold window:", len(IN_WINDOW), flush=True)
