@@ -68,6 +68,18 @@ __device__ __forceinline__ bool streams_in(int64_t bf16_elements) { return bf16_
 // (4096^2 with the caller's scale: 10.0 against 12.5 us).
 __device__ __forceinline__ bool streams_last_read(int64_t bf16_elements) { return bf16_elements >= ((int64_t)32 << 20); }
 __device__ __forceinline__ uint4 load16_rt(const uint4* p, bool nt) { return nt ? load16<true>(p) : load16<false>(p); }
+// N loads under one run-time choice of the policy.  Chosen load by load (load16_rt in an unrolled loop) every load
+// sits in a branch of its own, and the registers the two arms share are merged behind it: the compiler then waits for
+// each load before it issues the next one, and a wave has one request in flight instead of N.
+template <int N, class At> __device__ __forceinline__ void load16_group(uint4 (&v)[N], bool nt, At&& at) {
+    if (nt) {
+#pragma unroll
+        for (int k = 0; k < N; ++k) v[k] = load16<true>(at(k));
+    } else {
+#pragma unroll
+        for (int k = 0; k < N; ++k) v[k] = load16<false>(at(k));
+    }
+}
 
 // ---------------------------------------------------------------- bf16 <-> fp32
 // FQ:38-44: a bf16 is the upper half of an fp32.

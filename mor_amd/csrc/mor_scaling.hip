@@ -759,10 +759,12 @@ __device__ __forceinline__ uint4 bs_cols_vec_fast(uint4 v, const float (&cs)[8],
 
 // pass 2 / pass 4 for column blocks N x 1 with aligned rows: item = (strip, block row, workgroup of the Q that share
 // them), strips fastest.  A lane owns 8 adjacent columns: it loads their scales and reciprocals (k_bs_colfold) once and
-// takes every Q-th batch of 4 rows per row lane of the block, the next batch on its way while this one is quantized
-// (the arithmetic, 18 issue slots per element with the error term, overlaps the loads of the same wave; workgroups
-// that run side by side work on neighbouring rows).  Lanes whose scales are not all in the fast range use the exact
+// takes every Q-th batch of 4 rows per row lane of the block, two register buffers in turn (workgroups that run side
+// by side work on neighbouring rows).  Lanes whose scales are not all in the fast range use the exact
 // arithmetic.
+// (The loads of a batch sit in a branch -- the run-time cache policy, the bounds test of the last batch -- and are
+// waited for where it ends, so the two buffers do not in fact overlap loads with arithmetic.  With the policy fixed at
+// compile time and every load unconditional they do, and the kernel is slower: 47.9 against 45.3 us at 16384 x 4096.)
 template <bool WRITE, bool ERR>
 __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint4* in, uint4* out, uint32_t* ws, const float2* scales,
                                                      Finish fin, int gate, Shape sh, ColPlan p) {
@@ -787,10 +789,14 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint4* in, uint4* out
         const uint4* cin = in + cg;
         uint4* cout = out + cg;
         auto load_batch = [&](uint4 (&v)[4], int64_t r) {
+            if ((r - rl) + step <= r_end) {        // a whole batch (uniform over the workgroup): four loads in a row
+                load16_group(v, nt_in, [&](int k) { return cin + (r + k * row_lanes) * row_stride; });
+            } else {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                v[k] = make_uint4(0, 0, 0, 0);
-                if (r + k * row_lanes < r_end) v[k] = load16_rt(cin + (r + k * row_lanes) * row_stride, nt_in);
+                for (int k = 0; k < 4; ++k) {
+                    v[k] = make_uint4(0, 0, 0, 0);
+                    if (r + k * row_lanes < r_end) v[k] = load16_rt(cin + (r + k * row_lanes) * row_stride, nt_in);
+                }
             }
         };
         uint4 va[4], vb[4];
@@ -910,9 +916,16 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
         bool ok[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
+            // every lane loads: a lane beyond the block reads the block's first chunk and drops it (a load under a
+            // condition is waited for before the next one is issued: the registers of its two outcomes are merged behind it)
             ok[k] = FULL || (k * WGS + tid < nch);
-            v[k] = make_uint4(0, 0, 0, 0);
-            if (ok[k]) v[k] = in[base + off_k(k) + off_tid];
+            v[k] = in[base + (ok[k] ? off_k(k) + off_tid : 0u)];
+        }
+        if constexpr (!FULL) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                v[k].x = ok[k] ? v[k].x : 0u; v[k].y = ok[k] ? v[k].y : 0u; v[k].z = ok[k] ? v[k].z : 0u; v[k].w = ok[k] ? v[k].w : 0u;
+            }
         }
         // amax and the non-zero count.  Large blocks: on packed 16-bit magnitudes, the data staying packed in its
         // registers from pass to pass (NV = 8: 100 registers instead of 220).  Small blocks: float maxima, whose
@@ -1053,12 +1066,13 @@ __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* ou
     constexpr int ROW = 64 * NVW;                                   // chunks of a block
     float gmax = 0.0f, err = 0.0f;
     int nnz_total = 0;
+    // (Issuing a wave's next row before the arithmetic of the row it holds -- two register buffers in turn -- was measured
+    // slower: 56.3 against 52.5 us for 16384 rows of 4096 elements, at 168 registers.)
     for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < nrows; row += (int64_t)gridDim.x * WAVES) {
         const uint4* bin = in + row * ROW + lane;
         uint4* bout = out + row * ROW + lane;
         uint4 v[NVW];
-#pragma unroll
-        for (int k = 0; k < NVW; ++k) v[k] = load16_rt(bin + 64 * k, nt_in);
+        load16_group(v, nt_in, [&](int k) { return bin + 64 * k; });
         uint32_t amax2 = 0, nnz2 = 0, negz2 = NEGZERO_INIT;
 #pragma unroll
         for (int k = 0; k < NVW; ++k) {
@@ -1118,7 +1132,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* ou
                 if (write) out16[i] = store_bf16<false>(q);
             }
         }
-    }
+        }
     err = wave_sum(err);
     nnz_total = wave_sum_i(nnz_total);
     gmax = group_max(gmax, 64);
@@ -1457,7 +1471,8 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
     if (flat_ok && brows == 1 && ss_mode != 4 && (blk_chunks == 128 || blk_chunks == 256 || blk_chunks == 512)) {
         // row blocks of 1024, 2048 or 4096 elements: a wave per block
         if (global) tensor_amax_pass();
-        // (four workgroups per CU: 16384 rows of 4096 elements from HBM take 54.7 us with 1024 workgroups, 59 with 2048, 57.6 with 4096)
+        // (four workgroups per CU: 16384 rows of 4096 elements from HBM take 52.6 us with 1024 workgroups, 55.7 with 768,
+        // 55.1 with 1536, 54.9 with 2048, 53.4 with 4096)
         const int grid = (int)std::min<int64_t>(cdiv(nb, WAVES), 1024);
         fin.nerr = grid;
         fin.nstat = global ? npart1 : grid;
