@@ -42,37 +42,46 @@ __device__ __forceinline__ void acc_amax_nnz(float& amax, int& nnz, uint4 v) {
     nnz += nnz_word(v.x) + nnz_word(v.y) + nnz_word(v.z) + nnz_word(v.w);
 }
 
-// one workgroup's amax / nnz -> its slot of the partial arrays; returns the workgroup amax to every thread
-__device__ __forceinline__ float publish_partial(uint32_t* ws, float amax, int nnz, float* s_f, int* s_i) {
+// one workgroup's amax / nnz -> its slot of the partial arrays; returns the workgroup amax to every thread.
+// `special` (any thread): the workgroup saw a NaN or a -0.  An amax is not negative, so the flag rides in the sign bit
+// of the partial; every reader takes the magnitude.
+__device__ __forceinline__ float publish_partial(uint32_t* ws, float amax, int nnz, float* s_f, int* s_i, bool special = false) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     amax = group_max(amax, 64);
     nnz = wave_sum_i(nnz);
+    const bool wave_special = __builtin_amdgcn_ballot_w64(special) != 0;
     __syncthreads();
-    if (lane == 0) { s_f[wave] = amax; s_i[wave] = nnz; }
+    if (lane == 0) { s_f[wave] = wave_special ? -amax : amax; s_i[wave] = nnz; }
     __syncthreads();
-    const float a = fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+    const float a = fmaxf(fmaxf(fabsf(s_f[0]), fabsf(s_f[1])), fmaxf(fabsf(s_f[2]), fabsf(s_f[3])));
     if (threadIdx.x == 0) {
-        reinterpret_cast<float*>(ws)[WS_PAMAX + blockIdx.x] = a;
+        const uint32_t sign = (f2u(s_f[0]) | f2u(s_f[1]) | f2u(s_f[2]) | f2u(s_f[3])) & 0x80000000u;
+        ws[WS_PAMAX + blockIdx.x] = f2u(a) | sign;
         reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = s_i[0] + s_i[1] + s_i[2] + s_i[3];
     }
     return a;
 }
 
-// tensor amax from the pass-1 partials (every thread of the workgroup gets it)
-__device__ __forceinline__ float reduce_partial_amax(const uint32_t* ws, int npart, float* s_f) {
-    const float* pa = reinterpret_cast<const float*>(ws) + WS_PAMAX;
-    float a = 0.0f;
+// tensor amax from the pass-1 partials (every thread of the workgroup gets it); `special`: one of them carries the flag
+__device__ __forceinline__ float reduce_partial_amax(const uint32_t* ws, int npart, float* s_f, bool* special = nullptr) {
+    const uint32_t* pa = ws + WS_PAMAX;
+    uint32_t a = 0, sign = 0;                      // (magnitudes of non-negative floats order as integers)
 #pragma unroll 8
-    for (int i = threadIdx.x; i < npart; i += WG) a = fmaxf(a, pa[i]);
-    a = group_max(a, 64);
+    for (int i = threadIdx.x; i < npart; i += WG) { const uint32_t b = pa[i]; a = max(a, b & 0x7FFFFFFFu); sign |= b; }
+    a = group_umax(a, 64) | (__builtin_amdgcn_ballot_w64((sign >> 31) != 0) != 0 ? 0x80000000u : 0u);
     __syncthreads();
-    if ((threadIdx.x & 63) == 0) s_f[threadIdx.x >> 6] = a;
+    if ((threadIdx.x & 63) == 0) s_f[threadIdx.x >> 6] = u2f(a);
     __syncthreads();
-    return fmaxf(fmaxf(s_f[0], s_f[1]), fmaxf(s_f[2], s_f[3]));
+    const uint32_t b0 = f2u(s_f[0]), b1 = f2u(s_f[1]), b2 = f2u(s_f[2]), b3 = f2u(s_f[3]);
+    if (special) *special = ((b0 | b1 | b2 | b3) >> 31) != 0;
+    return u2f(max(max(b0 & 0x7FFFFFFFu, b1 & 0x7FFFFFFFu), max(b2 & 0x7FFFFFFFu, b3 & 0x7FFFFFFFu)));
 }
 
 // pass 1, blocks 1 x 8G as lane groups over the flat chunk array (FQ:1430-1457, 1611-1629).  A workgroup takes
 // tiles of 8 * 256 consecutive chunks, all loads of a tile in flight at once.  block_amax may be NULL (e8mx).
+// Without block maxima (the tensor-amax strategies that keep no per-block array, e8mx) the maxima and the count are
+// taken on packed 16-bit magnitudes, and the partial carries a flag when the workgroup saw a NaN or a -0, so that the
+// quantize pass of a tensor without either need not look for them again.
 __global__ __launch_bounds__(WG) void k_bs_amax_flat(const uint4* in, uint32_t* ws, float* block_amax,
                                                      int64_t nchunks, int G, int logG) {
     __shared__ float s_f[WAVES];
@@ -81,6 +90,45 @@ __global__ __launch_bounds__(WG) void k_bs_amax_flat(const uint4* in, uint32_t* 
     float gmax = 0.0f;
     int nnz = 0;
     const int64_t ntiles = (nchunks + NV * WG - 1) / (NV * WG);
+    if (!block_amax) {
+        uint32_t negz2 = NEGZERO_INIT;
+        bool special = false;
+        const bool nt = streams_in(nchunks * 8);
+        for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+            const int64_t base = tile * (NV * WG) + threadIdx.x;
+            uint4 v[NV];
+            if (base + (NV - 1) * WG < nchunks) {          // a whole tile for this lane: eight loads in a row
+                load16_group(v, nt, [&](int k) { return in + base + k * WG; });
+            } else {
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    v[k] = make_uint4(0, 0, 0, 0);
+                    if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, nt);
+                }
+            }
+            uint32_t amax2 = 0, nnz2 = 0;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
+                acc_nnz_pk(nnz2, v[k].x); acc_nnz_pk(nnz2, v[k].y); acc_nnz_pk(nnz2, v[k].z); acc_nnz_pk(nnz2, v[k].w);
+                acc_negzero_pk(negz2, v[k].x); acc_negzero_pk(negz2, v[k].y); acc_negzero_pk(negz2, v[k].z); acc_negzero_pk(negz2, v[k].w);
+            }
+            if (amax_bits_of(amax2) > 0x7F800000u) {      // a NaN among the lane's 64 values (rare): the float maximum and count skip it
+                special = true;
+                float amax = 0.0f;
+                int n = 0;
+#pragma unroll
+                for (int k = 0; k < NV; ++k) acc_amax_nnz(amax, n, v[k]);
+                gmax = fmaxf(gmax, amax);
+                nnz += n;
+            } else {
+                gmax = fmaxf(gmax, u2f(amax_bits_of(amax2)));
+                nnz += (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
+            }
+        }
+        publish_partial(ws, gmax, nnz, s_f, s_i, special || saw_negzero(negz2));
+        return;
+    }
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int64_t base = tile * (NV * WG) + threadIdx.x;
         uint4 v[NV];
@@ -541,7 +589,7 @@ __device__ __forceinline__ int finish_decision(const Finish& f, float* s_f, int*
 #pragma unroll 4
         for (int i = threadIdx.x; i < f.nerr; i += WG) acc += part[i];
 #pragma unroll 4
-        for (int i = threadIdx.x; i < f.nstat; i += WG) { a = fmaxf(a, pa[i]); n += pn[i]; }
+        for (int i = threadIdx.x; i < f.nstat; i += WG) { a = fmaxf(a, fabsf(pa[i])); n += pn[i]; }          // (sign bit: publish_partial's flag)
     }
     acc = wave_sum(acc);
     a = group_max(a, 64);
@@ -1161,17 +1209,59 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
     __shared__ float s_f[2 * WAVES];
     __shared__ int s_i[WAVES];
     if (phase == 2 && finish_decision(fin, s_f, s_i) != 1) return;          // phases as in k_bs_fused
-    const float gamax = GM != 0 ? reduce_partial_amax(ws, npart1, s_f) : 0.0f;
+    constexpr int NV = BS_ROWS_NV;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t ntiles = (nchunks + NV * WG - 1) / (NV * WG);
+    auto load_tile = [&](uint4 (&v)[NV], int64_t tile) {
+        const int64_t base = tile * (NV * WG) + tid;
+        if (base + (NV - 1) * WG < nchunks) {
+            load16_group(v, streams_last_read(nchunks * 8), [&](int k) { return in + base + k * WG; });
+        } else {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                v[k] = make_uint4(0, 0, 0, 0);
+                if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_last_read(nchunks * 8));
+            }
+        }
+    };
+    // One scale for the tensor: the first tile's loads go out before the partials of the pass that found the amax are
+    // reduced (about 2 us that every workgroup spends before it knows the scale)
+    uint4 v0[NV];
+    if (GM == 2 && (int64_t)blockIdx.x < ntiles) load_tile(v0, blockIdx.x);
+    bool special = false;                      // (a NaN or a -0 somewhere in the tensor, as the pass that found its amax saw it)
+    const float gamax = GM != 0 ? reduce_partial_amax(ws, npart1, s_f, &special) : 0.0f;
     __syncthreads();
     const Scale scu = make_scale(scaling_factor(gamax, 1.0f, 4));           // (GM == 2)
     const bool write = phase != 1;
-    constexpr int NV = BS_ROWS_NV;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool nt = streams_out(nchunks * 8);
     float gmax = 0.0f, err = 0.0f;
     int nnz = 0;
-    const int64_t ntiles = (nchunks + NV * WG - 1) / (NV * WG);
-    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    // ... in the fast range, and neither a NaN nor a -0 in the tensor: nothing to test per vector
+    const bool plain = GM == 2 && !special && scu.fast;
+    for (int64_t tile = blockIdx.x; plain && tile < ntiles; tile += gridDim.x) {
+        const int64_t base = tile * (NV * WG) + tid;
+        const bool whole = base + (NV - 1) * WG < nchunks;
+        uint4 v[NV];
+        if (tile == (int64_t)blockIdx.x) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) v[k] = v0[k];
+        } else {
+            load_tile(v, tile);
+        }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int64_t c = base + k * WG;
+            opaque(v[k]);
+            uint4 q;
+            if (phase == 1) q = bs_vec_fast<E8, true, false, false>(v[k], scu, err);
+            else if (phase == 2) q = bs_vec_fast<E8, false, true, false>(v[k], scu, err);
+            else q = bs_vec_fast<E8, true, true, false>(v[k], scu, err);
+            opaque(q);
+            asm volatile("" : "+v"(err));
+            if (write && (whole || c < nchunks)) store16_rt(out + c, q, nt);
+        }
+    }
+    for (int64_t tile = blockIdx.x; !plain && tile < ntiles; tile += gridDim.x) {
         const int64_t base = tile * (NV * WG) + tid;
         uint4 v[NV];
 #pragma unroll
@@ -1464,7 +1554,7 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
     const bool global = (ss_mode == 1 || ss_mode == 4);
     int npart1 = 0;
     auto tensor_amax_pass = [&]() {
-        npart1 = (int)std::min<int64_t>(cdiv(n / 8, 8 * WG), PASS1_MAX);
+        npart1 = (int)std::min<int64_t>(cdiv(n / 8, 8 * WG), 512);
         k_bs_amax_flat<<<npart1, WG, 0, st>>>(static_cast<const uint4*>(input), ws, nullptr, n / 8, 1, 0);
     };
     const bool flat_ok = !emu && vec && n % 8 == 0;
@@ -1530,7 +1620,9 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
     if (flat_ok && (ss_mode == 4 || (!col && brows == 1 && bcols % 8 == 0 && is_pow2(bcols / 8) && bcols / 8 <= 64))) {
         if (global) tensor_amax_pass();
         const int64_t nchunks = rows * cols / 8;
-        const int grid = (int)std::min<int64_t>(cdiv(nchunks, BS_ROWS_NV * WG), PASS2_MAX);
+        // (after a tensor-amax pass every workgroup starts by reducing that pass's partials, and the last kernel reduces this
+        // one's: 512 and 1024 of them instead of 1024 and 2048 take 1 us off the three launches at 4096^2, 2 us at 8192^2)
+        const int grid = (int)std::min<int64_t>(cdiv(nchunks, BS_ROWS_NV * WG), global ? 1024 : PASS2_MAX);
         fin.nerr = grid;
         fin.nstat = global ? npart1 : grid;
         const uint4* i4 = static_cast<const uint4*>(input);

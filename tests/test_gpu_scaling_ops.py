@@ -319,6 +319,28 @@ def test_scaling_zeros_of_both_signs(G, ss, shape):
     assert gnnz[0] == wnnz[0] and np.array_equal(out, want)
 
 
+@pytest.mark.parametrize("shape", [(256, 256, 128, 128, False), (64, 4096, 1, 4096, True), (96, 80, 32, 16, False), (1000, 1024, 8, 1024, False),
+                                   (2048, 256, 2048, 1, True), (512, 1024, 1, 32, True)])
+def test_scaling_tensor_scale_without_special_values(G, shape):
+    """ss_mode 4 on tensors that hold neither a NaN nor a -0 (the quantize pass then tests no vector for them), with and
+    without zeros, out of place and in place; then one -0, then one NaN, which must switch the tests back on."""
+    rows, cols, br, bc, channel = shape
+    a = uniform_bits(rows + 13 * cols, rows, cols, -60.0, 60.0)
+    a[a == 0x8000] = 0
+    check_scaling(G, a, br, bc, 0.045, 4, channel)
+    a[::3, ::5] = 0
+    a[2, :] = 0
+    check_scaling(G, a, br, bc, 0.045, 4, channel)
+    check_scaling(G, a, br, bc, 0.045, 4, channel, inplace=True)
+    check_scaling(G, a, br, bc, 0.001, 4, channel)
+    a[rows - 1, cols - 1] = 0x8000
+    check_scaling(G, a, br, bc, 0.045, 4, channel)
+    a[rows // 2, 3] = 0x7FC0
+    out, meta, gamax, gnnz, gerr = G.block_scaling(a, br, bc, 0.045, 4, channel=channel)
+    want, wmeta, wamax, wnnz, werr = O.block_scaling(a, br, bc, 0.045, 4, channel=channel)
+    assert gnnz[0] == wnnz[0] and gamax[0] == wamax[0] and np.array_equal(out, want)
+
+
 def test_zz_no_case_was_within_the_threshold_window():
     """runs last in this file: how many of the cases above had a mean error within 1e-5 of the threshold"""
     print("scaling cases inside the 1e-5 threshold window:", len(IN_WINDOW), flush=True)
