@@ -394,6 +394,12 @@ def mor_breakdown(torch, run, cabi, rows, cols):
     outs = [torch.empty_like(xs[0]) for _ in range(NB)]
     res["linear_copy_mode7"] = rate_of(nb, n, cold_launches(torch, lambda i: run.fake_quantize(xs[i], outs[i], meta, 128, 128, 0.0, 7, 1), NB))
     res["tile_walk_copy_128x128"] = rate_of(n * 4, n, cold_launches(torch, lambda i: run.block_format(xs[i], outs[i], 128, 128, cabi.FMT_COPY, 1), NB))
+    # the same copy through the same kernel (a block in a workgroup's registers, 8 vectors per lane) for blocks of other
+    # shapes with as many elements: 2 whole rows (32 KiB that lie together: a linear copy in thick workgroups) and
+    # 16 rows x 2 KiB; and for thin blocks of one row of 4096 elements (2 vectors per lane)
+    for name, br, bc in (("block_walk_copy_2x8192", 2, 8192), ("block_walk_copy_16x1024", 16, 1024), ("block_walk_copy_1x4096", 1, 4096)):
+        if rows % br == 0 and cols % bc == 0:
+            res[name] = rate_of(n * 4, n, cold_launches(torch, lambda i: run.block_format(xs[i], outs[i], br, bc, cabi.FMT_COPY, 1), NB))
     res["block_e4m3_128x128"] = rate_of(nb, n, cold_launches(torch, lambda i: run.fake_quantize(xs[i], outs[i], meta, 128, 128, 0.0, 2, 1), NB))
     res["mor_normal_data"] = rate_of(nb, n, cold_launches(torch, lambda i: run.fake_quantize(xs[i], outs[i], meta, 128, 128, 1e-15, 1, 1), NB))
     torch.cuda.synchronize()
