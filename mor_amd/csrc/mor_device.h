@@ -469,6 +469,12 @@ __device__ __forceinline__ uint32_t pk_min_i16(uint32_t a, uint32_t b) {
 constexpr uint32_t NEGZERO_INIT = 0x7FFF7FFFu;
 __device__ __forceinline__ void acc_negzero_pk(uint32_t& m, uint32_t w) { m = pk_min_i16(m, w); }
 __device__ __forceinline__ bool saw_negzero(uint32_t m) { return (m & 0xFFFFu) == 0x8000u || (m >> 16) == 0x8000u; }
+__device__ __forceinline__ uint32_t pk_lshr_u16(uint32_t a, int n) {          // both halves shifted right, nothing crosses
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, a) >> (unsigned short)n);
+}
+__device__ __forceinline__ uint32_t pk_mul_lo_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, a) * __builtin_bit_cast(u16x2, b));
+}
 __device__ __forceinline__ uint32_t pk_sub_u16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, a) - __builtin_bit_cast(u16x2, b));
 }

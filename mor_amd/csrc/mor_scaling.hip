@@ -43,38 +43,42 @@ __device__ __forceinline__ void acc_amax_nnz(float& amax, int& nnz, uint4 v) {
 }
 
 // one workgroup's amax / nnz -> its slot of the partial arrays; returns the workgroup amax to every thread.
-// `special` (any thread): the workgroup saw a NaN or a -0.  An amax is not negative, so the flag rides in the sign bit
-// of the partial; every reader takes the magnitude.
-__device__ __forceinline__ float publish_partial(uint32_t* ws, float amax, int nnz, float* s_f, int* s_i, bool special = false) {
+// An amax of bf16 values has 16 low zero bits as a float: two of them carry what the workgroup saw besides
+// (PART_SPECIAL: a NaN or a -0; PART_TINY: a non-zero magnitude below 2^-94, denormals included).  Every reader masks
+// them off; k_bs_amax_flat sets them, the other producers leave them 0 and their consumers do not ask.
+constexpr uint32_t PART_SPECIAL = 1u, PART_TINY = 2u, PART_FLAGS = 0xFFFFu;
+__device__ __forceinline__ float publish_partial(uint32_t* ws, float amax, int nnz, float* s_f, int* s_i, uint32_t flags = 0u) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     amax = group_max(amax, 64);
     nnz = wave_sum_i(nnz);
-    const bool wave_special = __builtin_amdgcn_ballot_w64(special) != 0;
+    const uint32_t wave_flags = (__builtin_amdgcn_ballot_w64((flags & PART_SPECIAL) != 0) != 0 ? PART_SPECIAL : 0u)
+                              | (__builtin_amdgcn_ballot_w64((flags & PART_TINY) != 0) != 0 ? PART_TINY : 0u);
     __syncthreads();
-    if (lane == 0) { s_f[wave] = wave_special ? -amax : amax; s_i[wave] = nnz; }
-    __syncthreads();
-    const float a = fmaxf(fmaxf(fabsf(s_f[0]), fabsf(s_f[1])), fmaxf(fabsf(s_f[2]), fabsf(s_f[3])));
-    if (threadIdx.x == 0) {
-        const uint32_t sign = (f2u(s_f[0]) | f2u(s_f[1]) | f2u(s_f[2]) | f2u(s_f[3])) & 0x80000000u;
-        ws[WS_PAMAX + blockIdx.x] = f2u(a) | sign;
-        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = s_i[0] + s_i[1] + s_i[2] + s_i[3];
-    }
-    return a;
-}
-
-// tensor amax from the pass-1 partials (every thread of the workgroup gets it); `special`: one of them carries the flag
-__device__ __forceinline__ float reduce_partial_amax(const uint32_t* ws, int npart, float* s_f, bool* special = nullptr) {
-    const uint32_t* pa = ws + WS_PAMAX;
-    uint32_t a = 0, sign = 0;                      // (magnitudes of non-negative floats order as integers)
-#pragma unroll 8
-    for (int i = threadIdx.x; i < npart; i += WG) { const uint32_t b = pa[i]; a = max(a, b & 0x7FFFFFFFu); sign |= b; }
-    a = group_umax(a, 64) | (__builtin_amdgcn_ballot_w64((sign >> 31) != 0) != 0 ? 0x80000000u : 0u);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) s_f[threadIdx.x >> 6] = u2f(a);
+    if (lane == 0) { s_f[wave] = u2f((f2u(amax) & ~PART_FLAGS) | wave_flags); s_i[wave] = nnz; }
     __syncthreads();
     const uint32_t b0 = f2u(s_f[0]), b1 = f2u(s_f[1]), b2 = f2u(s_f[2]), b3 = f2u(s_f[3]);
-    if (special) *special = ((b0 | b1 | b2 | b3) >> 31) != 0;
-    return u2f(max(max(b0 & 0x7FFFFFFFu, b1 & 0x7FFFFFFFu), max(b2 & 0x7FFFFFFFu, b3 & 0x7FFFFFFFu)));
+    const uint32_t a = max(max(b0 & ~PART_FLAGS, b1 & ~PART_FLAGS), max(b2 & ~PART_FLAGS, b3 & ~PART_FLAGS));       // (non-negative floats order as integers)
+    if (threadIdx.x == 0) {
+        ws[WS_PAMAX + blockIdx.x] = a | ((b0 | b1 | b2 | b3) & PART_FLAGS);
+        reinterpret_cast<int*>(ws)[WS_PNNZ + blockIdx.x] = s_i[0] + s_i[1] + s_i[2] + s_i[3];
+    }
+    return u2f(a);
+}
+
+// tensor amax from the pass-1 partials (every thread of the workgroup gets it); `flags`: the OR of the partials' flags
+__device__ __forceinline__ float reduce_partial_amax(const uint32_t* ws, int npart, float* s_f, uint32_t* flags = nullptr) {
+    const uint32_t* pa = ws + WS_PAMAX;
+    uint32_t a = 0, fl = 0;
+#pragma unroll 8
+    for (int i = threadIdx.x; i < npart; i += WG) { const uint32_t b = pa[i]; a = max(a, b & ~PART_FLAGS); fl |= b; }
+    a = group_umax(a, 64);
+    fl = (__builtin_amdgcn_ballot_w64((fl & PART_SPECIAL) != 0) != 0 ? PART_SPECIAL : 0u) | (__builtin_amdgcn_ballot_w64((fl & PART_TINY) != 0) != 0 ? PART_TINY : 0u);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s_f[threadIdx.x >> 6] = u2f(a | fl);
+    __syncthreads();
+    const uint32_t b0 = f2u(s_f[0]), b1 = f2u(s_f[1]), b2 = f2u(s_f[2]), b3 = f2u(s_f[3]);
+    if (flags) *flags = (b0 | b1 | b2 | b3) & PART_FLAGS;
+    return u2f(max(max(b0 & ~PART_FLAGS, b1 & ~PART_FLAGS), max(b2 & ~PART_FLAGS, b3 & ~PART_FLAGS)));
 }
 
 // pass 1, blocks 1 x 8G as lane groups over the flat chunk array (FQ:1430-1457, 1611-1629).  A workgroup takes
@@ -91,7 +95,7 @@ __global__ __launch_bounds__(WG) void k_bs_amax_flat(const uint4* in, uint32_t* 
     int nnz = 0;
     const int64_t ntiles = (nchunks + NV * WG - 1) / (NV * WG);
     if (!block_amax) {
-        uint32_t negz2 = NEGZERO_INIT;
+        uint32_t negz2 = NEGZERO_INIT, amin2 = AMIN2_INIT_M1;
         bool special = false;
         const bool nt = streams_in(nchunks * 8);
         for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
@@ -112,6 +116,7 @@ __global__ __launch_bounds__(WG) void k_bs_amax_flat(const uint4* in, uint32_t* 
                 acc_amax_pk(amax2, v[k].x); acc_amax_pk(amax2, v[k].y); acc_amax_pk(amax2, v[k].z); acc_amax_pk(amax2, v[k].w);
                 acc_nnz_pk(nnz2, v[k].x); acc_nnz_pk(nnz2, v[k].y); acc_nnz_pk(nnz2, v[k].z); acc_nnz_pk(nnz2, v[k].w);
                 acc_negzero_pk(negz2, v[k].x); acc_negzero_pk(negz2, v[k].y); acc_negzero_pk(negz2, v[k].z); acc_negzero_pk(negz2, v[k].w);
+                acc_amin_pk(amin2, v[k].x); acc_amin_pk(amin2, v[k].y); acc_amin_pk(amin2, v[k].z); acc_amin_pk(amin2, v[k].w);
             }
             if (amax_bits_of(amax2) > 0x7F800000u) {      // a NaN among the lane's 64 values (rare): the float maximum and count skip it
                 special = true;
@@ -126,7 +131,9 @@ __global__ __launch_bounds__(WG) void k_bs_amax_flat(const uint4* in, uint32_t* 
                 nnz += (int)((nnz2 & 0xFFFFu) + (nnz2 >> 16));
             }
         }
-        publish_partial(ws, gmax, nnz, s_f, s_i, special || saw_negzero(negz2));
+        // (amin_m1_of: fp32 bits of the smallest non-zero magnitude minus one bf16 step, low half ones)
+        const bool tiny = amin_m1_of(amin2) < ((33u << 23) - 1u);
+        publish_partial(ws, gmax, nnz, s_f, s_i, ((special || saw_negzero(negz2)) ? PART_SPECIAL : 0u) | (tiny ? PART_TINY : 0u));
         return;
     }
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
@@ -159,7 +166,7 @@ __global__ __launch_bounds__(WG) void k_amax_scalar(const uint16_t* in, uint32_t
     float amax = 0.0f;
     for (int64_t i = (int64_t)blockIdx.x * WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * WG)
         amax = fmaxf(amax, fabsf(bf16_one(in[i])));
-    publish_partial(ws, amax, 0, s_f, s_i);
+    publish_partial(ws, amax, 0, s_f, s_i, PART_SPECIAL | PART_TINY);          // (nothing was looked for: consumers assume the worst)
 }
 
 // pass 1, one workgroup per block of any shape (FQ:951-1015), blocks taken grid-stride;
@@ -589,7 +596,7 @@ __device__ __forceinline__ int finish_decision(const Finish& f, float* s_f, int*
 #pragma unroll 4
         for (int i = threadIdx.x; i < f.nerr; i += WG) acc += part[i];
 #pragma unroll 4
-        for (int i = threadIdx.x; i < f.nstat; i += WG) { a = fmaxf(a, fabsf(pa[i])); n += pn[i]; }          // (sign bit: publish_partial's flag)
+        for (int i = threadIdx.x; i < f.nstat; i += WG) { a = fmaxf(a, u2f(f2u(pa[i]) & ~PART_FLAGS)); n += pn[i]; }          // (low bits: publish_partial's flags)
     }
     acc = wave_sum(acc);
     a = group_max(a, 64);
@@ -1228,8 +1235,9 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
     // reduced (about 2 us that every workgroup spends before it knows the scale)
     uint4 v0[NV];
     if (GM == 2 && (int64_t)blockIdx.x < ntiles) load_tile(v0, blockIdx.x);
-    bool special = false;                      // (a NaN or a -0 somewhere in the tensor, as the pass that found its amax saw it)
-    const float gamax = GM != 0 ? reduce_partial_amax(ws, npart1, s_f, &special) : 0.0f;
+    uint32_t pflags = 0;
+    const float gamax = GM != 0 ? reduce_partial_amax(ws, npart1, s_f, &pflags) : 0.0f;
+    const bool special = (pflags & PART_SPECIAL) != 0;          // a NaN or a -0 somewhere in the tensor, as the pass that found its amax saw it
     __syncthreads();
     const Scale scu = make_scale(scaling_factor(gamax, 1.0f, 4));           // (GM == 2)
     const bool write = phase != 1;
@@ -1406,14 +1414,56 @@ template <int MB, bool UNIT> __device__ __forceinline__ float e8mx_element(float
     }
 }
 
+// The rounding of quant_e8m in closed form.  With h = the mantissa in bf16 steps, rounded up (the threshold tables look at
+// nothing finer), the count of thresholds below the mantissa is h / S rounded to nearest, ties to even, S = 2^(7-MB); a
+// carry out of the mantissa is the exponent's increment.  So on hb = (e << 7) + h, the value's bf16 bit pattern rounded
+// up: (hb + S/2 - 1 + bit LS of hb) with the low LS bits cleared.  Holds for 0 < e < 255 and for zero; e = 0 gives 0 in
+// the reference (the callers see to that), a result of e = 255 is the reference's clamp to the largest finite value.
+//
+// Scale 1 (no tensor-amax strategy): the input is bf16, so hb is its magnitude and the result is again a bf16 pattern --
+// both halves of a packed word at once, no conversion to float.  Vectors with a NaN, an infinity (passed through by
+// the reference, FQ:1243-1327) or a -0 (zeros leave as +0, FQ:1399-1419) take the element-wise code.
+template <int MB> __device__ __forceinline__ uint32_t e8mx_pair_unit(uint32_t w) {
+    constexpr int LS = 7 - MB;
+    constexpr uint32_t S = 1u << LS, MAXF = (254u << 7) | (((1u << MB) - 1u) << LS);
+    const uint32_t mag = w & 0x7FFF7FFFu;
+    const uint32_t odd = (mag >> LS) & 0x00010001u;                       // (bits that cross from the upper half are masked off)
+    uint32_t r = (mag + (S / 2 - 1) * 0x00010001u + odd) & ~((S - 1) * 0x00010001u);          // (no carry out of a half: 0x7F7F + 32)
+    r = pk_min_u16(r, MAXF * 0x00010001u);
+    const uint32_t normal = pk_min_u16(pk_lshr_u16(mag, 7), 0x00010001u);                       // 1 where the exponent field is not 0
+    r = pk_mul_lo_u16(r, normal);                                           // denormals give 0 (the sign stays: FQ keeps it)
+    return r | (w & 0x80008000u);
+}
+// whether a vector holds a value the packed form does not cover: a magnitude of 0x7F80 or more (infinity, NaN), a -0
+__device__ __forceinline__ bool e8mx_vec_special(uint4 v) {
+    uint32_t m = 0;
+    acc_amax_pk(m, v.x); acc_amax_pk(m, v.y); acc_amax_pk(m, v.z); acc_amax_pk(m, v.w);
+    return amax_bits_of(m) >= 0x7F800000u || vec_has_negzero(v);
+}
+// Tensor-amax strategy on a tensor the amax pass found plain (no NaN, no -0, no non-zero magnitude below 2^-94, amax below
+// 2^96, Markstein's condition on the scale): |x| * sf, the closed form on its bits, the exact quotient by sf, half-up
+// store; the sign bits are copied.  Nothing is tested per element.
+template <int MB> __device__ __forceinline__ uint32_t e8mx_pair_plain(uint32_t w, float sf, float rs) {
+    constexpr int LS = 7 - MB;
+    constexpr uint32_t S = 1u << LS;
+    const uint32_t b0 = f2u(fabsf(bf16_lo(w)) * sf), b1 = f2u(fabsf(bf16_hi(w)) * sf);
+    const uint32_t h0 = (b0 + 0xFFFFu) >> 16, h1 = (b1 + 0xFFFFu) >> 16;
+    const float d0 = u2f(((h0 + (S / 2 - 1) + ((h0 >> LS) & 1u)) & ~(S - 1)) << 16);
+    const float d1 = u2f(((h1 + (S / 2 - 1) + ((h1 >> LS) & 1u)) & ~(S - 1)) << 16);
+    return store_pair<false>(div_by_scale(d0, sf, rs), div_by_scale(d1, sf, rs)) | (w & 0x80008000u);
+}
+
 // FQ:1361-1428
 template <int MB, bool EMU, bool UNIT>
 __global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, const uint32_t* ws, int npart, int strategy, int64_t n, int64_t nvec) {
     __shared__ float s_f[WAVES];
-    const float gamax = (!UNIT && strategy == 1) ? reduce_partial_amax(ws, npart, s_f) : 0.0f;
+    uint32_t pflags = PART_SPECIAL | PART_TINY;
+    const float gamax = (!UNIT && strategy == 1) ? reduce_partial_amax(ws, npart, s_f, &pflags) : 0.0f;
     const float sf = UNIT ? 1.0f : e8mx_scale<MB>(gamax, strategy);
     const float rs = 1.0f / sf;
     const bool mk = (f2u(sf) & 0x7FFFFFu) != 0x7FFFFFu;
+    // (amax at least 2^-60: the scaled values of a tensor without tiny elements are then nowhere near the denormals either)
+    const bool plain = !UNIT && !EMU && strategy == 1 && pflags == 0 && mk && gamax < 0x1p96f && gamax >= 0x1p-60f;
     const int64_t stride = (int64_t)gridDim.x * WG;
     const int64_t gtid = (int64_t)blockIdx.x * WG + threadIdx.x;
     const uint4* in4 = reinterpret_cast<const uint4*>(in);
@@ -1428,9 +1478,17 @@ __global__ __launch_bounds__(WG) void k_e8mx(const uint16_t* in, uint16_t* out, 
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+            if (UNIT && !EMU && !e8mx_vec_special(v[k])) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                w[j] = store_pair<EMU>(e8mx_element<MB, UNIT>(bf16_lo(w[j]), sf, rs, mk), e8mx_element<MB, UNIT>(bf16_hi(w[j]), sf, rs, mk));
+                for (int j = 0; j < 4; ++j) w[j] = e8mx_pair_unit<MB>(w[j]);
+            } else if (plain) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w[j] = e8mx_pair_plain<MB>(w[j], sf, rs);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    w[j] = store_pair<EMU>(e8mx_element<MB, UNIT>(bf16_lo(w[j]), sf, rs, mk), e8mx_element<MB, UNIT>(bf16_hi(w[j]), sf, rs, mk));
+            }
             if (c0 + k * WG < nvec) store16_rt(out4 + c0 + k * WG, make_uint4(w[0], w[1], w[2], w[3]), streams_out(n));
         }
     }

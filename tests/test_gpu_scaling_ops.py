@@ -187,6 +187,38 @@ def test_e8mx(G, qt, strategy):
         assert np.array_equal(G.e8mx(small, 32, 32, qt, 3), E.e8mx_tensor(small, qt))
 
 
+@pytest.mark.parametrize("qt", [1, 2, 3])
+def test_e8mx_closed_form_paths(G, qt):
+    """The two forms of the e8mx kernel that test nothing per element.  Scale 1: every 16-bit pattern (vectors that
+    hold a NaN, an infinity or a -0 take the element-wise code, their neighbours the packed one).  Tensor amax: tensors
+    the amax pass finds plain, over a range of magnitudes, and the same tensors with one tiny element, one -0, one NaN,
+    which must send them back to the element-wise code; an amax of 2^96 and more, an all-zero tensor."""
+    every = np.arange(0x10000, dtype=np.uint32).astype(np.uint16)
+    rng = np.random.default_rng(qt)
+    every = np.concatenate([every, rng.permutation(every)]).reshape(-1, 512)
+    print("e8mx unit, every pattern", qt, flush=True)
+    want = O.e8mx(every, 32, 32, qt, 3)
+    got = G.e8mx(every, 32, 32, qt, 3)
+    nan = (every & 0x7FFF) > 0x7F80
+    assert np.array_equal(got[~nan], want[~nan]) and ((got[nan] & 0x7FFF) > 0x7F80).all()
+    for scale in (1e-20, 3e-5, 1.0, 777.0, 1e20, 5e28, 2e29, 1e33):
+        x = (rng.standard_normal((384, 1024)) * scale).astype(np.float32)
+        x[rng.random(x.shape) < 0.05] = 0.0
+        a = ((x.view(np.uint32) + 0x8000) >> 16).astype(np.uint16)
+        a[a == 0x8000] = 0
+        tiny = ((a & 0x7FFF) != 0) & ((a & 0x7FFF) < (33 << 7))
+        a[tiny] = 0
+        print("e8mx tensor amax", qt, scale, flush=True)
+        assert np.array_equal(G.e8mx(a, 32, 32, qt, 1), O.e8mx(a, 32, 32, qt, 1))
+        assert np.array_equal(G.e8mx(a, 32, 32, qt, 1, inplace=True), O.e8mx(a, 32, 32, qt, 1))
+        for special in (0x0001, 0x1040, 0x8000, 0x9000):            # a denormal, 2^-95, -0, a negative tiny value
+            b = a.copy()
+            b[7, 33] = special
+            assert np.array_equal(G.e8mx(b, 32, 32, qt, 1), O.e8mx(b, 32, 32, qt, 1)), hex(special)
+    z = np.zeros((64, 512), np.uint16)
+    assert np.array_equal(G.e8mx(z, 32, 32, qt, 1), O.e8mx(z, 32, 32, qt, 1))
+
+
 @pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2, O.E3M2, O.E2M3])
 def test_quant_dequant_ops(G, fmt):
     rng = np.random.default_rng(fmt)
