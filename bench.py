@@ -514,6 +514,13 @@ def other_configs(torch, run, cabi, K, W):
                                                                          meta_t.data_ptr(), 8192, 8192, 1e-15, mode, 1, st_())), n * 6, n)
     del out_t
     mor_tile_codes(torch, cabi, run, add, x, out, "8192x8192_normal")
+    # E8M2 rounding (mor_e8mx): without a scale (one pass, 4 B/element) and with the tensor-amax strategy (a pass that
+    # finds the amax, then the quantize pass: 6 B/element)
+    nb8 = run.L.mor_workspace_bytes(cabi.OP_E8MX, 8192, 8192, 32, 32)
+    ws8 = torch.empty(max(nb8, 4), dtype=torch.uint8, device="cuda")
+    for strat, key, bpe in ((3, "e8m2_no_scale_8192x8192", 4), (1, "e8m2_tensor_amax_8192x8192", 6)):
+        add(key, lambda: cabi.check(run.L.mor_e8mx(x.data_ptr(), out.data_ptr(), 8192, 8192, 32, 32, 2, strat, ws8.data_ptr(), nb8, 0, st_())), n * bpe, n)
+    del ws8
     # C1: per-tensor E4M3, 4096x4096, scale from the tensor amax (the quantize pass only: 4 B/element)
     x1 = x[:4096, :4096].contiguous()
     o1 = torch.empty_like(x1)
