@@ -370,8 +370,10 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
     write_transposed(meta_val);
 }
 
+// (MoR on blocks of 16 vectors per lane -- 256 x 256 tiles in 512 threads -- is held to 128 registers: at the 136 it takes
+// otherwise one workgroup fills a CU and nothing overlaps its phases; 8192^2: 60.6 -> 56.7 us)
 template <bool MOR, bool E8, int NV, bool FULL, int NT, int WGS = WG, bool GATHER = false, bool DUAL = false, bool WIRE = false>
-__global__ __launch_bounds__(WGS) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
+__global__ __launch_bounds__(WGS) __attribute__((amdgpu_waves_per_eu((MOR && NV == 16) ? 4 : 1, 8))) void k_wgblock(const uint4* in, uint4* out, int32_t* __restrict__ meta,
                                                  float* __restrict__ stats, Shape sh, QuantArgs qa, int cpr, int cpr_shift,
                                                  int64_t first, uint4* out_t, int32_t* __restrict__ meta_t) {
     // Workgroup -> block.  cpr_shift bit 8 (large tensors whose block grid is a multiple of 8 wide): consecutive
