@@ -707,7 +707,7 @@ __global__ __launch_bounds__(WG) void k_bs_quant(const uint16_t* in, uint16_t* o
         for (uint32_t c = blockIdx.x * WG + threadIdx.x; c < nchunks; c += gridDim.x * WG) {
             const uint32_t row = div_u32(c, d_rowchunks), cc = c - row * row_chunks;
             const uint32_t by = div_u32(row, d_brows);
-            uint4 v = load16_rt(in4 + c, streams_last_read(sh.rows * sh.cols));
+            uint4 v = load16_rt(in4 + c, WRITE && streams_last_read(sh.rows * sh.cols));
             uint32_t w[4] = {v.x, v.y, v.z, v.w};
             if constexpr (COL) {
                 const int64_t sp = (int64_t)by * sh.cols + (int64_t)cc * 8;
@@ -829,7 +829,9 @@ __global__ __launch_bounds__(WG) void k_bs_quant_col(const uint4* in, uint4* out
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cl = tid & ((1 << p.cg_log) - 1), rl = tid >> p.cg_log, row_lanes = WG >> p.cg_log;
     const int64_t row_stride = sh.cols >> 3, groups = row_stride;
-    const bool nt_in = streams_last_read(sh.rows * sh.cols), nt_out = streams_out(sh.rows * sh.cols);
+    // (the decision pass of the in-place op is not the last read: its loads allocate, and the write pass finds what
+    // the last-level cache kept of the tensor)
+    const bool nt_in = WRITE && streams_last_read(sh.rows * sh.cols), nt_out = streams_out(sh.rows * sh.cols);
     float err = 0.0f;
     for (int64_t item = blockIdx.x; item < p.items2; item += gridDim.x) {
         const int64_t pid = item / p.strips, strip = item - pid * p.strips;
@@ -950,6 +952,7 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
     const uint32_t row_stride = (uint32_t)(sh.cols >> 3);
     const int nch = (int)sh.brows * cpr;
     const bool nt = streams_out(sh.rows * sh.cols);
+    const bool nt_in = phase != 1 && streams_last_read(sh.rows * sh.cols);          // (the decision pass of the in-place op is not the last read)
     const bool bands = (cpr_shift & 256) != 0;      // XCD bands of block columns, as in k_wgblock (gx and the grid multiples of 8)
     cpr_shift &= 255;
     // chunk k * 256 + tid of a block is at off_k(k) + off_tid; cpr is a power of two, so off_k is uniform (no per-lane
@@ -970,12 +973,10 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
         uint4 v[NV];
         bool ok[NV];
 #pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            // every lane loads: a lane beyond the block reads the block's first chunk and drops it (a load under a
-            // condition is waited for before the next one is issued: the registers of its two outcomes are merged behind it)
-            ok[k] = FULL || (k * WGS + tid < nch);
-            v[k] = in[base + (ok[k] ? off_k(k) + off_tid : 0u)];
-        }
+        for (int k = 0; k < NV; ++k) ok[k] = FULL || (k * WGS + tid < nch);
+        // every lane loads: a lane beyond the block reads the block's first chunk and drops it (a load under a
+        // condition is waited for before the next one is issued: the registers of its two outcomes are merged behind it)
+        load16_group(v, nt_in, [&](int k) { return in + base + (ok[k] ? off_k(k) + off_tid : 0u); });
         if constexpr (!FULL) {
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
@@ -1117,7 +1118,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* ou
     __syncthreads();
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool write = phase != 1;
-    const bool nt_out = streams_out(sh.rows * sh.cols), nt_in = streams_last_read(sh.rows * sh.cols);
+    const bool nt_out = streams_out(sh.rows * sh.cols), nt_in = phase != 1 && streams_last_read(sh.rows * sh.cols);       // (phase 1 is not the last read)
     constexpr int ROW = 64 * NVW;                                   // chunks of a block
     float gmax = 0.0f, err = 0.0f;
     int nnz_total = 0;
@@ -1222,12 +1223,12 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
     auto load_tile = [&](uint4 (&v)[NV], int64_t tile) {
         const int64_t base = tile * (NV * WG) + tid;
         if (base + (NV - 1) * WG < nchunks) {
-            load16_group(v, streams_last_read(nchunks * 8), [&](int k) { return in + base + k * WG; });
+            load16_group(v, phase != 1 && streams_last_read(nchunks * 8), [&](int k) { return in + base + k * WG; });
         } else {
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
                 v[k] = make_uint4(0, 0, 0, 0);
-                if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_last_read(nchunks * 8));
+                if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, phase != 1 && streams_last_read(nchunks * 8));
             }
         }
     };
@@ -1275,7 +1276,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused_rows(const uint4* in, uint4* ou
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             v[k] = make_uint4(0, 0, 0, 0);
-            if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, streams_last_read(nchunks * 8));
+            if (base + k * WG < nchunks) v[k] = load16_rt(in + base + k * WG, phase != 1 && streams_last_read(nchunks * 8));
         }
         uint32_t slow = 0, nnz2 = 0;
 #pragma unroll
