@@ -2,6 +2,7 @@
 // "FQ" below is the reference file mor/csrc/cuda/fake_quantize.cu.
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 #include <algorithm>
 #include <atomic>
@@ -232,11 +233,27 @@ __global__ __launch_bounds__(WG) void k_bs_amax_sub(const uint4* in, uint32_t* w
         if (bid < nb) {
             const uint32_t by = div_u32(bid, d_gx), bx = bid - by * (uint32_t)sh.gx;
             const uint4* bin = in + ((int64_t)by * sh.brows * row_stride + (((int64_t)bx * sh.bcols) >> 3));
-#pragma unroll 4
-            for (uint32_t j = l; j < nchb; j += (uint32_t)L) {
-                const uint32_t r = div_u32(j, d_cpr), cc = j - r * cpr;
-                acc_amax_nnz(amax, nnz, load16_rt(bin + r * row_stride + cc, nt));
-            }
+            // Four loads at a time, unconditional (a chunk beyond the block reads the lane's first chunk again and counts
+            // as zeros), under one choice of the cache policy: loads chosen or bounded one by one are each waited for
+            // before the next is issued.
+            auto scan = [&](auto streaming) {
+#pragma unroll 1
+                for (uint32_t j = l; j < nchb; j += 4u * (uint32_t)L) {
+                    uint4 v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const uint32_t jj = j + (uint32_t)u * (uint32_t)L, js = jj < nchb ? jj : l;
+                        const uint32_t r = div_u32(js, d_cpr), cc = js - r * cpr;
+                        v[u] = load16<decltype(streaming)::value>(bin + r * row_stride + cc);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (j + (uint32_t)u * (uint32_t)L >= nchb) v[u] = make_uint4(0, 0, 0, 0);
+                        acc_amax_nnz(amax, nnz, v[u]);
+                    }
+                }
+            };
+            if (nt) scan(std::true_type{}); else scan(std::false_type{});
         }
         amax = group_max(amax, L);                   // (shuffles: every lane of the wave takes part)
         if (bid < nb && l == 0) block_amax[bid] = amax;
