@@ -1125,9 +1125,12 @@ __global__ __launch_bounds__(WGS) void k_bs_fused(const uint4* in, uint4* out, u
 // LDS exchange between them, every wave's loads in flight while the others quantize (one workgroup per row: 58 us for
 // 16384 rows of 4096 elements from HBM, the plain quantization of the same rows 43).  Rows are dealt out to the waves in
 // turn, so that the waves that run side by side work on neighbouring rows.  Phases and npart1 as in k_bs_fused.
-template <bool E8, int NVW>
+// TILE: blocks of several rows (512 * NVW elements in rows of 8 << cpr_log, e.g. 32 x 64: the smallest block the
+// reference's own launch geometry takes, FQ:2080-2094): chunk 64 k + lane of a block lies at row (64 k + lane) >> cpr_log
+// of the block; blocks in row-major order, so the four waves of a workgroup hold four neighbours.
+template <bool E8, int NVW, bool TILE>
 __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* out, uint32_t* ws, Shape sh, int ss_mode,
-                                                      int64_t nrows, Finish fin, int phase, int npart1) {
+                                                      int64_t nrows, Finish fin, int phase, int npart1, int cpr_log) {
     __shared__ float s_f[2 * WAVES];
     __shared__ int s_i[WAVES];
     if (phase == 2 && finish_decision(fin, s_f, s_i) != 1) return;
@@ -1139,13 +1142,26 @@ __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* ou
     constexpr int ROW = 64 * NVW;                                   // chunks of a block
     float gmax = 0.0f, err = 0.0f;
     int nnz_total = 0;
+    const uint32_t row_stride = (uint32_t)(sh.cols >> 3);
+    uint32_t off[NVW];                                              // where the lane's chunks lie in a block
+#pragma unroll
+    for (int k = 0; k < NVW; ++k) {
+        const uint32_t j = (uint32_t)(64 * k + lane);
+        off[k] = TILE ? (j >> cpr_log) * row_stride + (j & ((1u << cpr_log) - 1u)) : j;
+    }
     // (Issuing a wave's next row before the arithmetic of the row it holds -- two register buffers in turn -- was measured
     // slower: 56.3 against 52.5 us for 16384 rows of 4096 elements, at 168 registers.)
     for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < nrows; row += (int64_t)gridDim.x * WAVES) {
-        const uint4* bin = in + row * ROW + lane;
-        uint4* bout = out + row * ROW + lane;
+        int64_t base = row * ROW;                                  // (one-row blocks in whole rows lie one after the other)
+        uint32_t by32 = 0, bx32 = 0;
+        if constexpr (TILE) {
+            block_of(sh, (uint32_t)row, by32, bx32);               // (fewer than 2^31 blocks)
+            base = (int64_t)by32 * sh.brows * row_stride + (((int64_t)bx32 * sh.bcols) >> 3);
+        }
+        const uint4* bin = in + base;
+        uint4* bout = out + base;
         uint4 v[NVW];
-        load16_group(v, nt_in, [&](int k) { return bin + 64 * k; });
+        load16_group(v, nt_in, [&](int k) { return bin + (TILE ? off[k] : (uint32_t)(64 * k + lane)); });
         uint32_t amax2 = 0, nnz2 = 0, negz2 = NEGZERO_INIT;
 #pragma unroll
         for (int k = 0; k < NVW; ++k) {
@@ -1182,7 +1198,7 @@ __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* ou
                     if (negz) v[k] = drop_negzero_vec(v[k]);
                     uint4 q = bs_vec_fast<E8, false, true, false>(v[k], sc, err);
                     opaque(q);
-                    store16_rt(bout + 64 * k, q, nt_out);
+                    store16_rt(bout + (TILE ? off[k] : (uint32_t)(64 * k + lane)), q, nt_out);
                 }
             } else {
 #pragma unroll
@@ -1192,17 +1208,18 @@ __global__ __launch_bounds__(WG) void k_bs_fused_wave(const uint4* in, uint4* ou
                     uint4 q = bs_vec_fast<E8, true, true, false>(v[k], sc, err);
                     opaque(q);
                     asm volatile("" : "+v"(err));
-                    store16_rt(bout + 64 * k, q, nt_out);
+                    store16_rt(bout + (TILE ? off[k] : (uint32_t)(64 * k + lane)), q, nt_out);
                 }
             }
         } else {
             // the exact arithmetic, from memory again (non-unrolled: no run-time index into the register array)
-            const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in) + row * ROW * 8;
-            uint16_t* out16 = reinterpret_cast<uint16_t*>(out) + row * ROW * 8;
+            const uint16_t* in16 = reinterpret_cast<const uint16_t*>(in) + base * 8;
+            uint16_t* out16 = reinterpret_cast<uint16_t*>(out) + base * 8;
 #pragma unroll 1
             for (int i = lane; i < ROW * 8; i += 64) {
-                const float q = bs_element<E8, false>(bf16_one(in16[i]), sc, err);
-                if (write) out16[i] = store_bf16<false>(q);
+                const int64_t e = TILE ? (int64_t)(i >> (cpr_log + 3)) * sh.cols + (i & ((8 << cpr_log) - 1)) : i;
+                const float q = bs_element<E8, false>(bf16_one(in16[e]), sc, err);
+                if (write) out16[e] = store_bf16<false>(q);
             }
         }
         }
@@ -1634,8 +1651,12 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
         k_bs_amax_flat<<<npart1, WG, 0, st>>>(static_cast<const uint4*>(input), ws, nullptr, n / 8, 1, 0);
     };
     const bool flat_ok = !emu && vec && n % 8 == 0;
-    if (flat_ok && brows == 1 && ss_mode != 4 && (blk_chunks == 128 || blk_chunks == 256 || blk_chunks == 512)) {
-        // row blocks of 1024, 2048 or 4096 elements: a wave per block
+    const bool wave_rows = brows == 1 && cols % bcols == 0;
+    // (rows of a block of at least 128 bytes: with 64-byte pieces a load instruction touches 16 rows and the kernel is no
+    // faster than the two-read path, 76 us for 32 x 32 blocks at 8192^2)
+    const bool wave_tiles = brows > 1 && rows % brows == 0 && cols % bcols == 0 && is_pow2(bcols / 8) && bcols / 8 >= 8 && bcols / 8 <= 64 && nb < ((int64_t)1 << 31);
+    if (flat_ok && (wave_rows || wave_tiles) && ss_mode != 4 && (blk_chunks == 128 || blk_chunks == 256 || blk_chunks == 512)) {
+        // row blocks of 1024, 2048 or 4096 elements, tiles of as many elements in rows of up to 512: a wave per block
         if (global) tensor_amax_pass();
         // (four workgroups per CU: 16384 rows of 4096 elements from HBM take 52.6 us with 1024 workgroups, 55.7 with 768,
         // 55.1 with 1536, 54.9 with 2048, 53.4 with 4096)
@@ -1646,7 +1667,10 @@ static int block_scaling_run(const void* input, void* output, int32_t* meta,
         uint4* o4 = static_cast<uint4*>(output);
         const int nvw = (int)(blk_chunks / 64);
         for (int phase = inplace ? 1 : 0; phase <= (inplace ? 2 : 0); ++phase) {
-#define MOR_BS_WAVE(E8, NVW) k_bs_fused_wave<E8, NVW><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, nb, fin, phase, npart1)
+        const int cpr_log = wave_tiles ? ilog2(bcols / 8) : 0;
+#define MOR_BS_WAVE(E8, NVW) do { \
+            if (wave_tiles) k_bs_fused_wave<E8, NVW, true><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, nb, fin, phase, npart1, cpr_log); \
+            else k_bs_fused_wave<E8, NVW, false><<<grid, WG, 0, st>>>(i4, o4, ws, sh, (int)ss_mode, nb, fin, phase, npart1, cpr_log); } while (0)
             if (ss_mode == 2) { if (nvw == 2) MOR_BS_WAVE(true, 2); else if (nvw == 4) MOR_BS_WAVE(true, 4); else MOR_BS_WAVE(true, 8); }
             else { if (nvw == 2) MOR_BS_WAVE(false, 2); else if (nvw == 4) MOR_BS_WAVE(false, 4); else MOR_BS_WAVE(false, 8); }
 #undef MOR_BS_WAVE

@@ -373,6 +373,29 @@ def test_scaling_tensor_scale_without_special_values(G, shape):
     assert gnnz[0] == wnnz[0] and gamax[0] == wamax[0] and np.array_equal(out, want)
 
 
+@pytest.mark.parametrize("ss", [1, 2, 3])
+@pytest.mark.parametrize("shape", [(256, 512, 32, 64, False), (128, 256, 16, 64, False), (256, 256, 64, 64, False), (128, 1024, 32, 128, False),
+                                   (64, 2048, 2, 512, False), (64, 1024, 4, 256, False), (96, 192, 32, 64, False), (2048, 1024, 32, 32, False),
+                                   (64, 8192, 1, 4096, True), (64, 6144, 1, 2048, True), (96, 3072, 1, 1024, True), (100, 4096, 1, 4096, True),
+                                   (96, 512, 32, 128, False), (160, 448, 32, 64, False)])
+def test_scaling_a_wave_per_block(G, ss, shape):
+    """Blocks of 1024, 2048 and 4096 elements, one row or several (32 x 64 is the smallest block the reference's launch
+    geometry takes): a wave holds a block (the op takes whole blocks only)."""
+    rows, cols, br, bc, channel = shape
+    a = uniform_bits(rows + cols + ss, rows, cols, -100.0, 100.0)
+    a[3, 5] = 0x8000
+    a[rows // 2, :] = 0
+    a[rows - 1, cols - 9] = 0x7F00          # a large value: its block's scale is small
+    check_scaling(G, a, br, bc, 0.045, ss, channel)
+    check_scaling(G, a, br, bc, 0.045, ss, channel, inplace=True)
+    check_scaling(G, a, br, bc, 0.0005, ss, channel)
+    a[5, 64:72] = 0x0003                    # denormals in one block
+    a[9, 9] = 0x7FC0                        # a NaN in another
+    out, meta, gamax, gnnz, gerr = G.block_scaling(a, br, bc, 0.045, ss, channel=channel)
+    want, wmeta, wamax, wnnz, werr = O.block_scaling(a, br, bc, 0.045, ss, channel=channel)
+    assert gnnz[0] == wnnz[0] and np.array_equal(out, want)
+
+
 def test_zz_no_case_was_within_the_threshold_window():
     """runs last in this file: how many of the cases above had a mean error within 1e-5 of the threshold"""
     print("scaling cases inside the 1e-5 threshold window:", len(IN_WINDOW), flush=True)
