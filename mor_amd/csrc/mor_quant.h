@@ -209,6 +209,20 @@ template <int F> __device__ __forceinline__ uint32_t fq_pair_tab(uint32_t w, flo
     const uint32_t qa = tab[codes & 0xFFu], qb = tab[(codes >> 8) & 0xFFu];
     return qa | (qb << 16) | (w & 0x80008000u);
 }
+// the same from codes the error pass left (err_pair_fast: E4M3 codes of the pair in the low half, E5M2 codes in the high half)
+template <int F> __device__ __forceinline__ uint32_t fq_pair_tab_codes(uint32_t w, uint32_t codes, const uint16_t* tab) {
+    const uint32_t c = F == FMT_E4M3 ? codes : codes >> 16;
+    const uint32_t qa = tab[c & 0xFFu], qb = tab[(c >> 8) & 0xFFu];
+    return qa | (qb << 16) | (w & 0x80008000u);
+}
+template <int F> __device__ __forceinline__ uint4 fq_vec_tab_codes(uint4 v, const uint32_t (&codes)[4], const uint16_t* tab) {
+    uint4 o;
+    o.x = fq_pair_tab_codes<F>(v.x, codes[0], tab);
+    o.y = fq_pair_tab_codes<F>(v.y, codes[1], tab);
+    o.z = fq_pair_tab_codes<F>(v.z, codes[2], tab);
+    o.w = fq_pair_tab_codes<F>(v.w, codes[3], tab);
+    return o;
+}
 template <int F> __device__ __forceinline__ uint4 fq_vec_tab(uint4 v, float s, const uint16_t* tab, uint32_t& codes) {
     uint4 o;
     o.x = fq_pair_tab<F>(v.x, s, tab, codes);

@@ -207,6 +207,12 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
     int meta_val = qa.meta_val;
     int qt_t = Q_UNKNOWN;                  // DUAL: the decision of the transposed tile where it has sums of its own
     float e4 = 0.0f, e5 = 0.0f;
+    // The error pass converts every pair to its E4M3 and its E5M2 codes; pass 3 looks the winner's codes up again instead
+    // of multiplying and converting a second time (a register per pair: whole blocks of up to 8 vectors per lane).
+    // (256 threads only: with 512 threads the 132 registers this takes leave one workgroup per CU, 128 x 256 tiles 48 -> 57 us)
+    constexpr bool KEEP = MOR && !E8 && FULL && NV <= 8 && WGS == 256 && !GATHER && !WIRE;
+    uint32_t kc[KEEP ? NV : 1][4];
+    bool have_codes = false;
     if constexpr (MOR) {
         int qt = mor_decide_range(amax, amin, qa.clamp, qa.dyn_range);
         if (qt == Q_UNKNOWN) {
@@ -215,11 +221,21 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
 #pragma unroll
             for (int k = 0; k < NV; ++k)
                 if (ok[k]) {
-                    err_pair_fast<E8>(v[k].x, s4, e4, e5, codes);
-                    err_pair_fast<E8>(v[k].y, s4, e4, e5, codes);
-                    err_pair_fast<E8>(v[k].z, s4, e4, e5, codes);
-                    err_pair_fast<E8>(v[k].w, s4, e4, e5, codes);
+                    if constexpr (KEEP) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) asm volatile("" : "=v"(kc[k][j]));          // (any register: the converts write both halves)
+                        err_pair_fast<E8>(v[k].x, s4, e4, e5, kc[k][0]);
+                        err_pair_fast<E8>(v[k].y, s4, e4, e5, kc[k][1]);
+                        err_pair_fast<E8>(v[k].z, s4, e4, e5, kc[k][2]);
+                        err_pair_fast<E8>(v[k].w, s4, e4, e5, kc[k][3]);
+                    } else {
+                        err_pair_fast<E8>(v[k].x, s4, e4, e5, codes);
+                        err_pair_fast<E8>(v[k].y, s4, e4, e5, codes);
+                        err_pair_fast<E8>(v[k].z, s4, e4, e5, codes);
+                        err_pair_fast<E8>(v[k].w, s4, e4, e5, codes);
+                    }
                 }
+            have_codes = KEEP;
 #pragma unroll
             for (int k = 0; k < NV; ++k) if (ok[k]) opaque(v[k]);
             e4 = wave_sum(e4);
@@ -322,6 +338,18 @@ __device__ __forceinline__ void wgblock_body(const uint4* in, uint4* out, int32_
             }
             __syncthreads();
             uint32_t codes = 0;                       // (the converts write half of this register: carried from word to word)
+            if constexpr (KEEP) {
+                if (have_codes) {                     // uniform over the workgroup
+                    if (fmt == FMT_E4M3) {
+#pragma unroll
+                        for (int k = 0; k < NV; ++k) put(k, fq_vec_tab_codes<FMT_E4M3>(v[k], kc[k], s_q));
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < NV; ++k) put(k, fq_vec_tab_codes<FMT_E5M2>(v[k], kc[k], s_q));
+                    }
+                    return;
+                }
+            }
             if (fmt == FMT_E4M3) {
 #pragma unroll
                 for (int k = 0; k < NV; ++k) if (ok[k]) put(k, fq_vec_tab<FMT_E4M3>(v[k], s4.s, s_q, codes));
